@@ -1,0 +1,979 @@
+/*
+ * cacti_oracle.c -- CPU restatement of the reference's LLaMA forward + backward path.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It is the checker that the
+ * HIP kernels are compared against and the "CPU port" timed as a baseline; no
+ * product path may call into it.
+ *
+ * One function per reference thunk, each output stored in the thunk's declared
+ * dtype (that is where the reference rounds), composed exactly as the reference
+ * composes them.  Citations are relative to the reference tree.
+ *
+ * Conventions
+ *   h16          IEEE binary16 held in a uint16_t.
+ *   f16 thunks   evaluate their scalar lambda in f32 and round once on store
+ *                (how Futhark's C back ends emulate f16 scalars).
+ *   reductions   accumulate in f64, then round to the thunk's dtype: the
+ *                reference's association order is internal to Futhark.
+ *
+ * PARITY UNPINNED (the reference holds no tests or golden vectors, and its
+ * arithmetic lives in an un-vendored Futhark fork + futhark_ffi):
+ *   - whether an f16 thunk rounds between the scalar ops inside one lambda
+ *     (th_silu_f16, th_logistic_f16, th_bmul_f16_tab, vjp_bmul_row);
+ *   - the summation order of cross-row reductions delivered in f16
+ *     (vjp_bmul_row = RMSNorm dw, vjp_outer_select = embedding scatter-add);
+ *   - ulp-level behaviour of exp/log/sqrt/cos/sin/pow.
+ * Everything else is pinned in tests/ by closed forms, fp64 finite differences,
+ * adjoint identities, brute force and torch.autograd on the composed model.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+typedef uint16_t h16;
+typedef int64_t i64;
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------- */
+/* binary16 <-> binary32, round to nearest even, subnormals and inf/nan kept  */
+
+static inline float h2f(h16 h)
+{
+    uint32_t s = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t e = (h >> 10) & 0x1fu;
+    uint32_t m = h & 0x3ffu;
+    uint32_t u;
+    if (e == 0) {
+        if (m == 0) {
+            u = s;
+        } else {
+            int sh = 0;
+            while (!(m & 0x400u)) { m <<= 1; sh++; }
+            m &= 0x3ffu;
+            u = s | ((uint32_t)(113 - sh) << 23) | (m << 13);
+        }
+    } else if (e == 31) {
+        u = s | 0x7f800000u | (m << 13);
+    } else {
+        u = s | ((e + 112u) << 23) | (m << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline h16 f2h(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    uint32_t s = (u >> 16) & 0x8000u;
+    uint32_t a = u & 0x7fffffffu;
+    if (a >= 0x7f800000u) {                       /* inf / nan */
+        return (h16)(s | 0x7c00u | ((a > 0x7f800000u) ? (0x200u | ((a >> 13) & 0x3ffu)) : 0));
+    }
+    if (a >= 0x477ff000u) {                       /* rounds to >= 65520 -> inf */
+        return (h16)(s | 0x7c00u);
+    }
+    if (a < 0x38800000u) {                        /* subnormal half or zero */
+        if (a < 0x33000000u) return (h16)s;       /* < 2^-25 -> 0 */
+        uint32_t e = a >> 23;
+        uint32_t m = (a & 0x7fffffu) | 0x800000u;
+        uint32_t shift = 126u - e;                /* 14 .. 24 */
+        uint32_t r = m >> shift;
+        uint32_t rem = m & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1);
+        if (rem > half || (rem == half && (r & 1u))) r++;
+        return (h16)(s | r);
+    }
+    uint32_t r = a - 0x38000000u;                 /* rebias 127 -> 15 */
+    uint32_t rem = r & 0x1fffu;
+    r >>= 13;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) r++;
+    return (h16)(s | r);
+}
+
+ORACLE_API float oracle_h2f(h16 h) { return h2f(h); }
+ORACLE_API h16 oracle_f2h(float f) { return f2h(f); }
+
+/* ------------------------------------------------------------------------- */
+/* elementwise thunks                                                         */
+
+/* CastFutThunkSpec, src/thunk/op.rs:621-663 */
+ORACLE_API void th_cast_f16_f32(i64 n, const h16 *x, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = h2f(x[i]);
+}
+ORACLE_API void th_cast_f32_f16(i64 n, const float *x, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = f2h(x[i]);
+}
+
+/* SquareFutThunkSpec, src/thunk/op.rs:2522-2565: u*u; adjoint dy*(x+x) */
+ORACLE_API void th_square_f32(i64 n, const float *x, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = x[i] * x[i];
+}
+
+/* InnerMeanFutThunkSpec, src/thunk/op.rs:3150-3254: (reduce (+) 0 t) / len */
+ORACLE_API void th_inner_mean_f32(i64 rows, i64 len, const float *x, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        double acc = 0.0;
+        for (i64 j = 0; j < len; j++) acc += (double)x[r * len + j];
+        y[r] = (float)acc / (float)len;
+    }
+}
+
+/* AddScalarFutThunkSpec, src/thunk/op.rs:1395-1434 */
+ORACLE_API void th_add_scalar_f32(i64 n, const float *x, float c, float *y)
+{
+    for (i64 i = 0; i < n; i++) y[i] = x[i] + c;
+}
+
+/* SqrtFutThunkSpec, src/thunk/op.rs:2609-2649 */
+ORACLE_API void th_sqrt_f32(i64 n, const float *x, float *y)
+{
+    for (i64 i = 0; i < n; i++) y[i] = sqrtf(x[i]);
+}
+
+/* BroadcastDivFutThunkSpec, src/thunk/op.rs:2358-2435: (f32.f16 u) / (f32.f32 v),
+ * x16 [N,D], r32 [N,1] -> f32 [N,D] */
+ORACLE_API void th_bdiv_f16_col(i64 N, i64 D, const h16 *x, const float *r, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++)
+        for (i64 d = 0; d < D; d++) y[n * D + d] = h2f(x[n * D + d]) / r[n];
+}
+
+/* BroadcastMulFutThunkSpec, src/thunk/op.rs:2058-2134: (f32.f16 u) * (f32.f32 v),
+ * w16 [1,D], t32 [N,D] -> f32 [N,D] */
+ORACLE_API void th_bmul_row_f32(i64 N, i64 D, const h16 *w, const float *t, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++)
+        for (i64 d = 0; d < D; d++) y[n * D + d] = h2f(w[d]) * t[n * D + d];
+}
+
+/* BroadcastMulFutThunkSpec on x16 [S,H,Dh] * tab16 [S,1,Dh] -> f16 (RoPE) */
+ORACLE_API void th_bmul_f16_tab(i64 S, i64 H, i64 Dh, const h16 *x, const h16 *tab, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 s = 0; s < S; s++)
+        for (i64 h = 0; h < H; h++)
+            for (i64 d = 0; d < Dh; d++) {
+                i64 i = (s * H + h) * Dh + d;
+                y[i] = f2h(h2f(x[i]) * h2f(tab[s * Dh + d]));
+            }
+}
+
+/* BroadcastMulFutThunkSpec on s32 [N,1] * z32 [N,V] -> f32 (loss-scale seed) */
+ORACLE_API void th_bmul_col_f32(i64 N, i64 V, const float *s, const float *z, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++)
+        for (i64 v = 0; v < V; v++) y[n * V + v] = s[n] * z[n * V + v];
+}
+
+/* MulFutThunkSpec, src/thunk/op.rs:2001-2055 */
+ORACLE_API void th_mul_f16(i64 n, const h16 *a, const h16 *b, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = f2h(h2f(a[i]) * h2f(b[i]));
+}
+ORACLE_API void th_mul_f32(i64 n, const float *a, const float *b, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = a[i] * b[i];
+}
+
+/* AddFutThunkSpec, src/thunk/op.rs:1480-1535; also the Accumulate epilogue
+ * `map2 (+) oy y` of src/thunk/mod.rs:1691-1733 and accumulate_1d_f16 of
+ * src/pctx/nvgpu.rs:2598-2668 (y may alias a) */
+ORACLE_API void th_add_f16(i64 n, const h16 *a, const h16 *b, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = f2h(h2f(a[i]) + h2f(b[i]));
+}
+ORACLE_API void th_add_f32(i64 n, const float *a, const float *b, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = a[i] + b[i];
+}
+
+/* SubFutThunkSpec, src/thunk/op.rs:1782-1837 */
+ORACLE_API void th_sub_f32(i64 n, const float *a, const float *b, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = a[i] - b[i];
+}
+
+/* LeftSubScalarFutThunkSpec, src/thunk/op.rs:1618-1656: c - u */
+ORACLE_API void th_lsub_scalar_f16(i64 n, float c, const h16 *x, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) y[i] = f2h(c - h2f(x[i]));
+}
+
+/* NegFutThunkSpec, src/thunk/op.rs:2438-2476 (exact: sign flip) */
+ORACLE_API void th_neg_f16(i64 n, const h16 *x, h16 *y)
+{
+    for (i64 i = 0; i < n; i++) y[i] = (h16)(x[i] ^ 0x8000u);
+}
+ORACLE_API void th_neg_f32(i64 n, const float *x, float *y)
+{
+    for (i64 i = 0; i < n; i++) y[i] = -x[i];
+}
+
+/* StandardSiluFutThunkSpec, src/thunk/op.rs:2867-2909: u / (1 + exp(-u)) */
+ORACLE_API void th_silu_f16(i64 n, const h16 *x, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) {
+        float u = h2f(x[i]);
+        y[i] = f2h(u / (1.0f + expf(-u)));
+    }
+}
+
+/* LogisticFutThunkSpec, src/thunk/op.rs:2821-2864: 1 / (1 + exp(-u)) */
+ORACLE_API void th_logistic_f16(i64 n, const h16 *x, h16 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) {
+        float u = h2f(x[i]);
+        y[i] = f2h(1.0f / (1.0f + expf(-u)));
+    }
+}
+
+/* InnerSymplecticMapFutThunkSpec, src/librarium/llama.rs:975-1049:
+ * (map neg right) ++ left over the innermost dimension (exact) */
+ORACLE_API void th_symplectic_f16(i64 rows, i64 Dh, const h16 *x, h16 *y)
+{
+    i64 hf = Dh / 2;
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        for (i64 d = 0; d < hf; d++) {
+            y[r * Dh + d] = (h16)(x[r * Dh + hf + d] ^ 0x8000u);
+            y[r * Dh + hf + d] = x[r * Dh + d];
+        }
+    }
+}
+
+/* Auto-vjp of the symplectic map (src/thunk/mod.rs:523-667): [g_r, -g_l] */
+ORACLE_API void vjp_symplectic_f16(i64 rows, i64 Dh, const h16 *g, h16 *y)
+{
+    i64 hf = Dh / 2;
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        for (i64 d = 0; d < hf; d++) {
+            y[r * Dh + d] = g[r * Dh + hf + d];
+            y[r * Dh + hf + d] = (h16)(g[r * Dh + d] ^ 0x8000u);
+        }
+    }
+}
+
+/* BlockTriElemAffineFutThunkSpec, src/thunk/op.rs:4189-4278 on [B,R,H,C]:
+ * row index = dim 1, col index = dim 3 */
+ORACLE_API void th_tri_affine_f32(i64 B, i64 R, i64 H, i64 C, const float *x, float *y,
+                                  float diag_s, float diag_b, float lo_s, float lo_b,
+                                  float up_s, float up_b)
+{
+#pragma omp parallel for schedule(static) collapse(2)
+    for (i64 b = 0; b < B; b++)
+        for (i64 i = 0; i < R; i++)
+            for (i64 h = 0; h < H; h++) {
+                i64 o = ((b * R + i) * H + h) * C;
+                for (i64 j = 0; j < C; j++) {
+                    float u = x[o + j];
+                    y[o + j] = (i < j) ? (up_s * u + up_b) : (i > j) ? (lo_s * u + lo_b)
+                                                                     : (diag_s * u + diag_b);
+                }
+            }
+}
+
+/* ------------------------------------------------------------------------- */
+/* row thunks                                                                 */
+
+/* InnerSoftmaxFutThunkSpec, src/thunk/op.rs:3257-3383:
+ * max, exp(u - max), sum, divide */
+ORACLE_API void th_softmax_f32(i64 rows, i64 len, const float *x, float *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        const float *xr = x + r * len;
+        float *yr = y + r * len;
+        float mx = -INFINITY;
+        for (i64 j = 0; j < len; j++) mx = fmaxf(mx, xr[j]);
+        double sum = 0.0;
+        for (i64 j = 0; j < len; j++) {
+            float e = expf(xr[j] - mx);
+            yr[j] = e;
+            sum += (double)e;
+        }
+        float s = (float)sum;
+        for (i64 j = 0; j < len; j++) yr[j] = yr[j] / s;
+    }
+}
+
+/* InnerSoftmaxPostAdjFutThunkSpec, src/thunk/op.rs:3386-3457:
+ * t = y*dy; s = sum t; out = t - s*y */
+ORACLE_API void th_softmax_post_adj_f32(i64 rows, i64 len, const float *y, const float *dy,
+                                        float *out)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        const float *yr = y + r * len;
+        const float *gr = dy + r * len;
+        float *o = out + r * len;
+        double sum = 0.0;
+        for (i64 j = 0; j < len; j++) {
+            float t = yr[j] * gr[j];
+            o[j] = t;
+            sum += (double)t;
+        }
+        float s = (float)sum;
+        for (i64 j = 0; j < len; j++) o[j] = o[j] - s * yr[j];
+    }
+}
+
+/* InnerSoftmaxCategoricalNLLFutThunkSpec, src/thunk/op.rs:3460-3569:
+ * softmax as above, then -(log v[k]); asserts 0 <= k < len.
+ * Returns 0, or 1 + the first offending row if a key is out of range. */
+ORACLE_API i64 th_softmax_nll_f32(i64 rows, i64 len, const float *x, const uint16_t *key,
+                                  float *out)
+{
+    for (i64 r = 0; r < rows; r++)
+        if ((i64)key[r] >= len) return r + 1;
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        const float *xr = x + r * len;
+        float mx = -INFINITY;
+        for (i64 j = 0; j < len; j++) mx = fmaxf(mx, xr[j]);
+        double sum = 0.0;
+        for (i64 j = 0; j < len; j++) sum += (double)expf(xr[j] - mx);
+        float v = expf(xr[key[r]] - mx) / (float)sum;
+        out[r] = -logf(v);
+    }
+    return 0;
+}
+
+/* InnerOneHotFutThunkSpec, src/thunk/op.rs:883-997 */
+ORACLE_API void th_one_hot_f32(i64 rows, i64 len, const uint16_t *key, float *y)
+{
+    memset(y, 0, (size_t)(rows * len) * sizeof(float));
+    for (i64 r = 0; r < rows; r++)
+        if ((i64)key[r] < len) y[r * len + key[r]] = 1.0f;
+}
+
+/* InnerArgMaxFutThunkSpec, src/thunk/op.rs:806-880: first index of the row max */
+ORACLE_API void th_arg_max_f32(i64 rows, i64 len, const float *x, i64 *y)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 r = 0; r < rows; r++) {
+        const float *xr = x + r * len;
+        i64 best = 0;
+        float mx = xr[0];
+        for (i64 j = 1; j < len; j++)
+            if (xr[j] > mx) { mx = xr[j]; best = j; }
+        y[r] = best;
+    }
+}
+
+/* OuterSelectFutThunkSpec, src/thunk/op.rs:1229-1314: map (\k -> W[k]) idx */
+ORACLE_API i64 th_outer_select_f16(i64 V, i64 D, const h16 *W, i64 S, const uint16_t *idx, h16 *y)
+{
+    for (i64 s = 0; s < S; s++)
+        if ((i64)idx[s] >= V) return s + 1;
+#pragma omp parallel for schedule(static)
+    for (i64 s = 0; s < S; s++) memcpy(y + s * D, W + (i64)idx[s] * D, (size_t)D * sizeof(h16));
+    return 0;
+}
+
+/* Auto-vjp of the gather: scatter-add of dy rows, rows with equal ids summed
+ * (f64 accumulator in position order, one rounding), rows never selected = 0 */
+ORACLE_API void vjp_outer_select_f16(i64 V, i64 D, i64 S, const uint16_t *idx, const h16 *dy,
+                                     h16 *dW)
+{
+    double *acc = (double *)calloc((size_t)(V * D), sizeof(double));
+    for (i64 s = 0; s < S; s++) {
+        double *a = acc + (i64)idx[s] * D;
+        for (i64 d = 0; d < D; d++) a[d] += (double)h2f(dy[s * D + d]);
+    }
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < V * D; i++) dW[i] = f2h((float)acc[i]);
+    free(acc);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Auto-vjp adjoints of the broadcast thunks (src/thunk/mod.rs:523-667)       */
+
+/* vjp of (f32.f16 w) * t wrt w: per element f16(dy * t), then the adjoint of
+ * `replicate` = sum over rows */
+ORACLE_API void vjp_bmul_row(i64 N, i64 D, const float *dy, const float *t, h16 *dw)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 d = 0; d < D; d++) {
+        double acc = 0.0;
+        for (i64 n = 0; n < N; n++) acc += (double)h2f(f2h(dy[n * D + d] * t[n * D + d]));
+        dw[d] = f2h((float)acc);
+    }
+}
+
+/* vjp of (f32.f16 w) * t wrt t: dy * f32(w) */
+ORACLE_API void vjp_bmul_row_t(i64 N, i64 D, const float *dy, const h16 *w, float *dt)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++)
+        for (i64 d = 0; d < D; d++) dt[n * D + d] = dy[n * D + d] * h2f(w[d]);
+}
+
+/* vjp of (f32.f16 x) / r wrt x: f16(dt / r) */
+ORACLE_API void vjp_bdiv_x(i64 N, i64 D, const float *dt, const float *r, h16 *dx)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++)
+        for (i64 d = 0; d < D; d++) dx[n * D + d] = f2h(dt[n * D + d] / r[n]);
+}
+
+/* vjp of (f32.f16 x) / r wrt r: sum_d (-dt * x / r^2) */
+ORACLE_API void vjp_bdiv_r(i64 N, i64 D, const float *dt, const h16 *x, const float *r, float *dr)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++) {
+        double acc = 0.0;
+        float rr = r[n] * r[n];
+        for (i64 d = 0; d < D; d++) acc += (double)(-(dt[n * D + d] * h2f(x[n * D + d])) / rr);
+        dr[n] = (float)acc;
+    }
+}
+
+/* vjp of inner_mean: ds / len replicated along the row */
+ORACLE_API void vjp_inner_mean(i64 N, i64 D, const float *dm, float *dsq)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 n = 0; n < N; n++) {
+        float v = dm[n] / (float)D;
+        for (i64 d = 0; d < D; d++) dsq[n * D + d] = v;
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* GEMM thunks                                                                */
+
+/* MatrixMulThunkSpec / MatrixMulF16F32GpuThunkImpl, src/thunk/op.rs:4284-4716
+ * and BlockMatrixMulThunkSpec :4719-5471: per block
+ *   C = f16( alpha * op(A) op(B) + beta * f32(C) ),  f16 in, f32 accumulate.
+ * Row-major with leading dimensions; `nblk` independent blocks spaced by the
+ * given element strides.  op(A) is M x K: stored [M,K] (ta=0) or [K,M] (ta=1);
+ * op(B) is K x N: stored [K,N] (tb=0) or [N,K] (tb=1). */
+
+typedef float v8f __attribute__((vector_size(32)));
+
+static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h16 *A, i64 lda,
+                       const h16 *B, i64 ldb, float beta, h16 *C, i64 ldc)
+{
+    /* pack op(A) as f32 [M,K] and op(B) as f32 [K,Np] with Np a multiple of 16 */
+    i64 Np = (N + 15) / 16 * 16;
+    float *a = (float *)aligned_alloc(64, (size_t)((M + 3) / 4 * 4) * (size_t)K * 4 + 64);
+    float *b = (float *)aligned_alloc(64, (size_t)K * (size_t)Np * 4 + 64);
+    i64 Mp = (M + 3) / 4 * 4;
+#pragma omp parallel for schedule(static)
+    for (i64 m = 0; m < Mp; m++)
+        for (i64 k = 0; k < K; k++)
+            a[m * K + k] = (m < M) ? h2f(ta ? A[k * lda + m] : A[m * lda + k]) : 0.0f;
+#pragma omp parallel for schedule(static)
+    for (i64 k = 0; k < K; k++)
+        for (i64 n = 0; n < Np; n++)
+            b[k * Np + n] = (n < N) ? h2f(tb ? B[n * ldb + k] : B[k * ldb + n]) : 0.0f;
+
+    const i64 KB = 256;
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+    for (i64 m0 = 0; m0 < Mp; m0 += 4)
+        for (i64 n0 = 0; n0 < Np; n0 += 16) {
+            v8f acc[4][2];
+            for (int i = 0; i < 4; i++) {
+                acc[i][0] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
+                acc[i][1] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
+            }
+            for (i64 k0 = 0; k0 < K; k0 += KB) {
+                i64 k1 = k0 + KB < K ? k0 + KB : K;
+                for (i64 k = k0; k < k1; k++) {
+                    v8f b0, b1;
+                    memcpy(&b0, b + k * Np + n0, 32);
+                    memcpy(&b1, b + k * Np + n0 + 8, 32);
+                    for (int i = 0; i < 4; i++) {
+                        float av = a[(m0 + i) * K + k];
+                        v8f avv = {av, av, av, av, av, av, av, av};
+                        acc[i][0] += avv * b0;
+                        acc[i][1] += avv * b1;
+                    }
+                }
+            }
+            for (int i = 0; i < 4; i++) {
+                i64 m = m0 + i;
+                if (m >= M) break;
+                for (int j = 0; j < 16; j++) {
+                    i64 n = n0 + j;
+                    if (n >= N) break;
+                    float v = alpha * acc[i][j >> 3][j & 7];
+                    if (beta != 0.0f) v += beta * h2f(C[m * ldc + n]);
+                    C[m * ldc + n] = f2h(v);
+                }
+            }
+        }
+    free(a);
+    free(b);
+}
+
+ORACLE_API void th_matmul_f16(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h16 *A,
+                              i64 lda, const h16 *B, i64 ldb, float beta, h16 *C, i64 ldc)
+{
+    gemm_block(ta, tb, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+}
+
+ORACLE_API void th_block_matmul_f16(int ta, int tb, i64 nblk, i64 M, i64 N, i64 K, float alpha,
+                                    const h16 *A, i64 lda, i64 sa, const h16 *B, i64 ldb, i64 sb,
+                                    float beta, h16 *C, i64 ldc, i64 sc)
+{
+    for (i64 h = 0; h < nblk; h++)
+        gemm_block(ta, tb, M, N, K, alpha, A + h * sa, lda, B + h * sb, ldb, beta, C + h * sc, ldc);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Fused units = the reference's thunk chains with its rounding schedule      */
+
+static void *xmalloc(size_t n) { return malloc(n ? n : 1); }
+
+/* RoPE tables, Llama::init_constants, src/librarium/llama.rs:389-411:
+ * inv_freq_i = 10000^(i * (-2/Dh)) (f32), freq = f32(s) * inv_freq, duplicated
+ * to width Dh, cos16/sin16 = f16(cos/sin(freq)) */
+ORACLE_API void oracle_rope_tables(i64 S, i64 Dh, h16 *cos16, h16 *sin16)
+{
+    i64 hf = Dh / 2;
+    float ex = -2.0f / (float)Dh;
+    for (i64 s = 0; s < S; s++)
+        for (i64 i = 0; i < hf; i++) {
+            float e = (float)i * ex;
+            float inv = powf(10000.0f, e);
+            float fr = (float)s * inv;
+            h16 c = f2h(cosf(fr)), sn = f2h(sinf(fr));
+            cos16[s * Dh + i] = c;
+            cos16[s * Dh + hf + i] = c;
+            sin16[s * Dh + i] = sn;
+            sin16[s * Dh + hf + i] = sn;
+        }
+}
+
+/* rms_norm closure, src/librarium/llama.rs:442-451.  Saves t (f32 [N,D]) and
+ * s = mean+eps (f32 [N]) as the reference keeps them for the backward pass. */
+ORACLE_API void oracle_rmsnorm_fwd(i64 N, i64 D, const h16 *x, const h16 *w, float eps, h16 *y,
+                                   float *t_save, float *s_save)
+{
+    size_t nd = (size_t)(N * D);
+    float *xf = xmalloc(nd * 4), *sq = xmalloc(nd * 4), *u = xmalloc(nd * 4);
+    float *m = xmalloc((size_t)N * 4), *r = xmalloc((size_t)N * 4);
+    th_cast_f16_f32(N * D, x, xf);
+    th_square_f32(N * D, xf, sq);
+    th_inner_mean_f32(N, D, sq, m);
+    th_add_scalar_f32(N, m, eps, s_save);
+    th_sqrt_f32(N, s_save, r);
+    th_bdiv_f16_col(N, D, x, r, t_save);
+    th_bmul_row_f32(N, D, w, t_save, u);
+    th_cast_f32_f16(N * D, u, y);
+    free(xf); free(sq); free(u); free(m); free(r);
+}
+
+/* Adjoint of the rms_norm chain in reverse log order (src/spine.rs:447-690):
+ * cast, broadcast_mul (vjp), broadcast_div (vjp), sqrt :2643-2648, add_scalar,
+ * inner_mean (vjp), square :2556-2564, cast :658-662.
+ * dx receives two separately rounded f16 contributions; `dx_acc`/`dw_acc` say
+ * whether dx/dw already hold a value (Accumulate) or are first written (Apply),
+ * src/op.rs:20-188. */
+ORACLE_API void oracle_rmsnorm_bwd(i64 N, i64 D, const h16 *x, const h16 *w, const float *t_save,
+                                   const float *s_save, const h16 *dy, h16 *dx, int dx_acc, h16 *dw,
+                                   int dw_acc)
+{
+    size_t nd = (size_t)(N * D);
+    float *du = xmalloc(nd * 4), *dt = xmalloc(nd * 4), *dsq = xmalloc(nd * 4);
+    float *xf = xmalloc(nd * 4), *x2 = xmalloc(nd * 4), *dxf = xmalloc(nd * 4);
+    h16 *c16 = xmalloc(nd * 2), *dw1 = xmalloc((size_t)D * 2);
+    float *dr = xmalloc((size_t)N * 4), *r = xmalloc((size_t)N * 4), *yy = xmalloc((size_t)N * 4);
+    float *ds = xmalloc((size_t)N * 4);
+
+    th_cast_f16_f32(N * D, dy, du);                 /* adjoint of lossy_cast: f32(dy) */
+    vjp_bmul_row(N, D, du, t_save, dw1);            /* dw */
+    if (dw_acc) th_add_f16(D, dw, dw1, dw); else memcpy(dw, dw1, (size_t)D * 2);
+    vjp_bmul_row_t(N, D, du, w, dt);                /* dt */
+    th_sqrt_f32(N, s_save, r);                      /* r is a saved cell in the reference */
+    vjp_bdiv_x(N, D, dt, r, c16);                   /* dx (+)= f16(dt / r) */
+    if (dx_acc) th_add_f16(N * D, dx, c16, dx); else memcpy(dx, c16, nd * 2);
+    vjp_bdiv_r(N, D, dt, x, r, dr);                 /* dr */
+    th_sqrt_f32(N, s_save, r);                      /* y = sqrt(s) recomputed by Sqrt::pop_adj */
+    th_add_f32(N, r, r, yy);
+    for (i64 n = 0; n < N; n++) ds[n] = dr[n] / yy[n];
+    /* add_scalar adjoint = memcpy(ds) */
+    vjp_inner_mean(N, D, ds, dsq);
+    th_cast_f16_f32(N * D, x, xf);
+    th_add_f32(N * D, xf, xf, x2);
+    th_mul_f32(N * D, dsq, x2, dxf);
+    th_cast_f32_f16(N * D, dxf, c16);               /* cast adjoint: lossy cast to f16 */
+    th_add_f16(N * D, dx, c16, dx);
+    free(du); free(dt); free(dsq); free(xf); free(x2); free(dxf); free(c16); free(dw1);
+    free(dr); free(r); free(yy); free(ds);
+}
+
+/* symplectic_embed, src/librarium/llama.rs:463-465: (x*cos) + (rot(x)*sin), all f16 */
+ORACLE_API void oracle_rope_fwd(i64 S, i64 H, i64 Dh, const h16 *x, const h16 *cos16,
+                                const h16 *sin16, h16 *y)
+{
+    size_t n = (size_t)(S * H * Dh);
+    h16 *a = xmalloc(n * 2), *rx = xmalloc(n * 2), *b = xmalloc(n * 2);
+    th_bmul_f16_tab(S, H, Dh, x, cos16, a);
+    th_symplectic_f16(S * H, Dh, x, rx);
+    th_bmul_f16_tab(S, H, Dh, rx, sin16, b);
+    th_add_f16(S * H * Dh, a, b, y);
+    free(a); free(rx); free(b);
+}
+
+/* Adjoint in reverse log order: Add -> (da, db) = dy; rot*sin -> drx = f16(db*sin)
+ * (sin is const_: no adjoint); rot -> dx (+)= [drx_r, -drx_l]; x*cos -> dx += f16(da*cos) */
+ORACLE_API void oracle_rope_bwd(i64 S, i64 H, i64 Dh, const h16 *dy, const h16 *cos16,
+                                const h16 *sin16, h16 *dx, int dx_acc)
+{
+    size_t n = (size_t)(S * H * Dh);
+    h16 *drx = xmalloc(n * 2), *c = xmalloc(n * 2);
+    th_bmul_f16_tab(S, H, Dh, dy, sin16, drx);
+    vjp_symplectic_f16(S * H, Dh, drx, c);
+    if (dx_acc) th_add_f16(S * H * Dh, dx, c, dx); else memcpy(dx, c, n * 2);
+    th_bmul_f16_tab(S, H, Dh, dy, cos16, c);
+    th_add_f16(S * H * Dh, dx, c, dx);
+    free(drx); free(c);
+}
+
+/* src/librarium/llama.rs:526-527: y = silu(g) (saved), h = y * u */
+ORACLE_API void oracle_silu_gate_fwd(i64 n, const h16 *g, const h16 *u, h16 *y_save, h16 *h)
+{
+    th_silu_f16(n, g, y_save);
+    th_mul_f16(n, y_save, u, h);
+}
+
+/* Mul::pop_adj src/thunk/op.rs:2050-2054 then StandardSilu::pop_adj :2901-2908 */
+ORACLE_API void oracle_silu_gate_bwd(i64 n, const h16 *g, const h16 *u, const h16 *y_save,
+                                     const h16 *dh, h16 *dg, int dg_acc, h16 *du, int du_acc)
+{
+    size_t sz = (size_t)n * 2;
+    h16 *t0 = xmalloc(sz), *dy = xmalloc(sz), *y = xmalloc(sz), *t = xmalloc(sz);
+    h16 *a = xmalloc(sz), *b = xmalloc(sz), *c = xmalloc(sz);
+    th_mul_f16(n, y_save, dh, t0);                  /* du (+)= y * dh */
+    if (du_acc) th_add_f16(n, du, t0, du); else memcpy(du, t0, sz);
+    th_mul_f16(n, dh, u, dy);                       /* dy = dh * u */
+    th_silu_f16(n, g, y);
+    th_logistic_f16(n, g, t);
+    th_lsub_scalar_f16(n, 1.0f, t, a);
+    th_mul_f16(n, y, a, b);
+    th_add_f16(n, b, t, c);
+    th_mul_f16(n, dy, c, t0);                       /* dg (+)= dy * c */
+    if (dg_acc) th_add_f16(n, dg, t0, dg); else memcpy(dg, t0, sz);
+    free(t0); free(dy); free(y); free(t); free(a); free(b); free(c);
+}
+
+/* src/librarium/llama.rs:501-505: P16 = f16(softmax(mask(f32(S16)))) on [S,H,S]
+ * (row i = dim 0, head = dim 1, col j = dim 2; batch 1) */
+ORACLE_API void oracle_causal_softmax_fwd(i64 S, i64 H, const h16 *s16, h16 *p16)
+{
+    size_t n = (size_t)(S * H * S);
+    float *s32 = xmalloc(n * 4), *m = xmalloc(n * 4);
+    th_cast_f16_f32(S * H * S, s16, s32);
+    th_tri_affine_f32(1, S, H, S, s32, m, 1.0f, 0.0f, 1.0f, 0.0f, 0.0f, -INFINITY);
+    th_softmax_f32(S * H, S, m, s32);
+    th_cast_f32_f16(S * H * S, s32, p16);
+    free(s32); free(m);
+}
+
+/* Adjoint: cast -> dP32; InnerSoftmax::pop_adj recomputes softmax(M) then post_adj;
+ * BlockTriElemAffine::pop_adj (shifts 0); cast adjoint -> f16 */
+ORACLE_API void oracle_causal_softmax_bwd(i64 S, i64 H, const h16 *s16, const h16 *dp16, h16 *ds16)
+{
+    size_t n = (size_t)(S * H * S);
+    float *s32 = xmalloc(n * 4), *m = xmalloc(n * 4), *dp = xmalloc(n * 4);
+    th_cast_f16_f32(S * H * S, s16, s32);
+    th_tri_affine_f32(1, S, H, S, s32, m, 1.0f, 0.0f, 1.0f, 0.0f, 0.0f, -INFINITY);
+    th_softmax_f32(S * H, S, m, s32);               /* P' */
+    th_cast_f16_f32(S * H * S, dp16, dp);
+    th_softmax_post_adj_f32(S * H, S, s32, dp, m);  /* dM */
+    th_tri_affine_f32(1, S, H, S, m, dp, 1.0f, 0.0f, 1.0f, 0.0f, 0.0f, 0.0f);
+    th_cast_f32_f16(S * H * S, dp, ds16);
+    free(s32); free(m); free(dp);
+}
+
+/* src/librarium/llama.rs:541-546: logit32 = f32(logit16); prob = softmax;
+ * loss = nll; tok = argmax.  Any output pointer may be NULL. */
+ORACLE_API i64 oracle_softmax_ce_fwd(i64 N, i64 V, const h16 *logit16, const uint16_t *tok,
+                                     float *prob, float *loss, uint16_t *amax)
+{
+    size_t n = (size_t)(N * V);
+    float *l32 = xmalloc(n * 4);
+    i64 rc = 0;
+    th_cast_f16_f32(N * V, logit16, l32);
+    if (prob) th_softmax_f32(N, V, l32, prob);
+    if (loss) rc = th_softmax_nll_f32(N, V, l32, tok, loss);
+    if (amax) {
+        i64 *am = xmalloc((size_t)N * 8);
+        th_arg_max_f32(N, V, l32, am);
+        for (i64 i = 0; i < N; i++) amax[i] = (uint16_t)am[i];
+        free(am);
+    }
+    free(l32);
+    return rc;
+}
+
+/* InnerSoftmaxCategoricalNLL::pop_adj src/thunk/op.rs:3555-3568 with the sink
+ * seed dloss = scale (examples/open_llama_3b_train.rs:384), then the cast adjoint */
+ORACLE_API i64 oracle_softmax_ce_bwd(i64 N, i64 V, const h16 *logit16, const uint16_t *tok,
+                                     const float *scale, h16 *dlogit16)
+{
+    size_t n = (size_t)(N * V);
+    for (i64 r = 0; r < N; r++)
+        if ((i64)tok[r] >= V) return r + 1;
+    float *l32 = xmalloc(n * 4), *p = xmalloc(n * 4), *e = xmalloc(n * 4);
+    th_cast_f16_f32(N * V, logit16, l32);
+    th_softmax_f32(N, V, l32, p);
+    th_one_hot_f32(N, V, tok, e);
+    th_sub_f32(N * V, p, e, l32);
+    th_bmul_col_f32(N, V, scale, l32, p);
+    th_cast_f32_f16(N * V, p, dlogit16);
+    free(l32); free(p); free(e);
+    return 0;
+}
+
+/* One attention block as the reference stages it, batch 1, layout [S,H,Dh]
+ * (src/librarium/llama.rs:501-507); S16 and P16 are returned for the backward. */
+ORACLE_API void oracle_attention_fwd(i64 S, i64 H, i64 Dh, float alpha, const h16 *q, const h16 *k,
+                                     const h16 *v, h16 *s16, h16 *p16, h16 *o)
+{
+    i64 ld = H * Dh, lds = H * S;
+    th_block_matmul_f16(0, 1, H, S, S, Dh, alpha, q, ld, Dh, k, ld, Dh, 0.0f, s16, lds, S);
+    oracle_causal_softmax_fwd(S, H, s16, p16);
+    th_block_matmul_f16(0, 0, H, S, Dh, S, 1.0f, p16, lds, S, v, ld, Dh, 0.0f, o, ld, Dh);
+}
+
+/* BlockMatrixMul::pop_adj src/thunk/op.rs:4882-4896 around the softmax adjoint.
+ * Order: P.V adjoint -> dV then dP; softmax chain; Q.K^T adjoint -> dK then dQ. */
+ORACLE_API void oracle_attention_bwd(i64 S, i64 H, i64 Dh, float alpha, const h16 *q, const h16 *k,
+                                     const h16 *v, const h16 *s16, const h16 *p16, const h16 *dO,
+                                     h16 *dq, h16 *dk, h16 *dv)
+{
+    i64 ld = H * Dh, lds = H * S;
+    size_t n = (size_t)(S * H * S);
+    h16 *dp16 = xmalloc(n * 2), *ds16 = xmalloc(n * 2);
+    /* (ff): arg_adj[1] += A^T x dY ; arg_adj[0] += dY x B^T */
+    th_block_matmul_f16(1, 0, H, S, Dh, S, 1.0f, p16, lds, S, dO, ld, Dh, 0.0f, dv, ld, Dh);
+    th_block_matmul_f16(0, 1, H, S, S, Dh, 1.0f, dO, ld, Dh, v, ld, Dh, 0.0f, dp16, lds, S);
+    oracle_causal_softmax_bwd(S, H, s16, dp16, ds16);
+    /* (ft): arg_adj[1] += dY^T x A ; arg_adj[0] += dY x B, both scaled by alpha */
+    th_block_matmul_f16(1, 0, H, S, Dh, S, alpha, ds16, lds, S, q, ld, Dh, 0.0f, dk, ld, Dh);
+    th_block_matmul_f16(0, 0, H, S, Dh, S, alpha, ds16, lds, S, k, ld, Dh, 0.0f, dq, ld, Dh);
+    free(dp16); free(ds16);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Whole model: Llama::apply (src/librarium/llama.rs:420-548) + the adjoint    */
+/* pass that CellMap::vadd_vjp stages (src/spine.rs:447-690), batch 1.         */
+
+typedef struct {
+    i64 S, D, H, Dh, F, V, L;
+    float eps;
+} oracle_cfg;
+
+/* Parameter / gradient block layout (element offsets into one h16 array):
+ *   embed [V,D]; per layer: pre_norm [D], q,k,v,o [D,D], post_norm [D],
+ *   gate [F,D], up [F,D], down [D,F]; head_norm [D]; lm_head [V,D]. */
+ORACLE_API i64 oracle_layer_elems(const oracle_cfg *c)
+{
+    return 2 * c->D + 4 * c->D * c->D + 3 * c->F * c->D;
+}
+ORACLE_API i64 oracle_param_elems(const oracle_cfg *c)
+{
+    return 2 * c->V * c->D + c->D + c->L * oracle_layer_elems(c);
+}
+
+typedef struct {
+    float *t1, *s1, *t2, *s2;
+    h16 *x0, *pre, *q, *k, *qr, *kr, *v, *s16, *p16, *attn, *x1, *post, *up, *gate, *y, *h;
+} layer_save;
+
+static h16 *halloc(i64 n) { return (h16 *)xmalloc((size_t)n * 2); }
+static float *falloc(i64 n) { return (float *)xmalloc((size_t)n * 4); }
+
+/* Returns 0 on success, 1+row when a token id is out of range.
+ * loss [S] f32; logit16 [S,V] (may be NULL); grad has the layout of param. */
+ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const uint16_t *tok,
+                                 const uint16_t *lm_tok, const float *loss_scale, float *loss,
+                                 h16 *logit_out, uint16_t *amax_out, h16 *grad, int n_layers_bwd)
+{
+    const i64 S = c->S, D = c->D, H = c->H, Dh = c->Dh, F = c->F, V = c->V, L = c->L;
+    const float alpha = 1.0f / sqrtf((float)Dh);
+    (void)n_layers_bwd;
+    if (H * Dh != D) return -1;
+    const h16 *embed = param;
+    const h16 *layers = param + V * D;
+    const i64 lsz = oracle_layer_elems(c);
+    const h16 *head_norm = layers + L * lsz;
+    const h16 *lm_head = head_norm + D;
+    h16 *g_embed = grad, *g_layers = grad + V * D, *g_head_norm = g_layers + L * lsz;
+    h16 *g_lm_head = g_head_norm + D;
+
+    h16 *cos16 = halloc(S * Dh), *sin16 = halloc(S * Dh);
+    oracle_rope_tables(S, Dh, cos16, sin16);
+
+    layer_save *sv = (layer_save *)calloc((size_t)L, sizeof(layer_save));
+    h16 *stream = halloc(S * D);
+    i64 rc = th_outer_select_f16(V, D, embed, S, tok, stream);
+    if (rc) return rc;
+
+    for (i64 l = 0; l < L; l++) {
+        const h16 *P = layers + l * lsz;
+        const h16 *w_pre = P, *wq = P + D, *wk = wq + D * D, *wv = wk + D * D, *wo = wv + D * D;
+        const h16 *w_post = wo + D * D, *wg = w_post + D, *wu = wg + F * D, *wd = wu + F * D;
+        layer_save *s = &sv[l];
+        s->x0 = stream;
+        s->t1 = falloc(S * D); s->s1 = falloc(S); s->t2 = falloc(S * D); s->s2 = falloc(S);
+        s->pre = halloc(S * D); s->q = halloc(S * D); s->k = halloc(S * D); s->v = halloc(S * D);
+        s->qr = halloc(S * D); s->kr = halloc(S * D);
+        s->s16 = halloc(S * H * S); s->p16 = halloc(S * H * S); s->attn = halloc(S * D);
+        s->x1 = halloc(S * D); s->post = halloc(S * D);
+        s->up = halloc(S * F); s->gate = halloc(S * F); s->y = halloc(S * F); s->h = halloc(S * F);
+        h16 *o = halloc(S * D), *down = halloc(S * D);
+
+        oracle_rmsnorm_fwd(S, D, s->x0, w_pre, c->eps, s->pre, s->t1, s->s1);
+        th_matmul_f16(0, 1, S, D, D, 1.0f, s->pre, D, wq, D, 0.0f, s->q, D);
+        oracle_rope_fwd(S, H, Dh, s->q, cos16, sin16, s->qr);
+        th_matmul_f16(0, 1, S, D, D, 1.0f, s->pre, D, wk, D, 0.0f, s->k, D);
+        oracle_rope_fwd(S, H, Dh, s->k, cos16, sin16, s->kr);
+        th_matmul_f16(0, 1, S, D, D, 1.0f, s->pre, D, wv, D, 0.0f, s->v, D);
+        oracle_attention_fwd(S, H, Dh, alpha, s->qr, s->kr, s->v, s->s16, s->p16, s->attn);
+        th_matmul_f16(0, 1, S, D, D, 1.0f, s->attn, D, wo, D, 0.0f, o, D);
+        th_add_f16(S * D, s->x0, o, s->x1);
+        oracle_rmsnorm_fwd(S, D, s->x1, w_post, c->eps, s->post, s->t2, s->s2);
+        th_matmul_f16(0, 1, S, F, D, 1.0f, s->post, D, wu, D, 0.0f, s->up, F);
+        th_matmul_f16(0, 1, S, F, D, 1.0f, s->post, D, wg, D, 0.0f, s->gate, F);
+        oracle_silu_gate_fwd(S * F, s->gate, s->up, s->y, s->h);
+        th_matmul_f16(0, 1, S, D, F, 1.0f, s->h, F, wd, F, 0.0f, down, D);
+        stream = halloc(S * D);
+        th_add_f16(S * D, s->x1, down, stream);
+        free(o); free(down);
+    }
+
+    /* head */
+    float *t3 = falloc(S * D), *s3 = falloc(S);
+    h16 *hn = halloc(S * D), *logit = halloc(S * V);
+    oracle_rmsnorm_fwd(S, D, stream, head_norm, c->eps, hn, t3, s3);
+    th_matmul_f16(0, 1, S, V, D, 1.0f, hn, D, lm_head, D, 0.0f, logit, V);
+    rc = oracle_softmax_ce_fwd(S, V, logit, lm_tok, NULL, loss, amax_out);
+    if (rc) return rc;
+    if (logit_out) memcpy(logit_out, logit, (size_t)(S * V) * 2);
+
+    if (grad) {
+        /* ---- backward, reverse log order ---- */
+        h16 *dlogit = halloc(S * V);
+        oracle_softmax_ce_bwd(S, V, logit, lm_tok, loss_scale, dlogit);
+        /* lm_head matmul (ft): dW += dY^T x A ; dA += dY x W */
+        th_matmul_f16(1, 0, V, D, S, 1.0f, dlogit, V, hn, D, 0.0f, g_lm_head, D);
+        h16 *dhn = halloc(S * D);
+        th_matmul_f16(0, 0, S, D, V, 1.0f, dlogit, V, lm_head, D, 0.0f, dhn, D);
+        h16 *dstream = halloc(S * D);
+        oracle_rmsnorm_bwd(S, D, stream, head_norm, t3, s3, dhn, dstream, 0, g_head_norm, 0);
+        free(dlogit); free(dhn);
+
+        for (i64 l = L - 1; l >= 0; l--) {
+            const h16 *P = layers + l * lsz;
+            const h16 *w_pre = P, *wq = P + D, *wk = wq + D * D, *wv = wk + D * D, *wo = wv + D * D;
+            const h16 *w_post = wo + D * D, *wg = w_post + D, *wu = wg + F * D, *wd = wu + F * D;
+            h16 *G = g_layers + l * lsz;
+            h16 *g_pre = G, *gq = G + D, *gk = gq + D * D, *gv = gk + D * D, *go = gv + D * D;
+            h16 *g_post = go + D * D, *gg = g_post + D, *gu = gg + F * D, *gd = gu + F * D;
+            layer_save *s = &sv[l];
+
+            /* x2 = x1 + down: dx1 = copy(dstream), ddown = copy(dstream) */
+            h16 *dx1 = halloc(S * D);
+            memcpy(dx1, dstream, (size_t)(S * D) * 2);
+            h16 *ddown = dstream;
+            /* down matmul */
+            th_matmul_f16(1, 0, D, F, S, 1.0f, ddown, D, s->h, F, 0.0f, gd, F);
+            h16 *dh = halloc(S * F);
+            th_matmul_f16(0, 0, S, F, D, 1.0f, ddown, D, wd, F, 0.0f, dh, F);
+            h16 *dgate = halloc(S * F), *dup = halloc(S * F);
+            oracle_silu_gate_bwd(S * F, s->gate, s->up, s->y, dh, dgate, 0, dup, 0);
+            /* gate matmul was staged after up: its adjoint comes first */
+            h16 *dpost = halloc(S * D);
+            th_matmul_f16(1, 0, F, D, S, 1.0f, dgate, F, s->post, D, 0.0f, gg, D);
+            th_matmul_f16(0, 0, S, D, F, 1.0f, dgate, F, wg, D, 0.0f, dpost, D);
+            th_matmul_f16(1, 0, F, D, S, 1.0f, dup, F, s->post, D, 0.0f, gu, D);
+            th_matmul_f16(0, 0, S, D, F, 1.0f, dup, F, wu, D, 1.0f, dpost, D);
+            oracle_rmsnorm_bwd(S, D, s->x1, w_post, s->t2, s->s2, dpost, dx1, 1, g_post, 0);
+            free(dh); free(dgate); free(dup); free(dpost); free(ddown);
+
+            /* x1 = x0 + o */
+            h16 *dx0 = halloc(S * D);
+            memcpy(dx0, dx1, (size_t)(S * D) * 2);
+            h16 *d_o = dx1;
+            th_matmul_f16(1, 0, D, D, S, 1.0f, d_o, D, s->attn, D, 0.0f, go, D);
+            h16 *dattn = halloc(S * D);
+            th_matmul_f16(0, 0, S, D, D, 1.0f, d_o, D, wo, D, 0.0f, dattn, D);
+            h16 *dqr = halloc(S * D), *dkr = halloc(S * D), *dv = halloc(S * D);
+            oracle_attention_bwd(S, H, Dh, alpha, s->qr, s->kr, s->v, s->s16, s->p16, dattn, dqr,
+                                 dkr, dv);
+            /* reverse log order of the q, k, v branches: v, k, q */
+            h16 *dpre = halloc(S * D);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, dv, D, s->pre, D, 0.0f, gv, D);
+            th_matmul_f16(0, 0, S, D, D, 1.0f, dv, D, wv, D, 0.0f, dpre, D);
+            h16 *dk = halloc(S * D), *dq = halloc(S * D);
+            oracle_rope_bwd(S, H, Dh, dkr, cos16, sin16, dk, 0);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, dk, D, s->pre, D, 0.0f, gk, D);
+            th_matmul_f16(0, 0, S, D, D, 1.0f, dk, D, wk, D, 1.0f, dpre, D);
+            oracle_rope_bwd(S, H, Dh, dqr, cos16, sin16, dq, 0);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, dq, D, s->pre, D, 0.0f, gq, D);
+            th_matmul_f16(0, 0, S, D, D, 1.0f, dq, D, wq, D, 1.0f, dpre, D);
+            oracle_rmsnorm_bwd(S, D, s->x0, w_pre, s->t1, s->s1, dpre, dx0, 1, g_pre, 0);
+            free(d_o); free(dattn); free(dqr); free(dkr); free(dv); free(dpre); free(dk); free(dq);
+            dstream = dx0;
+        }
+        vjp_outer_select_f16(V, D, S, tok, dstream, g_embed);
+        free(dstream);
+    }
+
+    for (i64 l = 0; l < L; l++) {
+        layer_save *s = &sv[l];
+        free(s->t1); free(s->s1); free(s->t2); free(s->s2); free(s->x0); free(s->pre); free(s->q);
+        free(s->k); free(s->qr); free(s->kr); free(s->v); free(s->s16); free(s->p16);
+        free(s->attn); free(s->x1); free(s->post); free(s->up); free(s->gate); free(s->y);
+        free(s->h);
+    }
+    free(sv); free(stream); free(t3); free(s3); free(hn); free(logit); free(cos16); free(sin16);
+    return 0;
+}
+
+ORACLE_API int oracle_num_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+ORACLE_API void oracle_set_num_threads(int n)
+{
+#ifdef _OPENMP
+    omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
+}

@@ -1,0 +1,282 @@
+"""ctypes binding of the CPU oracle (oracle/cacti_oracle.c).
+
+TEST INFRASTRUCTURE.  Only tests/, __graft_entry__.smoke() and the cpu_baseline
+leg of bench.py may import this module; the product never does.
+
+Arrays are numpy: f16 tensors as np.float16 (or uint16 views), indices uint16.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+i64 = C.c_int64
+f32 = C.c_float
+vp = C.c_void_p
+
+
+def build(force=False):
+    """Compile both oracle variants with gcc via the Makefile."""
+    if force:
+        subprocess.check_call(["make", "-C", _HERE, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", _HERE, "-j2"], stdout=subprocess.DEVNULL)
+
+
+def _cpu_has_avx2():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("flags"):
+                    fl = set(line.split(":", 1)[1].split())
+                    return {"avx2", "fma"} <= fl
+    except OSError:
+        pass
+    return False
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        name = "liboracle_avx2.so" if _cpu_has_avx2() else "liboracle_generic.so"
+        path = os.path.join(_HERE, name)
+        if not os.path.exists(path):
+            build()
+        _LIB = C.CDLL(path)
+        _LIB.oracle_h2f.restype = f32
+        _LIB.oracle_h2f.argtypes = [C.c_uint16]
+        _LIB.oracle_f2h.restype = C.c_uint16
+        _LIB.oracle_f2h.argtypes = [f32]
+        _LIB.oracle_llama_step.restype = i64
+        _LIB.oracle_softmax_ce_fwd.restype = i64
+        _LIB.oracle_softmax_ce_bwd.restype = i64
+        _LIB.th_softmax_nll_f32.restype = i64
+        _LIB.th_outer_select_f16.restype = i64
+        _LIB.oracle_layer_elems.restype = i64
+        _LIB.oracle_param_elems.restype = i64
+        _LIB.oracle_num_threads.restype = C.c_int
+    return _LIB
+
+
+def P(a):
+    """Pointer to a C-contiguous numpy array (or None)."""
+    if a is None:
+        return vp(0)
+    assert a.flags["C_CONTIGUOUS"], "oracle arrays must be contiguous"
+    return vp(a.ctypes.data)
+
+
+def h(a):
+    """np.float16 array from anything."""
+    return np.ascontiguousarray(np.asarray(a, dtype=np.float16))
+
+
+class Cfg(C.Structure):
+    _fields_ = [("S", i64), ("D", i64), ("H", i64), ("Dh", i64), ("F", i64), ("V", i64),
+                ("L", i64), ("eps", f32)]
+
+
+def num_threads():
+    return lib().oracle_num_threads()
+
+
+def set_num_threads(n):
+    lib().oracle_set_num_threads(C.c_int(n))
+
+
+# --------------------------------------------------------------------------
+# fused units
+
+def rope_tables(S, Dh):
+    cos = np.empty((S, Dh), np.float16)
+    sin = np.empty((S, Dh), np.float16)
+    lib().oracle_rope_tables(i64(S), i64(Dh), P(cos), P(sin))
+    return cos, sin
+
+
+def rmsnorm_fwd(x, w, eps):
+    N, D = x.shape
+    y = np.empty((N, D), np.float16)
+    t = np.empty((N, D), np.float32)
+    s = np.empty((N,), np.float32)
+    lib().oracle_rmsnorm_fwd(i64(N), i64(D), P(x), P(w), f32(eps), P(y), P(t), P(s))
+    return y, t, s
+
+
+def rmsnorm_bwd(x, w, eps, dy, dx_init=None, dw_init=None):
+    """Returns (dx, dw); *_init given => Accumulate into a copy of it."""
+    N, D = x.shape
+    _, t, s = rmsnorm_fwd(x, w, eps)
+    dx = np.empty((N, D), np.float16) if dx_init is None else dx_init.copy()
+    dw = np.empty((D,), np.float16) if dw_init is None else dw_init.copy()
+    lib().oracle_rmsnorm_bwd(i64(N), i64(D), P(x), P(w), P(t), P(s), P(dy), P(dx),
+                             C.c_int(dx_init is not None), P(dw), C.c_int(dw_init is not None))
+    return dx, dw
+
+
+def rope_fwd(x, cos, sin):
+    S, H, Dh = x.shape
+    y = np.empty_like(x)
+    lib().oracle_rope_fwd(i64(S), i64(H), i64(Dh), P(x), P(cos), P(sin), P(y))
+    return y
+
+
+def rope_bwd(dy, cos, sin, dx_init=None):
+    S, H, Dh = dy.shape
+    dx = np.empty_like(dy) if dx_init is None else dx_init.copy()
+    lib().oracle_rope_bwd(i64(S), i64(H), i64(Dh), P(dy), P(cos), P(sin), P(dx),
+                          C.c_int(dx_init is not None))
+    return dx
+
+
+def silu_gate_fwd(g, u):
+    y = np.empty_like(g)
+    hh = np.empty_like(g)
+    lib().oracle_silu_gate_fwd(i64(g.size), P(g), P(u), P(y), P(hh))
+    return y, hh
+
+
+def silu_gate_bwd(g, u, dh, dg_init=None, du_init=None):
+    y, _ = silu_gate_fwd(g, u)
+    dg = np.empty_like(g) if dg_init is None else dg_init.copy()
+    du = np.empty_like(g) if du_init is None else du_init.copy()
+    lib().oracle_silu_gate_bwd(i64(g.size), P(g), P(u), P(y), P(dh), P(dg),
+                               C.c_int(dg_init is not None), P(du), C.c_int(du_init is not None))
+    return dg, du
+
+
+def causal_softmax_fwd(s16):
+    S, H, S2 = s16.shape
+    assert S == S2
+    p = np.empty_like(s16)
+    lib().oracle_causal_softmax_fwd(i64(S), i64(H), P(s16), P(p))
+    return p
+
+
+def causal_softmax_bwd(s16, dp16):
+    S, H, _ = s16.shape
+    ds = np.empty_like(s16)
+    lib().oracle_causal_softmax_bwd(i64(S), i64(H), P(s16), P(dp16), P(ds))
+    return ds
+
+
+def softmax_ce_fwd(logit, tok, want_prob=True):
+    N, V = logit.shape
+    prob = np.empty((N, V), np.float32) if want_prob else None
+    loss = np.empty((N,), np.float32)
+    amax = np.empty((N,), np.uint16)
+    rc = lib().oracle_softmax_ce_fwd(i64(N), i64(V), P(logit), P(tok), P(prob), P(loss), P(amax))
+    if rc:
+        raise IndexError("token id out of range at row %d" % (rc - 1))
+    return prob, loss, amax
+
+
+def softmax_ce_bwd(logit, tok, scale):
+    N, V = logit.shape
+    d = np.empty((N, V), np.float16)
+    rc = lib().oracle_softmax_ce_bwd(i64(N), i64(V), P(logit), P(tok), P(scale), P(d))
+    if rc:
+        raise IndexError("token id out of range at row %d" % (rc - 1))
+    return d
+
+
+def matmul(ta, tb, A, B, alpha=1.0, beta=0.0, C_init=None):
+    """C = f16(alpha op(A) op(B) + beta C); A, B 2-d row-major."""
+    M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+    K2, N = (B.shape[1], B.shape[0]) if tb else B.shape
+    assert K == K2
+    Cm = np.zeros((M, N), np.float16) if C_init is None else C_init.copy()
+    lib().th_matmul_f16(C.c_int(ta), C.c_int(tb), i64(M), i64(N), i64(K), f32(alpha), P(A),
+                        i64(A.shape[1]), P(B), i64(B.shape[1]), f32(beta), P(Cm), i64(N))
+    return Cm
+
+
+def block_matmul(ta, tb, nblk, M, N, K, alpha, A, lda, sa, B, ldb, sb, beta, Cm, ldc, sc):
+    lib().th_block_matmul_f16(C.c_int(ta), C.c_int(tb), i64(nblk), i64(M), i64(N), i64(K),
+                              f32(alpha), P(A), i64(lda), i64(sa), P(B), i64(ldb), i64(sb),
+                              f32(beta), P(Cm), i64(ldc), i64(sc))
+    return Cm
+
+
+def attention_fwd(q, k, v, alpha):
+    S, H, Dh = q.shape
+    s16 = np.empty((S, H, S), np.float16)
+    p16 = np.empty((S, H, S), np.float16)
+    o = np.empty_like(q)
+    lib().oracle_attention_fwd(i64(S), i64(H), i64(Dh), f32(alpha), P(q), P(k), P(v), P(s16),
+                               P(p16), P(o))
+    return s16, p16, o
+
+
+def attention_bwd(q, k, v, dO, alpha):
+    S, H, Dh = q.shape
+    s16, p16, _ = attention_fwd(q, k, v, alpha)
+    dq, dk, dv = np.empty_like(q), np.empty_like(q), np.empty_like(q)
+    lib().oracle_attention_bwd(i64(S), i64(H), i64(Dh), f32(alpha), P(q), P(k), P(v), P(s16),
+                               P(p16), P(dO), P(dq), P(dk), P(dv))
+    return dq, dk, dv
+
+
+def embed_fwd(W, idx):
+    V, D = W.shape
+    y = np.empty((idx.size, D), np.float16)
+    rc = lib().th_outer_select_f16(i64(V), i64(D), P(W), i64(idx.size), P(idx), P(y))
+    if rc:
+        raise IndexError("token id out of range at position %d" % (rc - 1))
+    return y
+
+
+def embed_bwd(V, idx, dy):
+    D = dy.shape[1]
+    dW = np.empty((V, D), np.float16)
+    lib().vjp_outer_select_f16(i64(V), i64(D), i64(idx.size), P(idx), P(dy), P(dW))
+    return dW
+
+
+def accumulate_f16(a, b):
+    y = np.empty_like(a)
+    lib().th_add_f16(i64(a.size), P(a), P(b), P(y))
+    return y
+
+
+# --------------------------------------------------------------------------
+# whole model
+
+def param_layout(cfg):
+    """Ordered (name, shape) list matching the flat parameter block."""
+    D, F, V, L = cfg.D, cfg.F, cfg.V, cfg.L
+    out = [("embed", (V, D))]
+    for l in range(L):
+        out += [("l%d.pre_norm" % l, (D,)), ("l%d.q" % l, (D, D)), ("l%d.k" % l, (D, D)),
+                ("l%d.v" % l, (D, D)), ("l%d.o" % l, (D, D)), ("l%d.post_norm" % l, (D,)),
+                ("l%d.gate" % l, (F, D)), ("l%d.up" % l, (F, D)), ("l%d.down" % l, (D, F))]
+    out += [("head_norm", (D,)), ("lm_head", (V, D))]
+    return out
+
+
+def split_params(cfg, flat):
+    out, o = {}, 0
+    for name, shp in param_layout(cfg):
+        n = int(np.prod(shp))
+        out[name] = flat[o:o + n].reshape(shp)
+        o += n
+    assert o == flat.size
+    return out
+
+
+def llama_step(cfg, param, tok, lm_tok, loss_scale, want_grad=True):
+    """Returns dict(loss [S] f32, logit [S,V] f16, amax [S] u16, grad flat f16 or None)."""
+    n = lib().oracle_param_elems(C.byref(cfg))
+    assert param.size == n and param.dtype == np.float16
+    loss = np.empty((cfg.S,), np.float32)
+    logit = np.empty((cfg.S, cfg.V), np.float16)
+    amax = np.empty((cfg.S,), np.uint16)
+    grad = np.zeros((n,), np.float16) if want_grad else None
+    rc = lib().oracle_llama_step(C.byref(cfg), P(param), P(tok), P(lm_tok), P(loss_scale), P(loss),
+                                 P(logit), P(amax), P(grad), C.c_int(0))
+    if rc:
+        raise IndexError("oracle_llama_step failed rc=%d" % rc)
+    return dict(loss=loss, logit=logit, amax=amax, grad=grad)
