@@ -1,0 +1,260 @@
+// RMSNorm forward and adjoint, one 64-lane wavefront per row.
+//
+// A row (D halves) lives in registers as CH 16-byte chunks per lane, loaded once
+// from HBM; the two row reductions (sum x^2, sum dt*x) are DPP wave reductions, so
+// a row needs no barrier.  The adjoint keeps the reference's rounding schedule:
+//   du = f32(dy); t = f32(x)/r; dw += f32(f16(du t)); dt = du f32(w);
+//   c1 = f16(dt / r); dr = -sum(dt x)/r^2; ds = dr/(r+r); dsq = ds/D;
+//   c2 = f16(dsq (x+x)); dx = f16(f16(dx_old + c1) + c2)   (or f16(c1 + c2))
+// (rms_norm closure src/librarium/llama.rs:442-451 and its adjoint chain).
+#include "common.h"
+
+using namespace cacti;
+
+namespace {
+
+constexpr int kWaves = 8;                 // rows per block
+constexpr int kThreads = kWaves * 64;
+
+template <int CH>
+__global__ void __launch_bounds__(kThreads)
+rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t *__restrict__ w,
+                    float eps, half_t *__restrict__ y)
+{
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int64_t n = (int64_t)blockIdx.x * kWaves + wid;
+    if (n >= N) return;
+    const int nchunk = D / 8;
+    const half_t *xr = x + n * D;
+    h8 xv[CH];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * 64 + lane;
+        if (ch < nchunk) {
+            xv[c] = ld8(xr + ch * 8);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                float f = h2f(xv[c].v[i]);
+                ss += f * f;
+            }
+        }
+    }
+    ss = wave_sum(ss);
+    const float r = sqrtf(ss / (float)D + eps);
+    half_t *yr = y + n * D;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * 64 + lane;
+        if (ch < nchunk) {
+            h8 wv = ld8(w + ch * 8), o;
+#pragma unroll
+            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv.v[i]) * (h2f(xv[c].v[i]) / r));
+            st8(yr + ch * 8, o);
+        }
+    }
+}
+
+template <int CH>
+__global__ void __launch_bounds__(kThreads)
+rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t *__restrict__ w,
+                    float eps, const half_t *__restrict__ dy, half_t *dx, int dx_acc,
+                    float *__restrict__ dw_part)
+{
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    float *sdw = reinterpret_cast<float *>(smem_raw);     // [D]
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int64_t n = (int64_t)blockIdx.x * kWaves + wid;
+    const int nchunk = D / 8;
+    const bool live = n < N;
+
+    float dwp[CH][8];
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) dwp[c][i] = 0.f;
+
+    if (live) {
+        const half_t *xr = x + n * D, *gr = dy + n * D;
+        h8 xv[CH], gv[CH];
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            if (ch < nchunk) {
+                xv[c] = ld8(xr + ch * 8);
+                gv[c] = ld8(gr + ch * 8);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            if (ch < nchunk) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float f = h2f(xv[c].v[i]);
+                    ss += f * f;
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        const float r = sqrtf(ss / (float)D + eps);
+        float sdx = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            if (ch < nchunk) {
+                h8 wv = ld8(w + ch * 8);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float xf = h2f(xv[c].v[i]), du = h2f(gv[c].v[i]);
+                    float t = xf / r;
+                    dwp[c][i] = rnd16(du * t);
+                    float dt = du * h2f(wv.v[i]);
+                    sdx += dt * xf;
+                    gv[c].v[i] = f2h(dt / r);           // c1, kept in place of dy
+                    // dt is needed no further: c2 depends only on the row sum
+                }
+            }
+        }
+        sdx = wave_sum(sdx);
+        const float dr = -sdx / (r * r);
+        const float ds = dr / (r + r);
+        const float dsq = ds / (float)D;
+        half_t *or_ = dx + n * D;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            if (ch < nchunk) {
+                h8 o, old;
+                if (dx_acc) old = ld8(or_ + ch * 8);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    float xf = h2f(xv[c].v[i]);
+                    float c1 = h2f(gv[c].v[i]);
+                    float c2 = rnd16(dsq * (xf + xf));
+                    float base = dx_acc ? rnd16(h2f(old.v[i]) + c1) : c1;
+                    o.v[i] = f2h(base + c2);
+                }
+                st8(or_ + ch * 8, o);
+            }
+        }
+    }
+
+    // block partial of dw: waves add their rows into LDS one after another
+    for (int wv = 0; wv < kWaves; wv++) {
+        if (wid == wv) {
+#pragma unroll
+            for (int c = 0; c < CH; c++) {
+                const int ch = c * 64 + lane;
+                if (ch < nchunk) {
+#pragma unroll
+                    for (int i = 0; i < 8; i++) {
+                        if (wv == 0) sdw[ch * 8 + i] = dwp[c][i];
+                        else sdw[ch * 8 + i] += dwp[c][i];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    float *dst = dw_part + (int64_t)blockIdx.x * D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) dst[i] = sdw[i];
+}
+
+// dw[d] (+)= f16(sum over block partials); 64 columns x 16 slices per block
+__global__ void __launch_bounds__(1024)
+rms_norm_dw_finalize_kernel(int G, int D, const float *__restrict__ part, half_t *dw, int acc)
+{
+    __shared__ float red[16][64];
+    const int col = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int slice = threadIdx.x >> 6;
+    float a = 0.f;
+    if (col < D)
+        for (int g = slice; g < G; g += 16) a += part[(int64_t)g * D + col];
+    red[slice][threadIdx.x & 63] = a;
+    __syncthreads();
+    if (slice == 0 && col < D) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s += red[i][threadIdx.x];
+        dw[col] = acc ? f2h(h2f(dw[col]) + rnd16(s)) : f2h(s);
+    }
+}
+
+inline int ch_for(int64_t D) { return (int)((D / 8 + 63) / 64); }
+
+template <int CH>
+void launch_fwd(int64_t N, int D, const half_t *x, const half_t *w, float eps, half_t *y,
+                hipStream_t st)
+{
+    hipLaunchKernelGGL(rms_norm_fwd_kernel<CH>, dim3((unsigned)((N + kWaves - 1) / kWaves)),
+                       dim3(kThreads), 0, st, N, D, x, w, eps, y);
+}
+template <int CH>
+void launch_bwd(int64_t N, int D, const half_t *x, const half_t *w, float eps, const half_t *dy,
+                half_t *dx, int dx_acc, float *part, hipStream_t st)
+{
+    hipLaunchKernelGGL(rms_norm_bwd_kernel<CH>, dim3((unsigned)((N + kWaves - 1) / kWaves)),
+                       dim3(kThreads), (size_t)D * 4, st, N, D, x, w, eps, dy, dx, dx_acc, part);
+}
+
+}  // namespace
+
+#define CACTI_DISPATCH_CH(ch, CALL)                 \
+    switch (ch) {                                   \
+        case 1: { constexpr int CH = 1; CALL; } break;   \
+        case 2: { constexpr int CH = 2; CALL; } break;   \
+        case 3: case 4: { constexpr int CH = 4; CALL; } break;   \
+        case 5: case 6: case 7: { constexpr int CH = 7; CALL; } break;   \
+        case 8: { constexpr int CH = 8; CALL; } break;   \
+        case 9: case 10: case 11: case 12: { constexpr int CH = 12; CALL; } break; \
+        default: { constexpr int CH = 16; CALL; } break; \
+    }
+
+CACTI_API int cacti_hip_rms_norm_fwd(int64_t N, int64_t D, const void *x, const void *w, float eps,
+                                     void *y, void *stream)
+{
+    CACTI_REQUIRE(N > 0 && D > 0 && x && w && y, CACTI_E_INVALID,
+                  "rms_norm_fwd: null pointer or empty shape");
+    CACTI_REQUIRE(D % 8 == 0 && D <= 8192, CACTI_E_NOTIMPL,
+                  "rms_norm_fwd: need D %% 8 == 0 and D <= 8192 (D=%lld)", (long long)D);
+    CACTI_REQUIRE(aligned(x, 16) && aligned(w, 16) && aligned(y, 16), CACTI_E_INVALID,
+                  "rms_norm_fwd: tensors must be 16-byte aligned");
+    CACTI_DISPATCH_CH(ch_for(D), launch_fwd<CH>(N, (int)D, (const half_t *)x, (const half_t *)w,
+                                                eps, (half_t *)y, (hipStream_t)stream));
+    return launch_status("rms_norm_fwd");
+}
+
+CACTI_API size_t cacti_hip_rms_norm_bwd_workspace(int64_t N, int64_t D)
+{
+    if (N <= 0 || D <= 0) return 0;
+    return (size_t)((N + kWaves - 1) / kWaves) * (size_t)D * sizeof(float);
+}
+
+CACTI_API int cacti_hip_rms_norm_bwd(int64_t N, int64_t D, const void *x, const void *w, float eps,
+                                     const void *dy, void *dx, int dx_acc, void *dw, int dw_acc,
+                                     void *workspace, size_t workspace_bytes, void *stream)
+{
+    CACTI_REQUIRE(N > 0 && D > 0 && x && w && dy && dx && dw && workspace, CACTI_E_INVALID,
+                  "rms_norm_bwd: null pointer or empty shape");
+    CACTI_REQUIRE(D % 8 == 0 && D <= 8192, CACTI_E_NOTIMPL,
+                  "rms_norm_bwd: need D %% 8 == 0 and D <= 8192 (D=%lld)", (long long)D);
+    CACTI_REQUIRE(aligned(x, 16) && aligned(w, 16) && aligned(dy, 16) && aligned(dx, 16) &&
+                      aligned(workspace, 16),
+                  CACTI_E_INVALID, "rms_norm_bwd: tensors must be 16-byte aligned");
+    CACTI_REQUIRE(workspace_bytes >= cacti_hip_rms_norm_bwd_workspace(N, D), CACTI_E_INVALID,
+                  "rms_norm_bwd: workspace of %zu bytes is smaller than the %zu needed",
+                  workspace_bytes, cacti_hip_rms_norm_bwd_workspace(N, D));
+    hipStream_t st = (hipStream_t)stream;
+    CACTI_DISPATCH_CH(ch_for(D),
+                      launch_bwd<CH>(N, (int)D, (const half_t *)x, (const half_t *)w, eps,
+                                     (const half_t *)dy, (half_t *)dx, dx_acc, (float *)workspace,
+                                     st));
+    int rc = launch_status("rms_norm_bwd");
+    if (rc) return rc;
+    const int G = (int)((N + kWaves - 1) / kWaves);
+    hipLaunchKernelGGL(rms_norm_dw_finalize_kernel, dim3((unsigned)((D + 63) / 64)), dim3(1024), 0,
+                       st, G, (int)D, (const float *)workspace, (half_t *)dw, dw_acc);
+    return launch_status("rms_norm_dw_finalize");
+}

@@ -1,0 +1,382 @@
+// Row softmax kernels: causal softmax over attention scores (forward, adjoint) with one
+// wavefront per row, and the LM-head softmax / cross-entropy (forward, adjoint) with one
+// block per vocabulary row.  Rows are read from HBM once and held in registers.
+#include "common.h"
+
+using namespace cacti;
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// Causal softmax on [S,H,S]: row (i,h), columns j <= i are live, the rest are -inf.
+//   forward: P16 = f16( exp(u - max) / sum ),  u = f32(S16)
+//   adjoint: P' as above (fp32), T = P' f32(dP16), dS16 = f16( T - (sum T) P' ), 0 above
+//            the diagonal
+// (Cast, BlockTriElemAffine src/thunk/op.rs:4189-4278, InnerSoftmax :3257-3383,
+//  InnerSoftmaxPostAdj :3386-3457.)
+constexpr int kRowsPerBlock = 4;
+
+template <int CH, bool BWD>
+__global__ void __launch_bounds__(kRowsPerBlock * 64)
+causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
+                      const half_t *__restrict__ dp16, half_t *__restrict__ out)
+{
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wid;
+    if (row >= S * H) return;
+    const int i = (int)(row / H);                 // query position
+    const int nchunk = (int)(S / 8);
+    const half_t *sr = s16 + row * S;
+    float e[CH][8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * 64 + lane;
+        const int j0 = ch * 8;
+        if (ch < nchunk && j0 <= i) {
+            h8 v = ld8(sr + j0);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                e[c][k] = (j0 + k <= i) ? h2f(v.v[k]) : -INFINITY;
+                mx = fmaxf(mx, e[c][k]);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[c][k] = -INFINITY;
+        }
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            e[c][k] = expf(e[c][k] - mx);         // exp(-inf) = 0 above the diagonal
+            sum += e[c][k];
+        }
+    sum = wave_sum(sum);
+    half_t *orow = out + row * S;
+    if (!BWD) {
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            if (ch < nchunk) {
+                h8 o;
+#pragma unroll
+                for (int k = 0; k < 8; k++) o.v[k] = f2h(e[c][k] / sum);
+                st8(orow + ch * 8, o);
+            }
+        }
+    } else {
+        const half_t *gr = dp16 + row * S;
+        h8 g[CH];
+        float tsum = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            const int j0 = ch * 8;
+            const bool ld = ch < nchunk && j0 <= i;
+            if (ld) g[c] = ld8(gr + j0);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float p = e[c][k] / sum;          // 0 above the diagonal
+                e[c][k] = p;
+                if (ld && j0 + k <= i) tsum += p * h2f(g[c].v[k]);
+            }
+        }
+        tsum = wave_sum(tsum);
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            const int j0 = ch * 8;
+            if (ch < nchunk) {
+                h8 o;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const float p = e[c][k];
+                    if (j0 + k <= i) {
+                        const float t = p * h2f(g[c].v[k]);
+                        o.v[k] = f2h(t - tsum * p);
+                    } else {
+                        o.v[k] = (half_t)0.f;
+                    }
+                }
+                st8(orow + ch * 8, o);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// LM-head softmax / cross-entropy on [N,V], one block of 1024 lanes per row.
+constexpr int kCeThreads = 1024;
+
+template <int CH>
+__global__ void __launch_bounds__(kCeThreads)
+softmax_ce_fwd_kernel(int64_t N, int V, const half_t *__restrict__ logit,
+                      const uint16_t *__restrict__ tok, float *__restrict__ prob,
+                      float *__restrict__ loss, uint16_t *__restrict__ amax, int *status)
+{
+    __shared__ float red[16];
+    __shared__ float xt_s;
+    const int64_t n = blockIdx.x;
+    const int nchunk = V / 8;
+    const half_t *lr = logit + n * V;
+    const int t = tok ? (int)tok[n] : 0;
+    if (tok && t >= V) {
+        if (threadIdx.x == 0 && status) atomicMax(status, (int)n + 1);
+        return;                                    // uniform for the block
+    }
+    float e[CH][8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * kCeThreads + threadIdx.x;
+        if (ch < nchunk) {
+            h8 v = ld8(lr + ch * 8);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                e[c][k] = h2f(v.v[k]);
+                mx = fmaxf(mx, e[c][k]);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[c][k] = -INFINITY;
+        }
+    }
+    mx = block_reduce(mx, OpMax(), -INFINITY, red);
+    if (amax) {
+        // first index holding the maximum
+        float best = 3.0e38f;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * kCeThreads + threadIdx.x;
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if (e[c][k] == mx) best = fminf(best, (float)(ch * 8 + k));
+        }
+        best = -block_reduce(-best, OpMax(), -3.0e38f, red);
+        if (threadIdx.x == 0) amax[n] = (uint16_t)best;
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * kCeThreads + threadIdx.x;
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            if (loss && ch * 8 + k == t) xt_s = e[c][k];
+            e[c][k] = expf(e[c][k] - mx);
+            sum += e[c][k];
+        }
+    }
+    sum = block_reduce(sum, OpSum(), 0.f, red);     // barriers inside publish xt_s
+    if (loss && threadIdx.x == 0) loss[n] = -logf(expf(xt_s - mx) / sum);
+    if (prob) {
+        float *pr = prob + n * V;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * kCeThreads + threadIdx.x;
+            if (ch < nchunk) {
+                float4 a = make_float4(e[c][0] / sum, e[c][1] / sum, e[c][2] / sum, e[c][3] / sum);
+                float4 b = make_float4(e[c][4] / sum, e[c][5] / sum, e[c][6] / sum, e[c][7] / sum);
+                *reinterpret_cast<float4 *>(pr + ch * 8) = a;
+                *reinterpret_cast<float4 *>(pr + ch * 8 + 4) = b;
+            }
+        }
+    }
+}
+
+// dlogit16 (+)= f16( scale[n] * (softmax - one_hot(tok)) )
+template <int CH>
+__global__ void __launch_bounds__(kCeThreads)
+softmax_ce_bwd_kernel(int64_t N, int V, const half_t *__restrict__ logit,
+                      const uint16_t *__restrict__ tok, const float *__restrict__ scale,
+                      half_t *dlogit, int acc)
+{
+    __shared__ float red[16];
+    const int64_t n = blockIdx.x;
+    const int nchunk = V / 8;
+    const half_t *lr = logit + n * V;
+    const int t = (int)tok[n];
+    const float sc = scale[n];
+    float e[CH][8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * kCeThreads + threadIdx.x;
+        if (ch < nchunk) {
+            h8 v = ld8(lr + ch * 8);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                e[c][k] = h2f(v.v[k]);
+                mx = fmaxf(mx, e[c][k]);
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) e[c][k] = -INFINITY;
+        }
+    }
+    mx = block_reduce(mx, OpMax(), -INFINITY, red);
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; c++)
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            e[c][k] = expf(e[c][k] - mx);
+            sum += e[c][k];
+        }
+    sum = block_reduce(sum, OpSum(), 0.f, red);
+    half_t *dr = dlogit + n * V;
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = c * kCeThreads + threadIdx.x;
+        if (ch < nchunk) {
+            h8 o, old;
+            if (acc) old = ld8(dr + ch * 8);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                float p = e[c][k] / sum;
+                float z = p - ((ch * 8 + k == t) ? 1.0f : 0.0f);
+                float d = sc * z;
+                o.v[k] = acc ? f2h(h2f(old.v[k]) + rnd16(d)) : f2h(d);
+            }
+            st8(dr + ch * 8, o);
+        }
+    }
+}
+
+__global__ void check_tok_kernel(int64_t N, int V, const uint16_t *tok, int *status)
+{
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < N && (int)tok[i] >= V) atomicMax(status, (int)i + 1);
+}
+
+}  // namespace
+
+#define CACTI_DISPATCH_SM(ch, CALL)                                  \
+    switch (ch) {                                                    \
+        case 1: { constexpr int CH = 1; CALL; } break;               \
+        case 2: { constexpr int CH = 2; CALL; } break;               \
+        case 3: case 4: { constexpr int CH = 4; CALL; } break;       \
+        case 5: case 6: case 7: case 8: { constexpr int CH = 8; CALL; } break; \
+        default: { constexpr int CH = 16; CALL; } break;             \
+    }
+
+static int causal_check(int64_t S, int64_t H, const void *a, const void *b, const char *who)
+{
+    CACTI_REQUIRE(S > 0 && H > 0 && a && b, CACTI_E_INVALID, "%s: null pointer or empty shape", who);
+    CACTI_REQUIRE(S % 8 == 0 && S <= 8192, CACTI_E_NOTIMPL,
+                  "%s: need S %% 8 == 0 and S <= 8192 (S=%lld)", who, (long long)S);
+    CACTI_REQUIRE(aligned(a, 16) && aligned(b, 16), CACTI_E_INVALID,
+                  "%s: tensors must be 16-byte aligned", who);
+    return 0;
+}
+
+CACTI_API int cacti_hip_causal_softmax_fwd(int64_t S, int64_t H, const void *s16, void *p16,
+                                           void *stream)
+{
+    int rc = causal_check(S, H, s16, p16, "causal_softmax_fwd");
+    if (rc) return rc;
+    const unsigned grid = (unsigned)((S * H + kRowsPerBlock - 1) / kRowsPerBlock);
+    const int ch = (int)((S / 8 + 63) / 64);
+    CACTI_DISPATCH_SM(ch, hipLaunchKernelGGL((causal_softmax_kernel<CH, false>), dim3(grid),
+                                             dim3(kRowsPerBlock * 64), 0, (hipStream_t)stream, S,
+                                             (int)H, (const half_t *)s16, (const half_t *)nullptr,
+                                             (half_t *)p16));
+    return launch_status("causal_softmax_fwd");
+}
+
+CACTI_API int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const void *dp16,
+                                           void *ds16, void *stream)
+{
+    int rc = causal_check(S, H, s16, ds16, "causal_softmax_bwd");
+    if (rc) return rc;
+    CACTI_REQUIRE(dp16 && aligned(dp16, 16), CACTI_E_INVALID,
+                  "causal_softmax_bwd: dp16 null or not 16-byte aligned");
+    const unsigned grid = (unsigned)((S * H + kRowsPerBlock - 1) / kRowsPerBlock);
+    const int ch = (int)((S / 8 + 63) / 64);
+    CACTI_DISPATCH_SM(ch, hipLaunchKernelGGL((causal_softmax_kernel<CH, true>), dim3(grid),
+                                             dim3(kRowsPerBlock * 64), 0, (hipStream_t)stream, S,
+                                             (int)H, (const half_t *)s16, (const half_t *)dp16,
+                                             (half_t *)ds16));
+    return launch_status("causal_softmax_bwd");
+}
+
+static int ce_check(int64_t N, int64_t V, const void *logit, const char *who)
+{
+    CACTI_REQUIRE(N > 0 && V > 0 && logit, CACTI_E_INVALID, "%s: null pointer or empty shape", who);
+    CACTI_REQUIRE(V % 8 == 0 && V <= 65536, CACTI_E_NOTIMPL,
+                  "%s: need V %% 8 == 0 and V <= 65536 (V=%lld)", who, (long long)V);
+    CACTI_REQUIRE(aligned(logit, 16), CACTI_E_INVALID, "%s: logits must be 16-byte aligned", who);
+    return 0;
+}
+
+CACTI_API int cacti_hip_softmax_ce_fwd(int64_t N, int64_t V, const void *logit16, const void *tok,
+                                       void *prob, void *loss, void *amax, void *status,
+                                       void *stream)
+{
+    int rc = ce_check(N, V, logit16, "softmax_ce_fwd");
+    if (rc) return rc;
+    CACTI_REQUIRE(!loss || tok, CACTI_E_INVALID, "softmax_ce_fwd: loss requested without tokens");
+    CACTI_REQUIRE(!prob || aligned(prob, 16), CACTI_E_INVALID,
+                  "softmax_ce_fwd: prob must be 16-byte aligned");
+    const int ch = (int)((V / 8 + kCeThreads - 1) / kCeThreads);
+    CACTI_REQUIRE(ch <= 8, CACTI_E_NOTIMPL, "softmax_ce_fwd: V too large");
+    CACTI_DISPATCH_SM(ch, hipLaunchKernelGGL(softmax_ce_fwd_kernel<CH>, dim3((unsigned)N),
+                                             dim3(kCeThreads), 0, (hipStream_t)stream, N, (int)V,
+                                             (const half_t *)logit16, (const uint16_t *)tok,
+                                             (float *)prob, (float *)loss, (uint16_t *)amax,
+                                             (int *)status));
+    return launch_status("softmax_ce_fwd");
+}
+
+CACTI_API int cacti_hip_softmax_ce_bwd(int64_t N, int64_t V, const void *logit16, const void *tok,
+                                       const void *scale, void *dlogit16, int acc, void *stream)
+{
+    int rc = ce_check(N, V, logit16, "softmax_ce_bwd");
+    if (rc) return rc;
+    CACTI_REQUIRE(tok && scale && dlogit16 && aligned(dlogit16, 16), CACTI_E_INVALID,
+                  "softmax_ce_bwd: null pointer or misaligned output");
+    const int ch = (int)((V / 8 + kCeThreads - 1) / kCeThreads);
+    CACTI_REQUIRE(ch <= 8, CACTI_E_NOTIMPL, "softmax_ce_bwd: V too large");
+    CACTI_DISPATCH_SM(ch, hipLaunchKernelGGL(softmax_ce_bwd_kernel<CH>, dim3((unsigned)N),
+                                             dim3(kCeThreads), 0, (hipStream_t)stream, N, (int)V,
+                                             (const half_t *)logit16, (const uint16_t *)tok,
+                                             (const float *)scale, (half_t *)dlogit16, acc));
+    return launch_status("softmax_ce_bwd");
+}
+
+// Wave-reduction self-test (the DPP / swizzle path against a plain LDS loop).
+namespace {
+__global__ void selftest_wave_reduce_kernel(float *out)
+{
+    __shared__ float buf[64];
+    const int lane = threadIdx.x;
+    float v = (float)((lane * 37 + 11) % 101) - 50.0f;
+    buf[lane] = v;
+    __syncthreads();
+    float s = wave_sum(v), m = wave_max(v);
+    float rs = 0.f, rm = -INFINITY;
+    for (int i = 0; i < 64; i++) {
+        rs += buf[i];
+        rm = fmaxf(rm, buf[i]);
+    }
+    // every lane must agree with the loop; count the lanes that do
+    int ok = (s == rs) && (m == rm);
+    int cnt = __syncthreads_count(ok);
+    if (lane == 0) {
+        out[0] = s;
+        out[1] = rs;
+        out[2] = m;
+        out[3] = (float)cnt + (rm == m ? 0.f : 1000.f);
+    }
+}
+}  // namespace
+
+CACTI_API int cacti_hip_selftest_wave_reduce(void *out4, void *stream)
+{
+    CACTI_REQUIRE(out4, CACTI_E_INVALID, "selftest_wave_reduce: null pointer");
+    hipLaunchKernelGGL(selftest_wave_reduce_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream,
+                       (float *)out4);
+    return launch_status("selftest_wave_reduce");
+}

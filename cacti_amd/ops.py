@@ -1,0 +1,218 @@
+"""Operator-level Python mirror of the thunks on cacti's LLaMA backward path.
+
+Each function is one `ThunkImpl::apply` (or `accumulate` when an `*_acc` tensor is
+given) in the reference's terms (src/thunk/mod.rs:347-351), executed by the HIP kernels
+behind the C ABI.  torch is used only to own device memory and name the stream; every
+computation goes through libcacti_gpu_hip_ffi.so and fails if it is not built.
+"""
+import torch
+
+from . import ffi
+
+F16 = torch.float16
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _chk(t, dtype=F16):
+    assert t.is_cuda and t.is_contiguous() and t.dtype == dtype, (t.dtype, t.device, t.shape)
+    return t
+
+
+def selftest_wave_reduce():
+    out = torch.zeros(4, dtype=torch.float32, device="cuda")
+    ffi.call("cacti_hip_selftest_wave_reduce", out.data_ptr(), _stream())
+    return out.cpu().tolist()
+
+
+# ---------------------------------------------------------------- GEMM
+def gemm(a, b, ta=False, tb=False, alpha=1.0, beta=0.0, out=None):
+    """out = f16(alpha op(a) op(b) + beta out); a, b 2-d row-major f16 (rows may be strided)."""
+    assert a.dim() == 2 and b.dim() == 2 and a.stride(1) == 1 and b.stride(1) == 1
+    M, K = (a.shape[1], a.shape[0]) if ta else a.shape
+    K2, N = (b.shape[1], b.shape[0]) if tb else b.shape
+    assert K == K2, (a.shape, b.shape, ta, tb)
+    if out is None:
+        assert beta == 0.0
+        out = torch.empty((M, N), dtype=F16, device=a.device)
+    assert out.shape == (M, N) and out.stride(1) == 1
+    ffi.call("cacti_hip_gemm_f16", int(ta), int(tb), M, N, K, alpha, a.data_ptr(), a.stride(0),
+             b.data_ptr(), b.stride(0), beta, out.data_ptr(), out.stride(0), _stream())
+    return out
+
+
+def gemm_strided_batched(ta, tb, nblk, M, N, K, alpha, a, lda, sa, b, ldb, sb, beta, c, ldc, sc):
+    ffi.call("cacti_hip_gemm_f16_strided_batched", int(ta), int(tb), nblk, M, N, K, alpha,
+             a.data_ptr(), lda, sa, b.data_ptr(), ldb, sb, beta, c.data_ptr(), ldc, sc, _stream())
+    return c
+
+
+def block_matmul_qk(q, k, alpha):
+    """S16[i,h,j] = f16(alpha q[i,h,:] . k[j,h,:]) on [S,H,Dh] tensors (src/librarium/llama.rs:501)."""
+    S, H, Dh = q.shape
+    s16 = torch.empty((S, H, S), dtype=F16, device=q.device)
+    return gemm_strided_batched(False, True, H, S, S, Dh, alpha, q, H * Dh, Dh, k, H * Dh, Dh, 0.0,
+                                s16, H * S, S)
+
+
+def block_matmul_pv(p16, v):
+    """O[i,h,:] = f16(sum_j p16[i,h,j] v[j,h,:]) (src/librarium/llama.rs:506)."""
+    S, H, _ = p16.shape
+    Dh = v.shape[2]
+    o = torch.empty((S, H, Dh), dtype=F16, device=v.device)
+    return gemm_strided_batched(False, False, H, S, Dh, S, 1.0, p16, H * S, S, v, H * Dh, Dh, 0.0, o,
+                                H * Dh, Dh)
+
+
+# ---------------------------------------------------------------- fused thunks
+def rms_norm_fwd(x, w, eps):
+    _chk(x), _chk(w)
+    N, D = x.shape
+    y = torch.empty_like(x)
+    ffi.call("cacti_hip_rms_norm_fwd", N, D, x.data_ptr(), w.data_ptr(), eps, y.data_ptr(),
+             _stream())
+    return y
+
+
+def rms_norm_bwd(x, w, eps, dy, dx_acc=None, dw_acc=None):
+    """Returns (dx, dw).  dx_acc / dw_acc: tensors to accumulate into (updated in place)."""
+    _chk(x), _chk(w), _chk(dy)
+    N, D = x.shape
+    dx = torch.empty_like(x) if dx_acc is None else _chk(dx_acc)
+    dw = torch.empty_like(w) if dw_acc is None else _chk(dw_acc)
+    nbytes = ffi.lib().cacti_hip_rms_norm_bwd_workspace(N, D)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+    ffi.call("cacti_hip_rms_norm_bwd", N, D, x.data_ptr(), w.data_ptr(), eps, dy.data_ptr(),
+             dx.data_ptr(), int(dx_acc is not None), dw.data_ptr(), int(dw_acc is not None),
+             ws.data_ptr(), nbytes, _stream())
+    return dx, dw
+
+
+def rope_tables(S, Dh, device="cuda"):
+    cos = torch.empty((S, Dh), dtype=F16, device=device)
+    sin = torch.empty((S, Dh), dtype=F16, device=device)
+    ffi.call("cacti_hip_rope_tables", S, Dh, cos.data_ptr(), sin.data_ptr(), _stream())
+    return cos, sin
+
+
+def rope_fwd(x, cos, sin):
+    _chk(x), _chk(cos), _chk(sin)
+    S, H, Dh = x.shape
+    y = torch.empty_like(x)
+    ffi.call("cacti_hip_rope_fwd", S, H, Dh, x.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+             y.data_ptr(), _stream())
+    return y
+
+
+def rope_bwd(dy, cos, sin, dx_acc=None):
+    _chk(dy), _chk(cos), _chk(sin)
+    S, H, Dh = dy.shape
+    dx = torch.empty_like(dy) if dx_acc is None else _chk(dx_acc)
+    ffi.call("cacti_hip_rope_bwd", S, H, Dh, dy.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+             dx.data_ptr(), int(dx_acc is not None), _stream())
+    return dx
+
+
+def silu_gate_fwd(g, u):
+    _chk(g), _chk(u)
+    h = torch.empty_like(g)
+    ffi.call("cacti_hip_silu_gate_fwd", g.numel(), g.data_ptr(), u.data_ptr(), h.data_ptr(),
+             _stream())
+    return h
+
+
+def silu_gate_bwd(g, u, dh, dg_acc=None, du_acc=None):
+    _chk(g), _chk(u), _chk(dh)
+    dg = torch.empty_like(g) if dg_acc is None else _chk(dg_acc)
+    du = torch.empty_like(g) if du_acc is None else _chk(du_acc)
+    ffi.call("cacti_hip_silu_gate_bwd", g.numel(), g.data_ptr(), u.data_ptr(), dh.data_ptr(),
+             dg.data_ptr(), int(dg_acc is not None), du.data_ptr(), int(du_acc is not None),
+             _stream())
+    return dg, du
+
+
+def causal_softmax_fwd(s16):
+    _chk(s16)
+    S, H, S2 = s16.shape
+    assert S == S2
+    p = torch.empty_like(s16)
+    ffi.call("cacti_hip_causal_softmax_fwd", S, H, s16.data_ptr(), p.data_ptr(), _stream())
+    return p
+
+
+def causal_softmax_bwd(s16, dp16):
+    _chk(s16), _chk(dp16)
+    S, H, _ = s16.shape
+    ds = torch.empty_like(s16)
+    ffi.call("cacti_hip_causal_softmax_bwd", S, H, s16.data_ptr(), dp16.data_ptr(), ds.data_ptr(),
+             _stream())
+    return ds
+
+
+def _raise_index(status, what):
+    v = int(status.item())
+    if v:
+        raise IndexError("%s: id out of range at row %d" % (what, v - 1))
+
+
+def softmax_ce_fwd(logit, tok, want_prob=True):
+    """Returns (prob f32 or None, loss f32 [N], amax u16-as-int16 bits [N])."""
+    _chk(logit)
+    N, V = logit.shape
+    prob = torch.empty((N, V), dtype=torch.float32, device=logit.device) if want_prob else None
+    loss = torch.empty((N,), dtype=torch.float32, device=logit.device)
+    amax = torch.empty((N,), dtype=torch.int16, device=logit.device)
+    status = torch.zeros(1, dtype=torch.int32, device=logit.device)
+    ffi.call("cacti_hip_softmax_ce_fwd", N, V, logit.data_ptr(), tok.data_ptr(), _p(prob),
+             loss.data_ptr(), amax.data_ptr(), status.data_ptr(), _stream())
+    _raise_index(status, "softmax_ce_fwd")
+    return prob, loss, amax
+
+
+def softmax_ce_bwd(logit, tok, scale, acc=None):
+    _chk(logit), _chk(scale, torch.float32)
+    N, V = logit.shape
+    d = torch.empty_like(logit) if acc is None else _chk(acc)
+    ffi.call("cacti_hip_softmax_ce_bwd", N, V, logit.data_ptr(), tok.data_ptr(), scale.data_ptr(),
+             d.data_ptr(), int(acc is not None), _stream())
+    return d
+
+
+def embed_fwd(W, tok):
+    _chk(W)
+    V, D = W.shape
+    S = tok.numel()
+    y = torch.empty((S, D), dtype=F16, device=W.device)
+    status = torch.zeros(1, dtype=torch.int32, device=W.device)
+    ffi.call("cacti_hip_embed_fwd", V, D, W.data_ptr(), S, tok.data_ptr(), y.data_ptr(),
+             status.data_ptr(), _stream())
+    _raise_index(status, "embed_fwd")
+    return y
+
+
+def embed_bwd(V, tok, dy, acc=None):
+    _chk(dy)
+    S, D = dy.shape
+    dW = torch.empty((V, D), dtype=F16, device=dy.device) if acc is None else _chk(acc)
+    ffi.call("cacti_hip_embed_bwd", V, D, S, tok.data_ptr(), dy.data_ptr(), dW.data_ptr(),
+             int(acc is not None), _stream())
+    return dW
+
+
+def add_f16(a, b, out=None):
+    out = torch.empty_like(a) if out is None else out
+    ffi.call("cacti_hip_add_f16", a.numel(), a.data_ptr(), b.data_ptr(), out.data_ptr(), _stream())
+    return out
+
+
+def accumulate_1d(dst, src):
+    name = {torch.float32: "f32", torch.float16: "f16", torch.int16: "u16"}[dst.dtype]
+    ffi.call("cacti_hip_accumulate_1d_" + name, dst.data_ptr(), src.data_ptr(), dst.numel(),
+             _stream())
+    return dst

@@ -1,0 +1,209 @@
+/*
+ * cacti_gpu_hip_ffi.h -- C ABI of libcacti_gpu_hip_ffi.so
+ *
+ * The MI355X (gfx950) counterpart of cacti's `cacti_gpu_cu_ffi` crate plus the
+ * kernels its thunks dispatch to.  Every entry point is plain C: raw device
+ * pointers, integer sizes, a stream handle passed as `void*` (a hipStream_t;
+ * NULL = the null stream, which is the stream the reference computes on,
+ * src/pctx/nvgpu.rs:263).  No C++ or torch types cross this boundary.
+ *
+ * Conventions
+ *   - every function returns an int status: 0 = success, a positive value = the
+ *     hipError_t of the failing runtime call, a negative value = CACTI_E_*.
+ *     (reference: C level integer status, 0 = ok; Rust wrappers map it to
+ *     Result<_, code>, cacti_gpu_cu_ffi/src/lib.rs:98-885.)
+ *   - kernels are asynchronous on `stream`; results are complete at stream sync
+ *     (the reference syncs the stream around every thunk, src/thunk/mod.rs:3480,3536).
+ *   - pointers are borrowed for the duration of the call; nothing is freed or
+ *     retained by the library (src/thunk/op.rs:4574-4578 convention: the caller
+ *     owns and pre-allocates outputs).
+ *   - f16 tensors are IEEE binary16, row-major, contiguous unless a leading
+ *     dimension is given.  `acc` arguments: 0 = Apply (output is first written),
+ *     1 = Accumulate (output += result, added in the output dtype; for GEMMs
+ *     beta = 1 is added in fp32 before the single output rounding), mirroring
+ *     ThunkImpl::{apply,accumulate}, src/thunk/mod.rs:347-351.
+ *   - calls on one device context are not re-entrant (one thread per context,
+ *     as in the reference, src/ctx.rs:21-29).
+ */
+#ifndef CACTI_GPU_HIP_FFI_H
+#define CACTI_GPU_HIP_FFI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CACTI_OK 0
+#define CACTI_E_INVALID (-1)   /* bad shape / null pointer / misaligned operand      */
+#define CACTI_E_NOTIMPL (-2)   /* shape outside what the kernel supports             */
+#define CACTI_E_INDEX (-3)     /* token / key id out of range (reference: assert)     */
+#define CACTI_E_OOM (-4)       /* pool exhausted even after eviction                  */
+#define CACTI_E_STATE (-5)     /* call not valid in the current state                 */
+
+/* Human-readable text for the last non-zero status returned on this thread. */
+const char *cacti_hip_last_error(void);
+
+/* ------------------------------------------------------------------------- */
+/* Device, memory, streams, events.                                           */
+/* Replaces cacti_gpu_cu_ffi/src/lib.rs:98-131 (device), :204-268 (memory),   */
+/* :332-399 (runtime), :401-565 (events, streams).                            */
+
+int cacti_hip_device_count(int *count);                         /* lib.rs:98, :332  */
+int cacti_hip_device_get(int *dev);                             /* lib.rs:341       */
+int cacti_hip_device_set(int dev);                              /* lib.rs:350       */
+int cacti_hip_device_attribute(int dev, int attr, int *value);  /* lib.rs:116       */
+int cacti_hip_device_sync(void);                                /* lib.rs:368       */
+int cacti_hip_mem_get_info(size_t *free_bytes, size_t *total_bytes); /* lib.rs:358  */
+int cacti_hip_mem_alloc(void **dptr, size_t bytes);             /* lib.rs:204       */
+int cacti_hip_mem_free(void *dptr);                             /* lib.rs:222       */
+int cacti_hip_mem_alloc_host(void **ptr, size_t bytes);         /* lib.rs:213 (hipHostMalloc) */
+int cacti_hip_mem_free_host(void *ptr);                         /* lib.rs:230       */
+int cacti_hip_memcpy_d2h(void *dst, const void *src, size_t bytes);                 /* lib.rs:238 */
+int cacti_hip_memcpy_async(void *dst, const void *src, size_t bytes, void *stream); /* lib.rs:246 */
+int cacti_hip_memcpy_h2d_async(void *dst, const void *src, size_t bytes, void *stream); /* :254 */
+int cacti_hip_memcpy_d2h_async(void *dst, const void *src, size_t bytes, void *stream); /* :262 */
+int cacti_hip_memset_async(void *dst, int byte, size_t bytes, void *stream);
+int cacti_hip_stream_create(void **stream);                     /* lib.rs:518       */
+int cacti_hip_stream_create_nonblocking(void **stream);         /* lib.rs:529       */
+int cacti_hip_stream_destroy(void *stream);                     /* lib.rs:493       */
+int cacti_hip_stream_sync(void *stream);                        /* lib.rs:540       */
+int cacti_hip_stream_wait_event(void *stream, void *event);     /* lib.rs:548       */
+int cacti_hip_event_create(void **event, int enable_timing);    /* lib.rs:431       */
+int cacti_hip_event_destroy(void *event);                       /* lib.rs:415       */
+int cacti_hip_event_record(void *event, void *stream);          /* lib.rs:442       */
+int cacti_hip_event_query(void *event);                         /* lib.rs:453       */
+int cacti_hip_event_sync(void *event);                          /* lib.rs:461       */
+int cacti_hip_event_elapsed_ms(void *start, void *stop, float *ms);
+
+/* ------------------------------------------------------------------------- */
+/* GEMM: C = alpha * op(A) op(B) + beta * C, f16 x f16 -> fp32 accumulate ->   */
+/* f16 out, hand-written MFMA kernels.                                         */
+
+/* Row-major form.  op(A) is M x K: stored [M,K] (ta = 0) or [K,M] (ta = 1);
+ * op(B) is K x N: stored [K,N] (tb = 0) or [N,K] (tb = 1); C is [M,N].
+ * Leading dimensions in elements.  beta must be 0 or 1.
+ * Replaces MatrixMulF16F32GpuThunkImpl::_enter, src/thunk/op.rs:4423-4700. */
+int cacti_hip_gemm_f16(int ta, int tb, int64_t M, int64_t N, int64_t K, float alpha,
+                       const void *A, int64_t lda, const void *B, int64_t ldb, float beta,
+                       void *C, int64_t ldc, void *stream);
+
+/* `nblk` independent blocks, block h at A + h*stride_a etc. (strides in
+ * elements).  This is how the per-head blocks of [B,S,H,Dh] / [B,S,H,S]
+ * tensors are addressed; it replaces the pointer-array staging of
+ * BlockMatrixMulF16F32GpuThunkImpl::_enter, src/thunk/op.rs:5027-5471
+ * (cublasGemmBatchedEx, cacti_gpu_cu_ffi/src/lib.rs:793-885).  No padding of
+ * the inner dimension is needed (the reference pads Dh 100 -> 104,
+ * src/op.rs:1454-1482). */
+int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N,
+                                       int64_t K, float alpha, const void *A, int64_t lda,
+                                       int64_t stride_a, const void *B, int64_t ldb,
+                                       int64_t stride_b, float beta, void *C, int64_t ldc,
+                                       int64_t stride_c, void *stream);
+
+/* Column-major, cuBLAS-shaped form with host alpha/beta pointers, the call the
+ * reference makes (cublas_gemm, cacti_gpu_cu_ffi/src/lib.rs:727-791; row-major
+ * callers pass the operands swapped, src/thunk/op.rs:4469-4491).  tr_* = 0 (N)
+ * or 1 (T).  Only f16 in / f16 out / fp32 compute is provided. */
+int cacti_hip_gemm_colmajor_f16(int tr_a, int tr_b, int m, int n, int k, const float *alpha,
+                                const void *a, int lda, const void *b, int ldb,
+                                const float *beta, void *c, int ldc, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* accumulate_1d_{f32,f16,u16}: dst[i] += src[i]                               */
+/* Replaces the NVRTC kernels of src/pctx/nvgpu.rs:2598-2668 (n <= INT32_MAX). */
+
+int cacti_hip_accumulate_1d_f32(void *dst, const void *src, int64_t n, void *stream);
+int cacti_hip_accumulate_1d_f16(void *dst, const void *src, int64_t n, void *stream);
+int cacti_hip_accumulate_1d_u16(void *dst, const void *src, int64_t n, void *stream);
+
+/* ------------------------------------------------------------------------- */
+/* Fused thunks.  Each stands for a chain of reference thunks and reproduces   */
+/* that chain's rounding points in registers.                                  */
+
+/* RMSNorm, rms_norm closure src/librarium/llama.rs:442-451
+ * (Cast op.rs:621, Square :2522, InnerMean :3150, AddScalar :1395, Sqrt :2609,
+ *  BroadcastDiv :2358, BroadcastMul :2058, Cast).
+ * x, y: [N,D] f16; w: [D] f16.  D % 8 == 0, D <= 16384. */
+int cacti_hip_rms_norm_fwd(int64_t N, int64_t D, const void *x, const void *w, float eps,
+                           void *y, void *stream);
+
+/* Adjoint of the chain above (src/spine.rs:447-690 over the same thunks).
+ * dx [N,D] f16 receives the two f16 contributions of the reference in order
+ * (dx_acc: 0 first write, 1 dx already holds the residual gradient).
+ * dw [D] f16 (dw_acc likewise).  workspace: device scratch of at least
+ * cacti_hip_rms_norm_bwd_workspace(N, D) bytes, contents undefined on return. */
+size_t cacti_hip_rms_norm_bwd_workspace(int64_t N, int64_t D);
+int cacti_hip_rms_norm_bwd(int64_t N, int64_t D, const void *x, const void *w, float eps,
+                           const void *dy, void *dx, int dx_acc, void *dw, int dw_acc,
+                           void *workspace, size_t workspace_bytes, void *stream);
+
+/* RoPE tables, Llama::init_constants src/librarium/llama.rs:389-411.
+ * cos16, sin16: [S,Dh] f16 (two identical halves of width Dh/2). */
+int cacti_hip_rope_tables(int64_t S, int64_t Dh, void *cos16, void *sin16, void *stream);
+
+/* symplectic_embed src/librarium/llama.rs:463-465 and its adjoint
+ * (InnerSymplecticMapFutThunkSpec :975-1049, BroadcastMul, Add).
+ * x, y, dy, dx: [S,H,Dh] f16 (heads are the middle dimension); Dh even, H*Dh % 8 == 0. */
+int cacti_hip_rope_fwd(int64_t S, int64_t H, int64_t Dh, const void *x, const void *cos16,
+                       const void *sin16, void *y, void *stream);
+int cacti_hip_rope_bwd(int64_t S, int64_t H, int64_t Dh, const void *dy, const void *cos16,
+                       const void *sin16, void *dx, int dx_acc, void *stream);
+
+/* SiLU gate, src/librarium/llama.rs:526-527: h = f16(f16(silu(g)) * u)
+ * (StandardSiluFutThunkSpec op.rs:2867-2909, MulFutThunkSpec :2001-2055), and
+ * the adjoint: du (+)= f16(y*dh); dg (+)= f16(f16(dh*u) * c), c per :2901-2908.
+ * All [n] f16, n % 8 == 0. */
+int cacti_hip_silu_gate_fwd(int64_t n, const void *g, const void *u, void *h, void *stream);
+int cacti_hip_silu_gate_bwd(int64_t n, const void *g, const void *u, const void *dh, void *dg,
+                            int dg_acc, void *du, int du_acc, void *stream);
+
+/* Causal softmax over attention scores, src/librarium/llama.rs:501-505:
+ * P16 = f16(softmax_j(mask(f32(S16)))) with mask j > i -> -inf
+ * (Cast, BlockTriElemAffineFutThunkSpec op.rs:4189-4278, InnerSoftmaxFutThunkSpec
+ * :3257-3383), and its adjoint dS16 = f16(tril(T - (sum_j T) P')), T = P' * f32(dP16),
+ * P' recomputed in fp32 (InnerSoftmaxPostAdjFutThunkSpec :3386-3457).
+ * s16, p16, dp16, ds16: [S,H,S] f16 (row i, head, column j).  S % 8 == 0, S <= 16384. */
+int cacti_hip_causal_softmax_fwd(int64_t S, int64_t H, const void *s16, void *p16, void *stream);
+int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const void *dp16,
+                                 void *ds16, void *stream);
+
+/* LM loss, src/librarium/llama.rs:541-546 on logit16 [N,V] f16, tok [N] u16:
+ * prob [N,V] f32 = softmax(f32(logit)) (InnerSoftmax), loss [N] f32
+ * (InnerSoftmaxCategoricalNLLFutThunkSpec op.rs:3460-3569), amax [N] u16
+ * (InnerArgMaxFutThunkSpec :806-880, first index of the maximum).
+ * prob / loss / amax may each be NULL.  status [1] i32 on the device is set to
+ * 1 + row if a token id is >= V (the reference asserts, op.rs:3538); it must be
+ * zero-initialised by the caller, or NULL to skip the check. */
+int cacti_hip_softmax_ce_fwd(int64_t N, int64_t V, const void *logit16, const void *tok,
+                             void *prob, void *loss, void *amax, void *status, void *stream);
+
+/* Adjoint: dlogit16 (+)= f16(scale[n] * (softmax(f32(logit)) - one_hot(tok)))
+ * (pop_adj op.rs:3555-3568 with InnerOneHot :883-997, Sub :1782, BroadcastMul, Cast).
+ * scale [N] f32 is the sink seed (examples/open_llama_3b_train.rs:384). */
+int cacti_hip_softmax_ce_bwd(int64_t N, int64_t V, const void *logit16, const void *tok,
+                             const void *scale, void *dlogit16, int acc, void *stream);
+
+/* Embedding, OuterSelectFutThunkSpec src/thunk/op.rs:1229-1314: y[s] = W[tok[s]]
+ * (bit-exact gather) and its adjoint: dW[v] (+)= sum of dy rows with tok[s] == v,
+ * summed in position order with one rounding.  W, dW: [V,D] f16; tok: [S] u16;
+ * y, dy: [S,D] f16.  D % 8 == 0.  With acc = 0 rows never selected are zeroed.
+ * status as in cacti_hip_softmax_ce_fwd. */
+int cacti_hip_embed_fwd(int64_t V, int64_t D, const void *W, int64_t S, const void *tok,
+                        void *y, void *status, void *stream);
+int cacti_hip_embed_bwd(int64_t V, int64_t D, int64_t S, const void *tok, const void *dy,
+                        void *dW, int acc, void *stream);
+
+/* f16 residual add y = a + b (AddFutThunkSpec src/thunk/op.rs:1480-1535); y may alias a or b. */
+int cacti_hip_add_f16(int64_t n, const void *a, const void *b, void *y, void *stream);
+
+/* Wave-level reduction self-test: fills out[0..3] (f32, device) with the 64-lane
+ * sum and max of lane-dependent values computed two ways (cross-lane DPP path and
+ * LDS path).  Returns the kernel launch status only; the caller compares. */
+int cacti_hip_selftest_wave_reduce(void *out4, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CACTI_GPU_HIP_FFI_H */

@@ -1,0 +1,329 @@
+"""Parity of every HIP kernel against the CPU oracle on the same seeded inputs (MI355X).
+
+All calls go through the C ABI (cacti_amd.ops is a thin ctypes layer).  Tolerances:
+tests/util.py (rel-L2 <= 1e-3, max element relative error <= 2e-2); gather / argmax /
+index results bit-exact.  Elementwise kernels reproduce the oracle's rounding points, so
+most of them are in fact compared bit for bit (`exact_frac`).
+"""
+import numpy as np
+import pytest
+import torch
+
+from tests.util import assert_parity, rng, randn16
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    from cacti_amd import ops as o
+    return o
+
+
+def dev(a):
+    if a.dtype == np.uint16:
+        a = a.view(np.int16)
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    a = t.detach().cpu().numpy()
+    return a
+
+
+def exact_frac(a, b):
+    return float(np.mean(a.view(np.uint16) == b.view(np.uint16)))
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ---------------------------------------------------------------- wave reduce
+def test_wave_reduce_selftest(ops):
+    s, rs, m, cnt = ops.selftest_wave_reduce()
+    assert s == rs and cnt == 64.0, (s, rs, m, cnt)
+
+
+# ---------------------------------------------------------------- RMSNorm
+@pytest.mark.parametrize("N,D", [(2048, 3200), (128, 256), (37, 4096), (5, 8), (16, 8192)])
+def test_rms_norm_fwd(ops, oracle, N, D):
+    say("rms_norm_fwd", N, D)
+    r = rng(100 + D)
+    x, w = randn16(r, (N, D)), randn16(r, (D,))
+    want, _, _ = oracle.rmsnorm_fwd(x, w, 1e-6)
+    got = host(ops.rms_norm_fwd(dev(x), dev(w), 1e-6))
+    assert_parity(got, want, "rms_norm_fwd")
+    assert exact_frac(got, want) > 0.999
+
+
+@pytest.mark.parametrize("N,D", [(2048, 3200), (128, 256), (37, 4096), (5, 8), (16, 8192)])
+@pytest.mark.parametrize("acc", [False, True])
+def test_rms_norm_bwd(ops, oracle, N, D, acc):
+    say("rms_norm_bwd", N, D, acc)
+    r = rng(200 + D + acc)
+    x, w, dy = randn16(r, (N, D)), randn16(r, (D,)), randn16(r, (N, D))
+    dx0 = randn16(r, (N, D)) if acc else None
+    dw0 = randn16(r, (D,)) if acc else None
+    wdx, wdw = oracle.rmsnorm_bwd(x, w, 1e-6, dy, dx0, dw0)
+    gdx, gdw = ops.rms_norm_bwd(dev(x), dev(w), 1e-6, dev(dy), dev(dx0) if acc else None,
+                                dev(dw0) if acc else None)
+    assert_parity(host(gdx), wdx, "dx")
+    assert_parity(host(gdw), wdw, "dw")
+    assert exact_frac(host(gdx), wdx) > 0.99
+
+
+# ---------------------------------------------------------------- RoPE
+def test_rope_tables(ops, oracle):
+    for S, Dh in [(2048, 100), (128, 64)]:
+        c, s = ops.rope_tables(S, Dh)
+        wc, ws = oracle.rope_tables(S, Dh)
+        # device cos/sin/pow differ from libm in the last ulp of f32: allow one f16 ulp
+        assert np.max(np.abs(host(c).astype(np.float32) - wc.astype(np.float32))) <= 2 ** -10
+        assert np.max(np.abs(host(s).astype(np.float32) - ws.astype(np.float32))) <= 2 ** -10
+        assert exact_frac(host(c), wc) > 0.99 and exact_frac(host(s), ws) > 0.99
+
+
+@pytest.mark.parametrize("S,H,Dh", [(2048, 32, 100), (128, 4, 64), (7, 2, 12), (33, 32, 100)])
+def test_rope_fwd_bwd(ops, oracle, S, H, Dh):
+    say("rope", S, H, Dh)
+    r = rng(300 + S)
+    x, dy, dx0 = randn16(r, (S, H, Dh)), randn16(r, (S, H, Dh)), randn16(r, (S, H, Dh))
+    cos, sin = oracle.rope_tables(S, Dh)
+    dc, ds = dev(cos), dev(sin)
+    got = host(ops.rope_fwd(dev(x), dc, ds))
+    assert np.array_equal(got.view(np.uint16), oracle.rope_fwd(x, cos, sin).view(np.uint16))
+    got = host(ops.rope_bwd(dev(dy), dc, ds))
+    assert np.array_equal(got.view(np.uint16), oracle.rope_bwd(dy, cos, sin).view(np.uint16))
+    got = host(ops.rope_bwd(dev(dy), dc, ds, dev(dx0)))
+    assert np.array_equal(got.view(np.uint16), oracle.rope_bwd(dy, cos, sin, dx0).view(np.uint16))
+
+
+def test_rope_bwd_in_place(ops, oracle):
+    r = rng(310)
+    S, H, Dh = 64, 32, 100
+    dy = randn16(r, (S, H, Dh))
+    cos, sin = oracle.rope_tables(S, Dh)
+    t = dev(dy)
+    from cacti_amd import ffi
+    ffi.call("cacti_hip_rope_bwd", S, H, Dh, t.data_ptr(), dev(cos).data_ptr(),
+             dev(sin).data_ptr(), t.data_ptr(), 0, torch.cuda.current_stream().cuda_stream)
+    assert np.array_equal(host(t).view(np.uint16), oracle.rope_bwd(dy, cos, sin).view(np.uint16))
+
+
+# ---------------------------------------------------------------- SiLU gate
+@pytest.mark.parametrize("shape", [(2048, 8640), (128, 688), (1, 8)])
+def test_silu_gate(ops, oracle, shape):
+    say("silu_gate", shape)
+    r = rng(400 + shape[1])
+    g, u, dh = randn16(r, shape, 2.0), randn16(r, shape), randn16(r, shape)
+    _, wh = oracle.silu_gate_fwd(g, u)
+    gh = host(ops.silu_gate_fwd(dev(g), dev(u)))
+    assert_parity(gh, wh, "h")
+    assert exact_frac(gh, wh) > 0.999
+    wdg, wdu = oracle.silu_gate_bwd(g, u, dh)
+    gdg, gdu = ops.silu_gate_bwd(dev(g), dev(u), dev(dh))
+    assert_parity(host(gdg), wdg, "dg"), assert_parity(host(gdu), wdu, "du")
+    assert exact_frac(host(gdg), wdg) > 0.999 and exact_frac(host(gdu), wdu) > 0.999
+    dg0, du0 = randn16(r, shape), randn16(r, shape)
+    wdg, wdu = oracle.silu_gate_bwd(g, u, dh, dg0, du0)
+    gdg, gdu = ops.silu_gate_bwd(dev(g), dev(u), dev(dh), dev(dg0), dev(du0))
+    assert_parity(host(gdg), wdg, "dg+"), assert_parity(host(gdu), wdu, "du+")
+
+
+# ---------------------------------------------------------------- causal softmax
+@pytest.mark.parametrize("S,H", [(128, 4), (512, 3), (8, 1), (2048, 2)])
+def test_causal_softmax(ops, oracle, S, H):
+    say("causal_softmax", S, H)
+    r = rng(500 + S)
+    s16, dp = randn16(r, (S, H, S), 2.0), randn16(r, (S, H, S), 3.0)
+    wp = oracle.causal_softmax_fwd(s16)
+    gp = host(ops.causal_softmax_fwd(dev(s16)))
+    assert_parity(gp, wp, "p16")
+    iu = np.triu_indices(S, 1)
+    assert np.all(gp[iu[0], :, iu[1]] == 0)
+    wds = oracle.causal_softmax_bwd(s16, dp)
+    gds = host(ops.causal_softmax_bwd(dev(s16), dev(dp)))
+    assert_parity(gds, wds, "ds16")
+    assert np.all(gds[iu[0], :, iu[1]] == 0)
+
+
+# ---------------------------------------------------------------- softmax cross-entropy
+@pytest.mark.parametrize("N,V", [(64, 32000), (128, 1024), (3, 8), (5, 40000)])
+def test_softmax_ce(ops, oracle, N, V):
+    say("softmax_ce", N, V)
+    r = rng(600 + V)
+    logit = randn16(r, (N, V), 2.0)
+    tok = r.integers(0, V, N).astype(np.uint16)
+    scale = r.random(N).astype(np.float32)
+    scale[0] = 0.0
+    wprob, wloss, wamax = oracle.softmax_ce_fwd(logit, tok)
+    gprob, gloss, gamax = ops.softmax_ce_fwd(dev(logit), dev(tok))
+    assert_parity(host(gprob), wprob, "prob", l2=1e-5, mx=1e-4)
+    assert_parity(host(gloss), wloss, "loss", l2=1e-5, mx=1e-4)
+    assert np.array_equal(host(gamax).view(np.uint16), wamax)          # index work: bit-exact
+    wd = oracle.softmax_ce_bwd(logit, tok, scale)
+    gd = host(ops.softmax_ce_bwd(dev(logit), dev(tok), dev(scale)))
+    assert_parity(gd, wd, "dlogit")
+    assert exact_frac(gd, wd) > 0.995
+    assert np.all(gd[0] == 0)
+    d0 = randn16(r, (N, V), 0.01)
+    ga = host(ops.softmax_ce_bwd(dev(logit), dev(tok), dev(scale), dev(d0)))
+    assert_parity(ga, oracle.accumulate_f16(d0, wd), "dlogit+")
+
+
+def test_softmax_ce_argmax_ties_and_bad_token(ops, oracle):
+    logit = np.zeros((2, 64), np.float16)
+    logit[0, [9, 40]] = 2.0
+    logit[1, 63] = 1.0
+    tok = np.array([1, 2], np.uint16)
+    _, _, amax = ops.softmax_ce_fwd(dev(logit), dev(tok), want_prob=False)
+    assert host(amax).view(np.uint16).tolist() == [9, 63]
+    with pytest.raises(IndexError):
+        ops.softmax_ce_fwd(dev(logit), dev(np.array([1, 64], np.uint16)))
+
+
+# ---------------------------------------------------------------- embedding
+@pytest.mark.parametrize("V,D,S", [(32000, 3200, 2048), (1024, 256, 128), (16, 8, 50)])
+def test_embedding(ops, oracle, V, D, S):
+    say("embedding", V, D, S)
+    r = rng(700 + V)
+    W = randn16(r, (V, D), 0.02)
+    tok = r.integers(0, V, S).astype(np.uint16)
+    tok[S // 2] = tok[0]                                   # force a repeated id
+    got = host(ops.embed_fwd(dev(W), dev(tok)))
+    assert np.array_equal(got.view(np.uint16), oracle.embed_fwd(W, tok).view(np.uint16))
+    dy = randn16(r, (S, D))
+    want = oracle.embed_bwd(V, tok, dy)
+    got = host(ops.embed_bwd(V, dev(tok), dev(dy)))
+    assert_parity(got, want, "dW")
+    assert exact_frac(got, want) > 0.9999
+    never = np.setdiff1d(np.arange(V), tok)
+    assert np.all(got[never] == 0)
+    bad = tok.copy()
+    bad[1] = V
+    with pytest.raises(IndexError):
+        ops.embed_fwd(dev(W), dev(bad))
+
+
+# ---------------------------------------------------------------- accumulate / add
+def test_accumulate_and_add(ops, oracle):
+    r = rng(800)
+    a, b = randn16(r, (100003,)), randn16(r, (100003,))
+    got = host(ops.add_f16(dev(a), dev(b)))
+    assert np.array_equal(got.view(np.uint16), oracle.accumulate_f16(a, b).view(np.uint16))
+    t = dev(a)
+    ops.accumulate_1d(t, dev(b))
+    assert np.array_equal(host(t).view(np.uint16), oracle.accumulate_f16(a, b).view(np.uint16))
+    f, g = r.standard_normal(1000).astype(np.float32), r.standard_normal(1000).astype(np.float32)
+    t = dev(f)
+    ops.accumulate_1d(t, dev(g))
+    assert np.array_equal(host(t), f + g)
+    u, v = r.integers(0, 30000, 1000).astype(np.uint16), r.integers(0, 30000, 1000).astype(np.uint16)
+    t = dev(u)
+    ops.accumulate_1d(t, dev(v))
+    assert np.array_equal(host(t).view(np.uint16), (u + v).astype(np.uint16))
+
+
+# ---------------------------------------------------------------- GEMM
+GEMM_SHAPES = [
+    (128, 128, 32), (256, 384, 192), (100, 72, 40), (128, 688, 256), (128, 256, 688),
+    (61, 35, 27),            # nothing aligned: scalar path
+    (64, 100, 64), (64, 64, 100),   # head_dim 100: 8-byte path
+]
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_small(ops, oracle, ta, tb, M, N, K):
+    say("gemm", ta, tb, M, N, K)
+    r = rng(900 + M + 3 * N + 7 * K + 2 * ta + tb)
+    A = randn16(r, (K, M) if ta else (M, K))
+    B = randn16(r, (N, K) if tb else (K, N))
+    C0 = randn16(r, (M, N))
+    for alpha, beta in [(1.0, 0.0), (0.1, 1.0)]:
+        want = oracle.matmul(ta, tb, A, B, alpha, beta, C0)
+        c = dev(C0)
+        got = host(ops.gemm(dev(A), dev(B), bool(ta), bool(tb), alpha, beta, c))
+        assert_parity(got, want, "gemm")
+        assert exact_frac(got, want) > 0.98
+
+
+@pytest.mark.parametrize("case", ["fwd", "dgrad", "wgrad"])
+def test_gemm_projection_shapes(ops, oracle, case):
+    """The three GEMMs of one projection at a reduced token count (oracle finishes in seconds)."""
+    say("gemm projection", case)
+    r = rng(950)
+    T, Din, Dout = 256, 3200, 8640
+    x, W, dy = randn16(r, (T, Din)), randn16(r, (Dout, Din), 0.02), randn16(r, (T, Dout))
+    if case == "fwd":
+        got, want = ops.gemm(dev(x), dev(W), False, True), oracle.matmul(0, 1, x, W)
+    elif case == "dgrad":
+        got, want = ops.gemm(dev(dy), dev(W), False, False), oracle.matmul(0, 0, dy, W)
+    else:
+        got, want = ops.gemm(dev(dy), dev(x), True, False), oracle.matmul(1, 0, dy, x)
+    assert_parity(host(got), want, case)
+
+
+def test_gemm_linearity_full_size(ops):
+    """At full size (no oracle): (A1 + A2) B == A1 B + A2 B up to rounding, against fp32 torch."""
+    say("gemm full size")
+    torch.manual_seed(0)
+    M, N, K = 2048, 3200, 3200
+    A = torch.randn(M, K, device="cuda").half()
+    B = (torch.randn(N, K, device="cuda") * 0.02).half()
+    got = ops.gemm(A, B, False, True)
+    ref = (A.float() @ B.float().T)
+    err = (got.float() - ref).norm() / ref.norm()
+    assert err < 5e-4, err
+    got = ops.gemm(A, got, True, False)          # [K,M]^T... (K x N) wgrad-shaped product
+    ref = (A.float().T @ ref.half().float())
+    assert (got.float() - ref).norm() / ref.norm() < 5e-4
+
+
+def test_gemm_colmajor_entry(ops, oracle):
+    """The cuBLAS-shaped entry: row-major callers pass operands swapped (thunk/op.rs:4469-4491)."""
+    import ctypes as C
+    from cacti_amd import ffi
+    r = rng(960)
+    M, N, K = 96, 80, 64
+    x, W = randn16(r, (M, K)), randn16(r, (N, K))
+    want = oracle.matmul(0, 1, x, W)             # row-major y = x W^T
+    y = torch.empty((M, N), dtype=torch.float16, device="cuda")
+    one, zero = C.c_float(1.0), C.c_float(0.0)
+    # column-major: y^T (N x M) = W (as col-major K x N, transposed) * x (col-major K x M)
+    ffi.call("cacti_hip_gemm_colmajor_f16", 1, 0, N, M, K, C.byref(one), dev(W).data_ptr(), K,
+             dev(x).data_ptr(), K, C.byref(zero), y.data_ptr(), N,
+             torch.cuda.current_stream().cuda_stream)
+    assert_parity(host(y), want, "colmajor")
+
+
+# ---------------------------------------------------------------- attention block
+@pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100)])
+def test_attention_block_via_thunks(ops, oracle, S, H, Dh):
+    """Q K^T -> causal softmax -> P V and the adjoint, composed as the reference stages them."""
+    say("attention", S, H, Dh)
+    r = rng(1000 + S)
+    alpha = float(np.float32(1.0) / np.sqrt(np.float32(Dh)))
+    q, k, v, dO = (randn16(r, (S, H, Dh)) for _ in range(4))
+    ws16, wp16, wo = oracle.attention_fwd(q, k, v, alpha)
+    dq_, dk_, dv_ = oracle.attention_bwd(q, k, v, dO, alpha)
+    Q, K_, V_, DO = dev(q), dev(k), dev(v), dev(dO)
+    s16 = ops.block_matmul_qk(Q, K_, alpha)
+    assert_parity(host(s16), ws16, "s16")
+    p16 = ops.causal_softmax_fwd(s16)
+    assert_parity(host(p16), wp16, "p16")
+    o = ops.block_matmul_pv(p16, V_)
+    assert_parity(host(o), wo, "o")
+    ld, lds = H * Dh, H * S
+    dv = torch.empty_like(V_); dp = torch.empty_like(s16)
+    dq = torch.empty_like(Q); dk = torch.empty_like(Q)
+    ops.gemm_strided_batched(True, False, H, S, Dh, S, 1.0, p16, lds, S, DO, ld, Dh, 0.0, dv, ld, Dh)
+    ops.gemm_strided_batched(False, True, H, S, S, Dh, 1.0, DO, ld, Dh, V_, ld, Dh, 0.0, dp, lds, S)
+    ds = ops.causal_softmax_bwd(s16, dp)
+    ops.gemm_strided_batched(True, False, H, S, Dh, S, alpha, ds, lds, S, Q, ld, Dh, 0.0, dk, ld, Dh)
+    ops.gemm_strided_batched(False, False, H, S, Dh, S, alpha, ds, lds, S, K_, ld, Dh, 0.0, dq, ld, Dh)
+    assert_parity(host(dv), dv_, "dv")
+    assert_parity(host(dq), dq_, "dq")
+    assert_parity(host(dk), dk_, "dk")
