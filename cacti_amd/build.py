@@ -17,7 +17,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden",
     "-ffp-contract=off",                       # keep the reference's per-thunk rounding points
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+    "-Wall", "-Wno-unused-function", "-Wno-unused-value", "-Wno-unused-result", "-Wno-unknown-warning-option",
 ]
 
 

@@ -1,0 +1,380 @@
+// The LLaMA training cycle staged on the spine, and the runtime's C ABI.
+// Llama::apply, src/librarium/llama.rs:420-548; step recipe,
+// examples/open_llama_3b_train.rs:350-389.
+#include <math.h>
+#include <string.h>
+
+#include <string>
+
+#include "../../include/cacti_hip_runtime.h"
+#include "common.h"
+#include "thunks.h"
+
+using namespace cacti;
+
+struct cacti_ctx {
+    Ctx c;
+};
+
+struct LayerCells {
+    CellPtr pre_norm, q, k, v, o, post_norm, gate, up, down;
+};
+
+struct cacti_llama {
+    cacti_ctx *ctx;
+    cacti_llama_cfg cfg;
+    std::vector<CellPtr> params, grads;
+    std::vector<std::string> names;
+    CellPtr embed, head_norm, lm_head;
+    std::vector<LayerCells> layers;
+    CellPtr cos, sin;
+    CellPtr in_tok, in_lm_tok, in_loss_scale;
+    CellPtr out_logit = 0, out_loss = 0, out_amax = 0, out_prob = 0;
+};
+
+namespace {
+
+CellPtr new_param(cacti_llama *m, const std::string &name, std::vector<int64_t> shape)
+{
+    Ctx &c = m->ctx->c;
+    CellPtr p = c.cell_new(CellType(shape, F16), true, name.c_str());
+    CellPtr g = c.cell_new(CellType(shape, F16), true, ("grad:" + name).c_str());
+    m->params.push_back(p);
+    m->grads.push_back(g);
+    m->names.push_back(name);
+    return p;
+}
+
+// one staged thunk with a single output
+int ap(Ctx &c, std::unique_ptr<ThunkSpec> spec, const std::vector<CellPtr> &args, CellPtr *out)
+{
+    std::vector<CellPtr> outs;
+    int rc = c.stage_apply(c.add_thunk(std::move(spec)), args, &outs);
+    if (rc) return rc;
+    *out = outs[0];
+    return 0;
+}
+
+#define TRY(x)             \
+    do {                   \
+        int rc_ = (x);     \
+        if (rc_) return rc_; \
+    } while (0)
+
+}  // namespace
+
+// ===========================================================================
+// context + spine
+
+CACTI_API int cacti_ctx_create(cacti_ctx **ctx, int dev, size_t pool_bytes, int host_pagelocked)
+{
+    CACTI_REQUIRE(ctx, CACTI_E_INVALID, "ctx_create: null out pointer");
+    cacti_ctx *x = new cacti_ctx();
+    int rc = x->c.init(dev, pool_bytes, host_pagelocked);
+    if (rc) {
+        delete x;
+        return rc;
+    }
+    *ctx = x;
+    return 0;
+}
+
+CACTI_API int cacti_ctx_destroy(cacti_ctx *ctx)
+{
+    delete ctx;
+    return 0;
+}
+
+CACTI_API int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out)
+{
+    CACTI_REQUIRE(ctx && out, CACTI_E_INVALID, "ctx_stats: null pointer");
+    static_assert(sizeof(cacti_stats) == sizeof(Stats), "stats layouts must agree");
+    ctx->c.stats(reinterpret_cast<Stats *>(out));
+    return 0;
+}
+
+CACTI_API int cacti_ctx_sync(cacti_ctx *ctx) { return ctx->c.sync(); }
+CACTI_API void *cacti_ctx_stream(cacti_ctx *ctx) { return (void *)ctx->c.stream(); }
+
+CACTI_API int cacti_ctx_set_timing(cacti_ctx *ctx, int on)
+{
+    ctx->c.set_timing(on != 0);
+    return 0;
+}
+
+CACTI_API int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap)
+{
+    CACTI_REQUIRE(ctx && buf && cap > 0, CACTI_E_INVALID, "timing_report: null pointer");
+    size_t n = 0;
+    buf[0] = 0;
+    for (auto &kv : ctx->c.timings()) {
+        int w = snprintf(buf + n, cap - n, "%s %llu %.4f\n", kv.first.c_str(),
+                         (unsigned long long)kv.second.second, kv.second.first);
+        if (w < 0 || (size_t)w >= cap - n) break;
+        n += (size_t)w;
+    }
+    return 0;
+}
+
+CACTI_API int cacti_reset(cacti_ctx *ctx)
+{
+    ctx->c.reset();
+    return 0;
+}
+CACTI_API int cacti_compile(cacti_ctx *ctx) { return ctx->c.compile(); }
+CACTI_API int cacti_resume(cacti_ctx *ctx, int *yield_cell)
+{
+    CellPtr y = 0;
+    int rc = ctx->c.resume(&y);
+    if (yield_cell) *yield_cell = y;
+    return rc;
+}
+CACTI_API int cacti_resume_put(cacti_ctx *ctx, int cell, const void *host, size_t bytes)
+{
+    return ctx->c.resume_put(cell, host, bytes);
+}
+CACTI_API int cacti_cell_bytes(cacti_ctx *ctx, int cell, size_t *bytes)
+{
+    CACTI_REQUIRE(ctx && bytes && cell > 0, CACTI_E_INVALID, "cell_bytes: bad arguments");
+    *bytes = ctx->c.cell(cell).ty.bytes();
+    return 0;
+}
+CACTI_API int cacti_cell_get(cacti_ctx *ctx, int cell, void *host, size_t bytes)
+{
+    return ctx->c.cell_get(cell, host, bytes);
+}
+CACTI_API int cacti_log_len(cacti_ctx *ctx) { return (int)ctx->c.log().size(); }
+CACTI_API const char *cacti_log_name(cacti_ctx *ctx, int i)
+{
+    if (i < 0 || (size_t)i >= ctx->c.log().size()) return "";
+    return ctx->c.entry_name((size_t)i);
+}
+
+// ===========================================================================
+// pool policy over a plain offset range
+
+struct cacti_mempool {
+    MemPool p;
+};
+
+CACTI_API int cacti_mempool_create(cacti_mempool **pool, uint64_t cap)
+{
+    CACTI_REQUIRE(pool, CACTI_E_INVALID, "mempool_create: null out pointer");
+    *pool = new cacti_mempool();
+    (*pool)->p.reset((size_t)cap);
+    return 0;
+}
+CACTI_API int cacti_mempool_destroy(cacti_mempool *pool)
+{
+    delete pool;
+    return 0;
+}
+CACTI_API uint64_t cacti_mempool_alloc(cacti_mempool *pool, uint64_t bytes)
+{
+    size_t o = pool->p.alloc((size_t)bytes);
+    return o == kNoOffset ? UINT64_MAX : (uint64_t)o;
+}
+CACTI_API int cacti_mempool_free(cacti_mempool *pool, uint64_t offset)
+{
+    CACTI_REQUIRE(pool->p.size_of((size_t)offset) != 0, CACTI_E_INVALID,
+                  "mempool_free: offset %llu is not an allocation", (unsigned long long)offset);
+    pool->p.free((size_t)offset);
+    return 0;
+}
+CACTI_API int cacti_mempool_stats(cacti_mempool *pool, uint64_t out[5])
+{
+    out[0] = pool->p.cap();
+    out[1] = pool->p.used();
+    out[2] = pool->p.peak();
+    out[3] = pool->p.front();
+    out[4] = pool->p.largest_free();
+    return 0;
+}
+
+// ===========================================================================
+// model
+
+CACTI_API int cacti_llama_create(cacti_ctx *ctx, const cacti_llama_cfg *cfg, cacti_llama **model)
+{
+    CACTI_REQUIRE(ctx && cfg && model, CACTI_E_INVALID, "llama_create: null pointer");
+    CACTI_REQUIRE(cfg->S > 0 && cfg->L >= 0 && cfg->H > 0 && cfg->H * cfg->Dh == cfg->D &&
+                      cfg->F > 0 && cfg->V > 0 && cfg->V <= 65536 && cfg->Dh % 2 == 0,
+                  CACTI_E_INVALID, "llama_create: inconsistent configuration");
+    cacti_llama *m = new cacti_llama();
+    m->ctx = ctx;
+    m->cfg = *cfg;
+    Ctx &c = ctx->c;
+    const int64_t D = cfg->D, F = cfg->F, V = cfg->V, S = cfg->S;
+    m->embed = new_param(m, "embed", {V, D});
+    for (int64_t l = 0; l < cfg->L; l++) {
+        LayerCells lc;
+        const std::string p = "l" + std::to_string(l) + ".";
+        lc.pre_norm = new_param(m, p + "pre_norm", {D});
+        lc.q = new_param(m, p + "q", {D, D});
+        lc.k = new_param(m, p + "k", {D, D});
+        lc.v = new_param(m, p + "v", {D, D});
+        lc.o = new_param(m, p + "o", {D, D});
+        lc.post_norm = new_param(m, p + "post_norm", {D});
+        lc.gate = new_param(m, p + "gate", {F, D});
+        lc.up = new_param(m, p + "up", {F, D});
+        lc.down = new_param(m, p + "down", {D, F});
+        m->layers.push_back(lc);
+    }
+    m->head_norm = new_param(m, "head_norm", {D});
+    m->lm_head = new_param(m, "lm_head", {V, D});
+    // init_constants, src/librarium/llama.rs:389-411: computed once, kept on the device
+    m->cos = c.cell_new(CellType({S, cfg->Dh}, F16), true, "cos");
+    m->sin = c.cell_new(CellType({S, cfg->Dh}, F16), true, "sin");
+    c.set_const(m->cos);
+    c.set_const(m->sin);
+    int rc = c.ensure_vmem(m->cos, false);
+    if (!rc) rc = c.ensure_vmem(m->sin, false);
+    if (!rc)
+        rc = cacti_hip_rope_tables(S, cfg->Dh, c.dev_ptr(c.cell(m->cos).voff),
+                                   c.dev_ptr(c.cell(m->sin).voff), (void *)c.stream());
+    if (rc) {
+        delete m;
+        return rc;
+    }
+    c.cell(m->cos).v_valid = c.cell(m->sin).v_valid = true;
+    // fresh_input, src/librarium/llama.rs:380-387
+    m->in_tok = c.cell_new(CellType({S}, U16), true, "in_tok");
+    m->in_lm_tok = c.cell_new(CellType({S}, U16), true, "in_lm_tok");
+    m->in_loss_scale = c.cell_new(CellType({S}, F32), true, "in_lm_loss_scale");
+    c.set_const(m->in_tok);
+    c.set_const(m->in_lm_tok);
+    c.set_const(m->in_loss_scale);
+    *model = m;
+    return 0;
+}
+
+CACTI_API int cacti_llama_destroy(cacti_llama *model)
+{
+    delete model;
+    return 0;
+}
+
+CACTI_API int cacti_llama_num_params(cacti_llama *m) { return (int)m->params.size(); }
+
+CACTI_API int cacti_llama_param_info(cacti_llama *m, int i, char *name, size_t name_cap,
+                                     int64_t *rows, int64_t *cols, int *param_cell, int *grad_cell)
+{
+    CACTI_REQUIRE(m && i >= 0 && (size_t)i < m->params.size(), CACTI_E_INVALID,
+                  "param_info: index out of range");
+    const CellType &t = m->ctx->c.cell(m->params[i]).ty;
+    if (name && name_cap) snprintf(name, name_cap, "%s", m->names[i].c_str());
+    if (rows) *rows = t.shape[0];
+    if (cols) *cols = t.shape.size() > 1 ? t.shape[1] : 1;
+    if (param_cell) *param_cell = m->params[i];
+    if (grad_cell) *grad_cell = m->grads[i];
+    return 0;
+}
+
+CACTI_API int cacti_llama_param_put(cacti_llama *m, int i, const void *host, size_t bytes)
+{
+    CACTI_REQUIRE(m && i >= 0 && (size_t)i < m->params.size(), CACTI_E_INVALID,
+                  "param_put: index out of range");
+    return m->ctx->c.cell_put(m->params[i], host, bytes);
+}
+
+CACTI_API int cacti_llama_grad_get(cacti_llama *m, int i, void *host, size_t bytes)
+{
+    CACTI_REQUIRE(m && i >= 0 && (size_t)i < m->grads.size(), CACTI_E_INVALID,
+                  "grad_get: index out of range");
+    return m->ctx->c.cell_get(m->grads[i], host, bytes);
+}
+
+CACTI_API int cacti_llama_io_cells(cacti_llama *m, int *tok, int *lm_tok, int *loss_scale,
+                                   int *logit, int *loss, int *amax, int *prob)
+{
+    if (tok) *tok = m->in_tok;
+    if (lm_tok) *lm_tok = m->in_lm_tok;
+    if (loss_scale) *loss_scale = m->in_loss_scale;
+    if (logit) *logit = m->out_logit;
+    if (loss) *loss = m->out_loss;
+    if (amax) *amax = m->out_amax;
+    if (prob) *prob = m->out_prob;
+    return 0;
+}
+
+CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
+{
+    Ctx &c = m->ctx->c;
+    const cacti_llama_cfg &g = m->cfg;
+    const float alpha = 1.0f / sqrtf((float)g.Dh);
+    // in_.in_tok.mem_set_yield_() ..., examples/open_llama_3b_train.rs:350-358
+    c.stage_yield_set(m->in_tok);
+    c.stage_yield_set(m->in_lm_tok);
+    c.stage_yield_set(m->in_loss_scale);
+
+    CellPtr stream;
+    TRY(ap(c, make_embed(), {m->embed, m->in_tok}, &stream));
+    for (size_t l = 0; l < m->layers.size(); l++) {
+        const LayerCells &w = m->layers[l];
+        CellPtr pre, q, k, v, qr, kr, s16, p16, attn, o, x1, post, up, gate, h, down, x2;
+        TRY(ap(c, make_rms_norm(g.eps), {stream, w.pre_norm}, &pre));
+        TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.q}, &q));
+        TRY(ap(c, make_rope(g.H), {q, m->cos, m->sin}, &qr));
+        TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
+        TRY(ap(c, make_rope(g.H), {k, m->cos, m->sin}, &kr));
+        TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.v}, &v));
+        TRY(ap(c, make_block_matmul(false, true, alpha, g.H), {qr, kr}, &s16));
+        TRY(ap(c, make_causal_softmax(g.H), {s16}, &p16));
+        TRY(ap(c, make_block_matmul(false, false, 1.f, g.H), {p16, v}, &attn));
+        TRY(ap(c, make_matmul(false, true, 1.f), {attn, w.o}, &o));
+        TRY(ap(c, make_add(), {stream, o}, &x1));
+        TRY(ap(c, make_rms_norm(g.eps), {x1, w.post_norm}, &post));
+        TRY(ap(c, make_matmul(false, true, 1.f), {post, w.up}, &up));
+        TRY(ap(c, make_matmul(false, true, 1.f), {post, w.gate}, &gate));
+        TRY(ap(c, make_silu_gate(), {gate, up}, &h));
+        TRY(ap(c, make_matmul(false, true, 1.f), {h, w.down}, &down));
+        TRY(ap(c, make_add(), {x1, down}, &x2));
+        stream = x2;
+    }
+    CellPtr hn, logit;
+    TRY(ap(c, make_rms_norm(g.eps), {stream, m->head_norm}, &hn));
+    TRY(ap(c, make_matmul(false, true, 1.f), {hn, m->lm_head}, &logit));
+    std::vector<CellPtr> outs;
+    TRY(c.stage_apply(c.add_thunk(make_softmax_ce(want_prob != 0)), {logit, m->in_lm_tok}, &outs));
+    m->out_logit = logit;
+    m->out_loss = outs[0];
+    m->out_amax = outs[1];
+    m->out_prob = want_prob ? outs[2] : 0;
+    c.keep(m->out_logit);                                  // .keep(), llama.rs:541-546
+    c.keep(m->out_loss);
+    c.keep(m->out_amax);
+    if (m->out_prob) c.keep(m->out_prob);
+
+    if (want_grad) {
+        // sink.add(out_lm_loss, in_lm_loss_scale); grad_map.add(p, g); vadd_vjp(src, sink)
+        c.adj_seed(m->out_loss, m->in_loss_scale);
+        for (size_t i = 0; i < m->params.size(); i++) c.adj_bind(m->params[i], m->grads[i]);
+        TRY(c.vadd_vjp());
+    }
+    return 0;
+}
+
+CACTI_API int cacti_llama_step(cacti_llama *m, const uint16_t *tok, const uint16_t *lm_tok,
+                               const float *loss_scale, int want_prob, int want_grad,
+                               float *loss_out)
+{
+    CACTI_REQUIRE(m && tok && lm_tok && loss_scale, CACTI_E_INVALID, "llama_step: null input");
+    Ctx &c = m->ctx->c;
+    const size_t S = (size_t)m->cfg.S;
+    c.reset();
+    TRY(cacti_llama_stage(m, want_prob, want_grad));
+    TRY(c.compile());
+    for (;;) {
+        CellPtr y = 0;
+        int rc = c.resume(&y);
+        if (rc == R_DONE) break;
+        if (rc != R_YIELD) return rc;
+        if (y == m->in_tok) TRY(c.resume_put(y, tok, S * 2));
+        else if (y == m->in_lm_tok) TRY(c.resume_put(y, lm_tok, S * 2));
+        else if (y == m->in_loss_scale) TRY(c.resume_put(y, loss_scale, S * 4));
+        else CACTI_REQUIRE(false, CACTI_E_STATE, "llama_step: unexpected yield of cell %d", y);
+    }
+    TRY(c.check_status());
+    if (loss_out) TRY(c.cell_get(m->out_loss, loss_out, S * 4));
+    return c.sync();
+}

@@ -1,0 +1,617 @@
+// Device context, pooled allocator with host spill, cells and the spine interpreter.
+#include "runtime.h"
+
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+
+#include "common.h"
+
+namespace cacti {
+
+// ===========================================================================
+// MemPool
+
+void MemPool::reset(size_t cap)
+{
+    cap_ = cap;
+    front_ = used_ = peak_ = 0;
+    free_.clear();
+    alloc_.clear();
+}
+
+size_t MemPool::alloc(size_t bytes)
+{
+    if (bytes == 0) bytes = 1;
+    const size_t req = (bytes + kAllocAlign - 1) / kAllocAlign * kAllocAlign;
+    size_t off = kNoOffset;
+    for (auto it = free_.begin(); it != free_.end(); ++it) {      // first fit, lowest offset
+        if (it->second >= req) {
+            off = it->first;
+            const size_t rest = it->second - req;
+            free_.erase(it);
+            if (rest) free_[off + req] = rest;
+            break;
+        }
+    }
+    if (off == kNoOffset) {
+        if (front_ + req > cap_) return kNoOffset;
+        off = front_;
+        front_ += req;
+    }
+    alloc_[off] = req;
+    used_ += req;
+    if (used_ > peak_) peak_ = used_;
+    return off;
+}
+
+void MemPool::free(size_t off)
+{
+    auto it = alloc_.find(off);
+    if (it == alloc_.end()) return;
+    size_t sz = it->second;
+    alloc_.erase(it);
+    used_ -= sz;
+    auto next = free_.lower_bound(off);
+    if (next != free_.end() && off + sz == next->first) {         // merge with the next region
+        sz += next->second;
+        next = free_.erase(next);
+    }
+    if (next != free_.begin()) {                                  // merge with the previous one
+        auto prev = std::prev(next);
+        if (prev->first + prev->second == off) {
+            off = prev->first;
+            sz += prev->second;
+            free_.erase(prev);
+        }
+    }
+    if (off + sz == front_)
+        front_ = off;                                             // retract the bump cursor
+    else
+        free_[off] = sz;
+}
+
+size_t MemPool::size_of(size_t off) const
+{
+    auto it = alloc_.find(off);
+    return it == alloc_.end() ? 0 : it->second;
+}
+
+size_t MemPool::largest_free() const
+{
+    size_t best = cap_ - front_;
+    for (auto &kv : free_) best = std::max(best, kv.second);
+    return best;
+}
+
+// ===========================================================================
+// Ctx
+
+Ctx::Ctx() { cells_.emplace_back(); cells_[0].alive = false; }   // cell 0 = nil
+
+Ctx::~Ctx()
+{
+    if (stream_) hipStreamSynchronize(stream_);
+    for (auto &c : cells_) host_free(c);
+    if (ev0_) hipEventDestroy(ev0_);
+    if (ev1_) hipEventDestroy(ev1_);
+    if (base_) hipFree(base_);
+    if (own_stream_ && stream_) hipStreamDestroy(stream_);
+}
+
+int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
+{
+    dev_ = dev;
+    host_pagelocked_ = host_pagelocked;
+    CACTI_HIP(hipSetDevice(dev));
+    size_t avail = 0, total = 0;
+    CACTI_HIP(hipMemGetInfo(&avail, &total));
+    if (pool_bytes == 0) {
+        // default reserve: 90.01 % of the device, src/ctx.rs:43, src/pctx/nvgpu.rs:1434-1463
+        size_t want = (size_t)(((unsigned __int128)total * 9001 + 9999) / 10000);
+        size_t room = avail > (512u << 20) ? avail - (512u << 20) : avail / 2;
+        pool_bytes = std::min(want, room);
+    }
+    pool_bytes = (pool_bytes >> 16) << 16;                        // 64 KiB granules
+    CACTI_REQUIRE(pool_bytes > 0 && pool_bytes <= avail, CACTI_E_OOM,
+                  "ctx: cannot reserve %zu bytes (%zu available of %zu); lower the pool cap",
+                  pool_bytes, avail, total);
+    CACTI_HIP(hipMalloc((void **)&base_, pool_bytes));
+    CACTI_REQUIRE(((uintptr_t)base_ % kAllocAlign) == 0, CACTI_E_STATE, "ctx: misaligned reserve");
+    pool_.reset(pool_bytes);
+    status_off_ = pool_.alloc(kAllocAlign);
+    CACTI_HIP(hipMemset(base_ + status_off_, 0, kAllocAlign));
+    CACTI_HIP(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
+    own_stream_ = true;
+    CACTI_HIP(hipEventCreate(&ev0_));
+    CACTI_HIP(hipEventCreate(&ev1_));
+    return 0;
+}
+
+int Ctx::sync()
+{
+    CACTI_HIP(hipStreamSynchronize(stream_));
+    return 0;
+}
+
+int Ctx::check_status()
+{
+    int v = 0;
+    CACTI_HIP(hipMemcpyAsync(&v, status_ptr(), sizeof(int), hipMemcpyDeviceToHost, stream_));
+    CACTI_HIP(hipStreamSynchronize(stream_));
+    if (v) {
+        CACTI_HIP(hipMemsetAsync(status_ptr(), 0, sizeof(int), stream_));
+        set_error("token id out of range at position %d", v - 1);
+        return CACTI_E_INDEX;
+    }
+    return 0;
+}
+
+CellPtr Ctx::cell_new(const CellType &ty, bool stable, const char *name)
+{
+    Cell c;
+    c.ty = ty;
+    c.stable = stable;
+    c.name = name ? name : "";
+    cells_.push_back(std::move(c));
+    return (CellPtr)(cells_.size() - 1);
+}
+
+int Ctx::host_alloc(Cell &c)
+{
+    if (c.hptr) return 0;
+    const size_t n = std::max<size_t>(c.ty.bytes(), 1);
+    if (host_pagelocked_) {
+        CACTI_HIP(hipHostMalloc(&c.hptr, n, hipHostMallocDefault));
+    } else {
+        c.hptr = malloc(n);
+        CACTI_REQUIRE(c.hptr, CACTI_E_OOM, "host malloc of %zu bytes failed", n);
+    }
+    host_bytes_ += n;
+    return 0;
+}
+
+void Ctx::host_free(Cell &c)
+{
+    if (!c.hptr) return;
+    if (host_pagelocked_) hipHostFree(c.hptr); else free(c.hptr);
+    host_bytes_ -= std::max<size_t>(c.ty.bytes(), 1);
+    c.hptr = nullptr;
+    c.h_valid = false;
+}
+
+int Ctx::cell_free_all(CellPtr ci)
+{
+    Cell &c = cells_[ci];
+    if (c.voff != kNoOffset) {
+        pool_.free(c.voff);
+        c.voff = kNoOffset;
+    }
+    c.v_valid = false;
+    if (c.hptr) {
+        // a host buffer may still be the source or target of an in-flight copy
+        if (stream_) hipStreamSynchronize(stream_);
+        host_free(c);
+    }
+    return 0;
+}
+
+int Ctx::cell_put(CellPtr ci, const void *host, size_t bytes)
+{
+    Cell &c = cells_[ci];
+    CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "cell_put: dead cell %d", ci);
+    CACTI_REQUIRE(bytes == c.ty.bytes(), CACTI_E_INVALID, "cell_put: %zu bytes given, cell %s has %zu",
+                  bytes, c.name.c_str(), c.ty.bytes());
+    // an earlier upload from this host buffer may still be in flight
+    CACTI_HIP(hipStreamSynchronize(stream_));
+    int rc = host_alloc(c);
+    if (rc) return rc;
+    memcpy(c.hptr, host, bytes);
+    c.h_valid = true;
+    c.v_valid = false;
+    return 0;
+}
+
+int Ctx::cell_get(CellPtr ci, void *host, size_t bytes)
+{
+    Cell &c = cells_[ci];
+    CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "cell_get: dead cell %d", ci);
+    CACTI_REQUIRE(bytes == c.ty.bytes(), CACTI_E_INVALID, "cell_get: %zu bytes asked, cell %s has %zu",
+                  bytes, c.name.c_str(), c.ty.bytes());
+    if (c.v_valid) {
+        CACTI_HIP(hipMemcpyAsync(host, dev_ptr(c.voff), bytes, hipMemcpyDeviceToHost, stream_));
+        CACTI_HIP(hipStreamSynchronize(stream_));
+        bytes_d2h_ += bytes;
+        return 0;
+    }
+    CACTI_REQUIRE(c.h_valid, CACTI_E_STATE, "cell_get: cell %s holds no value", c.name.c_str());
+    CACTI_HIP(hipStreamSynchronize(stream_));
+    memcpy(host, c.hptr, bytes);
+    return 0;
+}
+
+// VMem -> Mem: keep (or make) a host copy of the current version, then drop the device
+// replica.  PCell::read_loc(.., Locus::Mem) + yeet, src/pctx/nvgpu.rs:2198-2251.
+int Ctx::evict(CellPtr ci)
+{
+    Cell &c = cells_[ci];
+    if (c.voff == kNoOffset) return 0;
+    if (c.v_valid && !c.h_valid) {
+        int rc = host_alloc(c);
+        if (rc) return rc;
+        CACTI_HIP(hipMemcpyAsync(c.hptr, dev_ptr(c.voff), c.ty.bytes(), hipMemcpyDeviceToHost,
+                                 stream_));
+        if (!host_pagelocked_) CACTI_HIP(hipStreamSynchronize(stream_));
+        c.h_valid = true;
+        bytes_d2h_ += c.ty.bytes();
+    }
+    pool_.free(c.voff);          // later users of the region are ordered after the copy
+    c.voff = kNoOffset;
+    c.v_valid = false;
+    n_evict_++;
+    return 0;
+}
+
+// NvGpuMemPool::_try_soft_oom, src/pctx/nvgpu.rs:2004-2283: dead cells are already freed
+// at their Unlive entry; here live, unpinned cells are spilled in creation order, first
+// only those at least as large as the request, then any.
+int Ctx::try_soft_oom(size_t need)
+{
+    n_soft_oom_++;
+    const size_t req = (need + kAllocAlign - 1) / kAllocAlign * kAllocAlign;
+    for (int pass = 0; pass < 2; pass++) {
+        for (size_t i = 1; i < cells_.size(); i++) {
+            Cell &c = cells_[i];
+            if (!c.alive || c.voff == kNoOffset || c.pin > 0) continue;
+            if (pass == 0 && pool_.size_of(c.voff) < req) continue;
+            int rc = evict((CellPtr)i);
+            if (rc) return rc;
+            if (pool_.largest_free() >= req) return 0;
+        }
+    }
+    return CACTI_E_OOM;
+}
+
+int Ctx::pool_alloc(size_t bytes, size_t *off)
+{
+    size_t o = pool_.alloc(bytes);
+    if (o == kNoOffset) {
+        int rc = try_soft_oom(bytes);
+        if (rc == 0) o = pool_.alloc(bytes);
+        if (o == kNoOffset) {
+            set_error("device pool exhausted: request %zu bytes, cap %zu, used %zu, front %zu, "
+                      "largest free %zu (every other cell is pinned by the running thunk)",
+                      bytes, pool_.cap(), pool_.used(), pool_.front(), pool_.largest_free());
+            return CACTI_E_OOM;
+        }
+    }
+    n_alloc_++;
+    *off = o;
+    return 0;
+}
+
+int Ctx::ensure_vmem(CellPtr ci, bool need_value)
+{
+    Cell &c = cells_[ci];
+    CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "use of dead cell %d (%s)", ci, c.name.c_str());
+    if (c.voff == kNoOffset) {
+        size_t off;
+        int rc = pool_alloc(c.ty.bytes(), &off);
+        if (rc) return rc;
+        cells_[ci].voff = off;
+        cells_[ci].v_valid = false;
+    }
+    Cell &d = cells_[ci];
+    if (need_value && !d.v_valid) {
+        CACTI_REQUIRE(d.h_valid, CACTI_E_STATE, "cell %d (%s) is read before it holds a value", ci,
+                      d.name.c_str());
+        CACTI_HIP(hipMemcpyAsync(dev_ptr(d.voff), d.hptr, d.ty.bytes(), hipMemcpyHostToDevice,
+                                 stream_));
+        d.v_valid = true;
+        n_upload_++;
+        bytes_h2d_ += d.ty.bytes();
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// staging
+
+void Ctx::reset()
+{
+    for (size_t i = 1; i < cells_.size(); i++) {
+        Cell &c = cells_[i];
+        if (c.alive && !c.stable) {
+            cell_free_all((CellPtr)i);
+            c.alive = false;
+        }
+    }
+    // compact trailing dead cells so ids do not grow without bound across cycles
+    while (cells_.size() > 1 && !cells_.back().alive) cells_.pop_back();
+    log_.clear();
+    thunks_.clear();
+    kept_.clear();
+    adj_.clear();
+    adj_wr_.clear();
+    pc_ = 0;
+    compiled_ = false;
+    fwd_end_ = 0;
+}
+
+int Ctx::add_thunk(std::unique_ptr<ThunkSpec> spec)
+{
+    thunks_.push_back(std::move(spec));
+    return (int)thunks_.size() - 1;
+}
+
+int Ctx::stage_apply(int thunk, const std::vector<CellPtr> &args, std::vector<CellPtr> *outs)
+{
+    const ThunkSpec &sp = *thunks_[thunk];
+    CACTI_REQUIRE((int)args.size() == sp.arity(), CACTI_E_INVALID, "%s: %zu args, arity %d",
+                  sp.name(), args.size(), sp.arity());
+    std::vector<CellType> aty, oty;
+    for (CellPtr a : args) {
+        CACTI_REQUIRE(a > 0 && (size_t)a < cells_.size() && cells_[a].alive, CACTI_E_INVALID,
+                      "%s: dead or nil argument cell", sp.name());
+        aty.push_back(cells_[a].ty);
+    }
+    int rc = sp.out_ty(aty, oty);
+    if (rc) return rc;
+    Entry e;
+    e.kind = E_APPLY;
+    e.thunk = thunk;
+    e.args = args;
+    for (auto &t : oty) e.outs.push_back(cell_new(t, false, sp.name()));
+    if (outs) *outs = e.outs;
+    log_.push_back(std::move(e));
+    return 0;
+}
+
+int Ctx::stage_into(int thunk, const std::vector<CellPtr> &args, const std::vector<CellPtr> &outs,
+                    uint32_t acc_mask)
+{
+    const ThunkSpec &sp = *thunks_[thunk];
+    std::vector<CellType> aty, oty;
+    for (CellPtr a : args) aty.push_back(cells_[a].ty);
+    int rc = sp.out_ty(aty, oty);
+    if (rc) return rc;
+    CACTI_REQUIRE(oty.size() == outs.size(), CACTI_E_INVALID, "%s: output count mismatch", sp.name());
+    for (size_t k = 0; k < outs.size(); k++)
+        CACTI_REQUIRE(cells_[outs[k]].ty == oty[k], CACTI_E_INVALID,
+                      "%s: output %zu type differs from the target cell %s", sp.name(), k,
+                      cells_[outs[k]].name.c_str());
+    Entry e;
+    e.kind = E_APPLY;
+    e.thunk = thunk;
+    e.args = args;
+    e.outs = outs;
+    e.acc_mask = acc_mask;
+    log_.push_back(std::move(e));
+    return 0;
+}
+
+void Ctx::stage_yield_set(CellPtr c)
+{
+    Entry e;
+    e.kind = E_YIELD_SET;
+    e.cell = c;
+    log_.push_back(std::move(e));
+}
+
+void Ctx::adj_seed(CellPtr primal, CellPtr adj)
+{
+    adj_[primal] = adj;
+    adj_wr_[adj] = true;
+}
+
+void Ctx::adj_bind(CellPtr primal, CellPtr adj)
+{
+    adj_[primal] = adj;
+    adj_wr_[adj] = false;
+}
+
+CellPtr Ctx::adj_of(CellPtr primal)
+{
+    if (cells_[primal].konst) return 0;
+    auto it = adj_.find(primal);
+    if (it != adj_.end()) return it->second;
+    CellPtr a = cell_new(cells_[primal].ty, false, ("d:" + cells_[primal].name).c_str());
+    adj_[primal] = a;
+    adj_wr_[a] = false;
+    return a;
+}
+
+bool Ctx::adj_written(CellPtr primal)
+{
+    auto it = adj_.find(primal);
+    return it != adj_.end() && adj_wr_[it->second];
+}
+
+int Ctx::adj_add(const std::vector<CellPtr> &primals, std::unique_ptr<ThunkSpec> spec,
+                 const std::vector<CellPtr> &args)
+{
+    std::vector<CellPtr> outs;
+    uint32_t mask = 0;
+    bool any = false;
+    for (size_t k = 0; k < primals.size(); k++) {
+        CellPtr a = adj_of(primals[k]);
+        if (a == 0) {
+            // no adjoint wanted for this argument: the fused thunk still needs a target
+            a = cell_new(cells_[primals[k]].ty, false, "d:unused");
+        } else {
+            any = true;
+            if (adj_wr_[a]) mask |= 1u << k;
+            adj_wr_[a] = true;
+        }
+        outs.push_back(a);
+    }
+    if (!any) return 0;
+    int t = add_thunk(std::move(spec));
+    return stage_into(t, args, outs, mask);
+}
+
+int Ctx::vadd_vjp()
+{
+    fwd_end_ = log_.size();
+    for (size_t i = fwd_end_; i-- > 0;) {
+        if (log_[i].kind != E_APPLY) continue;
+        const Entry e = log_[i];                 // copy: pop_adj appends to the log
+        std::vector<CellPtr> out_adj(e.outs.size(), 0);
+        bool any = false;
+        for (size_t k = 0; k < e.outs.size(); k++) {
+            auto it = adj_.find(e.outs[k]);
+            if (it != adj_.end() && adj_wr_[it->second]) {
+                out_adj[k] = it->second;
+                any = true;
+            }
+        }
+        if (!any) continue;
+        int rc = thunks_[e.thunk]->pop_adj(*this, e, out_adj);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+// Liveness: a non-stable, non-kept cell dies after its last use; an Unlive entry frees it
+// there (Spine::_compile splices Live/Unlive, src/spine.rs:1435-1478).
+int Ctx::compile()
+{
+    std::unordered_map<CellPtr, size_t> last;
+    for (size_t i = 0; i < log_.size(); i++) {
+        const Entry &e = log_[i];
+        if (e.kind == E_APPLY) {
+            for (CellPtr a : e.args) last[a] = i;
+            for (CellPtr o : e.outs) last[o] = i;
+        } else if (e.kind == E_YIELD_SET) {
+            last[e.cell] = i;
+        }
+    }
+    for (CellPtr k : kept_) last.erase(k);
+    std::vector<std::vector<CellPtr>> dies(log_.size());
+    for (auto &kv : last)
+        if (!cells_[kv.first].stable) dies[kv.second].push_back(kv.first);
+    std::vector<Entry> out;
+    out.reserve(log_.size() * 2);
+    for (size_t i = 0; i < log_.size(); i++) {
+        out.push_back(std::move(log_[i]));
+        std::sort(dies[i].begin(), dies[i].end());
+        for (CellPtr c : dies[i]) {
+            Entry u;
+            u.kind = E_UNLIVE;
+            u.cell = c;
+            out.push_back(std::move(u));
+        }
+    }
+    log_.swap(out);
+    compiled_ = true;
+    pc_ = 0;
+    return 0;
+}
+
+const char *Ctx::entry_name(size_t i) const
+{
+    const Entry &e = log_[i];
+    if (e.kind == E_APPLY) return thunks_[e.thunk]->name();
+    return e.kind == E_YIELD_SET ? "yield_set" : "unlive";
+}
+
+int Ctx::run_entry(const Entry &e)
+{
+    const ThunkSpec &sp = *thunks_[e.thunk];
+    std::vector<CellType> aty, oty;
+    for (CellPtr a : e.args) cells_[a].pin++;
+    for (CellPtr o : e.outs) cells_[o].pin++;
+    int rc = 0;
+    std::vector<void *> ap, op;
+    for (CellPtr a : e.args) {
+        if ((rc = ensure_vmem(a, true))) break;
+        aty.push_back(cells_[a].ty);
+    }
+    for (size_t k = 0; !rc && k < e.outs.size(); k++) {
+        if ((rc = ensure_vmem(e.outs[k], (e.acc_mask >> k) & 1))) break;
+        oty.push_back(cells_[e.outs[k]].ty);
+    }
+    size_t ws_off = kNoOffset, ws_bytes = 0;
+    if (!rc) {
+        ws_bytes = sp.workspace(aty);
+        if (ws_bytes) rc = pool_alloc(ws_bytes, &ws_off);
+    }
+    if (!rc) {
+        // resolve pointers only now: eviction during allocation cannot move pinned cells
+        for (CellPtr a : e.args) ap.push_back(dev_ptr(cells_[a].voff));
+        for (CellPtr o : e.outs) op.push_back(dev_ptr(cells_[o].voff));
+        if (timing_) hipEventRecord(ev0_, stream_);
+        rc = sp.run(*this, aty, ap.data(), oty, op.data(), e.acc_mask,
+                    ws_off == kNoOffset ? nullptr : dev_ptr(ws_off), ws_bytes);
+        if (timing_ && !rc) {
+            hipEventRecord(ev1_, stream_);
+            hipEventSynchronize(ev1_);
+            float ms = 0;
+            hipEventElapsedTime(&ms, ev0_, ev1_);
+            auto &t = times_[sp.name()];
+            t.first += ms;
+            t.second++;
+        }
+        n_run_++;
+    }
+    if (ws_off != kNoOffset) pool_.free(ws_off);      // reuse is ordered on the stream
+    if (!rc)
+        for (CellPtr o : e.outs) {
+            cells_[o].v_valid = true;
+            cells_[o].h_valid = false;
+        }
+    for (CellPtr a : e.args) cells_[a].pin--;
+    for (CellPtr o : e.outs) cells_[o].pin--;
+    return rc;
+}
+
+int Ctx::resume(CellPtr *yield_cell)
+{
+    CACTI_REQUIRE(compiled_, CACTI_E_STATE, "resume before compile");
+    while (pc_ < log_.size()) {
+        const Entry &e = log_[pc_];
+        if (e.kind == E_YIELD_SET) {
+            if (yield_cell) *yield_cell = e.cell;
+            return R_YIELD;                           // pc_ advances in resume_put
+        }
+        if (e.kind == E_UNLIVE) {
+            cell_free_all(e.cell);
+            cells_[e.cell].alive = false;
+        } else {
+            int rc = run_entry(e);
+            if (rc) return rc < 0 ? rc : -1000 - rc;  // keep 0/1 for DONE/YIELD
+        }
+        pc_++;
+    }
+    return R_DONE;
+}
+
+int Ctx::resume_put(CellPtr c, const void *host, size_t bytes)
+{
+    CACTI_REQUIRE(pc_ < log_.size() && log_[pc_].kind == E_YIELD_SET && log_[pc_].cell == c,
+                  CACTI_E_STATE, "resume_put: the spine is not waiting for cell %d", c);
+    int rc = cell_put(c, host, bytes);
+    if (rc) return rc;
+    pc_++;
+    return 0;
+}
+
+void Ctx::stats(Stats *s) const
+{
+    s->pool_cap = pool_.cap();
+    s->pool_used = pool_.used();
+    s->pool_peak = pool_.peak();
+    s->pool_front = pool_.front();
+    s->n_alloc = n_alloc_;
+    s->n_evict = n_evict_;
+    s->n_upload = n_upload_;
+    s->bytes_d2h = bytes_d2h_;
+    s->bytes_h2d = bytes_h2d_;
+    s->n_soft_oom = n_soft_oom_;
+    s->n_entries = log_.size();
+    s->n_thunks_run = n_run_;
+    s->host_bytes = host_bytes_;
+}
+
+}  // namespace cacti

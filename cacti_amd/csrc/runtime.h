@@ -1,0 +1,203 @@
+// Host runtime behind the C ABI: device context with a pooled allocator and host spill,
+// cells with VMem / Mem replicas, the thunk interface, and the spine (staged instruction
+// log, reverse-mode AD, liveness, interpreter).
+//
+// It mirrors the reference's structure for this path -- PCtx / NvGpuMemPool / PCell
+// (src/pctx/nvgpu.rs, src/cell/mod.rs:2245-2669), ThunkSpec / ThunkImpl
+// (src/thunk/mod.rs:257-351), Spine (src/spine.rs) -- at the granularity of the fused
+// thunks, with one in-order HIP stream and no per-thunk stream syncs.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <map>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace cacti {
+
+enum Dtype : int { F16 = 0, F32 = 1, U16 = 2, I32 = 3 };
+inline size_t dtype_size(Dtype d) { return d == F16 || d == U16 ? 2 : 4; }
+
+struct CellType {
+    std::vector<int64_t> shape;
+    Dtype dtype = F16;
+    CellType() {}
+    CellType(std::vector<int64_t> s, Dtype d) : shape(std::move(s)), dtype(d) {}
+    int64_t numel() const
+    {
+        int64_t n = 1;
+        for (int64_t v : shape) n *= v;
+        return n;
+    }
+    size_t bytes() const { return (size_t)numel() * dtype_size(dtype); }
+    bool operator==(const CellType &o) const { return dtype == o.dtype && shape == o.shape; }
+};
+
+typedef int32_t CellPtr;                 // 0 = nil
+constexpr size_t kNoOffset = ~(size_t)0;
+constexpr size_t kAllocAlign = 256;      // src/pctx/nvgpu.rs:30
+
+// ---------------------------------------------------------------------------
+// MemPool: offset arithmetic over one reserved region (no HIP calls, so the policy is
+// testable on a CPU).  First fit over the coalesced free-region set, else bump the
+// front cursor (src/pctx/nvgpu.rs:1633-1655); freeing the last region retracts it.
+class MemPool {
+   public:
+    explicit MemPool(size_t cap = 0) : cap_(cap) {}
+    void reset(size_t cap);
+    size_t alloc(size_t bytes);          // offset, or kNoOffset when it does not fit
+    void free(size_t off);
+    size_t size_of(size_t off) const;
+    size_t cap() const { return cap_; }
+    size_t used() const { return used_; }
+    size_t peak() const { return peak_; }
+    size_t front() const { return front_; }
+    size_t largest_free() const;         // largest request that would succeed now
+    size_t num_allocs() const { return alloc_.size(); }
+
+   private:
+    size_t cap_ = 0, front_ = 0, used_ = 0, peak_ = 0;
+    std::map<size_t, size_t> free_;                  // offset -> size, coalesced
+    std::unordered_map<size_t, size_t> alloc_;       // offset -> size
+};
+
+// ---------------------------------------------------------------------------
+struct Cell {
+    CellType ty;
+    std::string name;
+    bool stable = false;     // survives reset() (parameters, gradients, constants)
+    bool konst = false;      // no adjoint is generated for it (src/spine.rs:495-498)
+    bool alive = true;
+    size_t voff = kNoOffset; // VMem replica: offset into the pool
+    void *hptr = nullptr;    // Mem replica (host)
+    bool v_valid = false, h_valid = false;
+    int pin = 0;
+};
+
+struct Stats {
+    uint64_t pool_cap, pool_used, pool_peak, pool_front;
+    uint64_t n_alloc, n_evict, n_upload, bytes_d2h, bytes_h2d, n_soft_oom;
+    uint64_t n_entries, n_thunks_run, host_bytes;
+};
+
+class Ctx;
+struct Entry;
+
+// ThunkSpec + ThunkImpl in one object: type inference, execution (`run` covers both
+// apply and accumulate: bit k of acc_mask says output k already holds a value), and the
+// adjoint rule (pop_adj stages further thunks).  src/thunk/mod.rs:257-351.
+struct ThunkSpec {
+    virtual ~ThunkSpec() {}
+    virtual const char *name() const = 0;
+    virtual int arity() const = 0;
+    virtual int nout() const { return 1; }
+    virtual int out_ty(const std::vector<CellType> &arg, std::vector<CellType> &out) const = 0;
+    virtual size_t workspace(const std::vector<CellType> &) const { return 0; }
+    virtual int run(Ctx &ctx, const std::vector<CellType> &aty, void *const *a,
+                    const std::vector<CellType> &oty, void *const *o, uint32_t acc_mask,
+                    void *ws, size_t ws_bytes) const = 0;
+    // out_adj[k] = adjoint cell of output k or 0; stage contributions through ctx.adj_*
+    virtual int pop_adj(Ctx &, const Entry &, const std::vector<CellPtr> &) const { return 0; }
+};
+
+enum EntryKind : int { E_APPLY = 0, E_YIELD_SET = 1, E_UNLIVE = 2 };
+
+struct Entry {
+    EntryKind kind = E_APPLY;
+    int thunk = -1;
+    std::vector<CellPtr> args, outs;
+    uint32_t acc_mask = 0;
+    CellPtr cell = 0;        // E_YIELD_SET / E_UNLIVE
+};
+
+enum ResumeStatus : int { R_DONE = 0, R_YIELD = 1 };
+
+class Ctx {
+   public:
+    Ctx();
+    ~Ctx();
+    int init(int dev, size_t pool_bytes, int host_pagelocked);
+
+    // ---- cells
+    CellPtr cell_new(const CellType &ty, bool stable, const char *name = "");
+    Cell &cell(CellPtr c) { return cells_[c]; }
+    void set_const(CellPtr c) { cells_[c].konst = true; }
+    int cell_put(CellPtr c, const void *host, size_t bytes);     // host -> cell (Mem, then VMem)
+    int cell_get(CellPtr c, void *host, size_t bytes);           // cell -> host (syncs)
+    int cell_free_all(CellPtr c);
+    void *dev_ptr(size_t off) { return base_ + off; }
+    // make the VMem replica exist (evicting others if needed) and, if `need_value`, hold
+    // the current version (uploading from the host replica)
+    int ensure_vmem(CellPtr c, bool need_value);
+    int pool_alloc(size_t bytes, size_t *off);                   // with soft-OOM eviction
+    int try_soft_oom(size_t need);
+    int evict(CellPtr c);                                        // VMem -> Mem, drop VMem
+
+    // ---- staging (control thread side of the spine)
+    void reset();                                                // src/ctx.rs:150-235
+    int add_thunk(std::unique_ptr<ThunkSpec> spec);
+    int stage_apply(int thunk, const std::vector<CellPtr> &args, std::vector<CellPtr> *outs);
+    int stage_into(int thunk, const std::vector<CellPtr> &args, const std::vector<CellPtr> &outs,
+                   uint32_t acc_mask);
+    void stage_yield_set(CellPtr c);
+    void keep(CellPtr c) { kept_.push_back(c); }
+    // reverse-mode AD: src/spine.rs:447-690 (CellMap::vadd_vjp, src/op.rs:2386-2393)
+    void adj_seed(CellPtr primal, CellPtr adj);                  // sink.add(y, dy)
+    void adj_bind(CellPtr primal, CellPtr adj);                  // grad_map.add(p, g)
+    CellPtr adj_of(CellPtr primal);                              // 0 for const cells
+    bool adj_written(CellPtr primal);
+    // arg_adj[..] += thunk(args): Apply on first write, Accumulate afterwards (src/op.rs:20-188)
+    int adj_add(const std::vector<CellPtr> &primals, std::unique_ptr<ThunkSpec> spec,
+                const std::vector<CellPtr> &args);
+    int vadd_vjp();
+    int compile();                                               // liveness, src/spine.rs:1435-1478
+    int resume(CellPtr *yield_cell);                             // src/spine.rs:1484-1991
+    int resume_put(CellPtr c, const void *host, size_t bytes);
+
+    hipStream_t stream() const { return stream_; }
+    int sync();
+    // device word that kernels raise when a token / key id is out of range (the
+    // reference asserts inside the kernel, src/thunk/op.rs:3538); checked at sync points
+    void *status_ptr() { return base_ + status_off_; }
+    int check_status();
+    void stats(Stats *s) const;
+    const std::vector<Entry> &log() const { return log_; }
+    const ThunkSpec &thunk(int i) const { return *thunks_[i]; }
+    const char *entry_name(size_t i) const;
+    void set_timing(bool on) { timing_ = on; }
+    const std::map<std::string, std::pair<double, uint64_t>> &timings() const { return times_; }
+
+   private:
+    int run_entry(const Entry &e);
+    int host_alloc(Cell &c);
+    void host_free(Cell &c);
+
+    int dev_ = 0;
+    hipStream_t stream_ = nullptr;
+    bool own_stream_ = false;
+    char *base_ = nullptr;
+    size_t status_off_ = 0;
+    MemPool pool_;
+    int host_pagelocked_ = 1;
+    std::vector<Cell> cells_;
+    std::vector<std::unique_ptr<ThunkSpec>> thunks_;
+    std::vector<Entry> log_;
+    std::vector<CellPtr> kept_;
+    size_t pc_ = 0;
+    bool compiled_ = false;
+    size_t fwd_end_ = 0;
+    std::unordered_map<CellPtr, CellPtr> adj_;       // primal -> adjoint cell
+    std::unordered_map<CellPtr, bool> adj_wr_;       // adjoint already written in the log
+    std::vector<CellPtr> pending_yield_;
+    // statistics
+    uint64_t n_alloc_ = 0, n_evict_ = 0, n_upload_ = 0, bytes_d2h_ = 0, bytes_h2d_ = 0,
+             n_soft_oom_ = 0, n_run_ = 0, host_bytes_ = 0;
+    bool timing_ = false;
+    std::map<std::string, std::pair<double, uint64_t>> times_;
+    hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
+};
+
+}  // namespace cacti

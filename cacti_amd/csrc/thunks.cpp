@@ -1,0 +1,455 @@
+#include "thunks.h"
+
+#include "common.h"
+
+namespace cacti {
+namespace {
+
+inline void *S(Ctx &c) { return (void *)c.stream(); }
+
+#define TY_REQUIRE(cond, ...) CACTI_REQUIRE(cond, CACTI_E_INVALID, __VA_ARGS__)
+
+// ---------------------------------------------------------------------------
+// copy (the memcpy adjoint of Add / Identity, src/thunk/op.rs:1529-1534, 5474-5729)
+struct CopySpec : ThunkSpec {
+    const char *name() const override { return "copy"; }
+    int arity() const override { return 1; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        if (acc & 1) {
+            TY_REQUIRE(aty[0].dtype == F16, "copy: accumulate is f16 only");
+            return cacti_hip_add_f16(aty[0].numel(), o[0], a[0], o[0], S(c));
+        }
+        return cacti_hip_memcpy_async(o[0], a[0], aty[0].bytes(), S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        return c.adj_add({e.args[0]}, make_copy(), {dy[0]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// y = a + b (AddFutThunkSpec src/thunk/op.rs:1480-1535); both adjoints are copies of dy
+struct AddSpec : ThunkSpec {
+    const char *name() const override { return "add"; }
+    int arity() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[1] && a[0].dtype == F16, "add: operands must be equal f16 shapes");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        TY_REQUIRE(!(acc & 1), "add: accumulate mode not staged on this path");
+        return cacti_hip_add_f16(aty[0].numel(), a[0], a[1], o[0], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        int rc = c.adj_add({e.args[0]}, make_copy(), {dy[0]});
+        if (rc) return rc;
+        return c.adj_add({e.args[1]}, make_copy(), {dy[0]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// Embedding (OuterSelectFutThunkSpec src/thunk/op.rs:1229-1314) and its scatter-add adjoint
+struct EmbedBwdSpec : ThunkSpec {
+    int64_t V;
+    explicit EmbedBwdSpec(int64_t v) : V(v) {}
+    const char *name() const override { return "embed_bwd"; }
+    int arity() const override { return 2; }                       // (tok, dy) -> dW
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == U16 && a[1].dtype == F16 && a[1].shape.size() == 2,
+                   "embed_bwd: (tok u16, dy f16 [S,D]) expected");
+        o = {CellType({V, a[1].shape[1]}, F16)};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        return cacti_hip_embed_bwd(V, aty[1].shape[1], aty[1].shape[0], a[0], a[1], o[0], acc & 1,
+                                   S(c));
+    }
+};
+
+struct EmbedSpec : ThunkSpec {
+    const char *name() const override { return "embed"; }
+    int arity() const override { return 2; }                       // (W, tok) -> y
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[1].dtype == U16,
+                   "embed: (W f16 [V,D], tok u16) expected");
+        o = {CellType({a[1].numel(), a[0].shape[1]}, F16)};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        return cacti_hip_embed_fwd(aty[0].shape[0], aty[0].shape[1], a[0], aty[1].numel(), a[1],
+                                   o[0], c.status_ptr(), S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        const int64_t V = c.cell(e.args[0]).ty.shape[0];
+        return c.adj_add({e.args[0]}, std::unique_ptr<ThunkSpec>(new EmbedBwdSpec(V)),
+                         {e.args[1], dy[0]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// RMSNorm (rms_norm closure src/librarium/llama.rs:442-451) and its fused adjoint
+struct RmsNormBwdSpec : ThunkSpec {
+    float eps;
+    explicit RmsNormBwdSpec(float e) : eps(e) {}
+    const char *name() const override { return "rms_norm_bwd"; }
+    int arity() const override { return 3; }                       // (x, w, dy) -> dx, dw
+    int nout() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[2] && a[0].shape.size() == 2 && a[1].numel() == a[0].shape[1],
+                   "rms_norm_bwd: shape mismatch");
+        o = {a[0], a[1]};
+        return 0;
+    }
+    size_t workspace(const std::vector<CellType> &a) const override
+    {
+        return cacti_hip_rms_norm_bwd_workspace(a[0].shape[0], a[0].shape[1]);
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *ws, size_t wsb) const override
+    {
+        return cacti_hip_rms_norm_bwd(aty[0].shape[0], aty[0].shape[1], a[0], a[1], eps, a[2], o[0],
+                                      acc & 1, o[1], (acc >> 1) & 1, ws, wsb, S(c));
+    }
+};
+
+struct RmsNormSpec : ThunkSpec {
+    float eps;
+    explicit RmsNormSpec(float e) : eps(e) {}
+    const char *name() const override { return "rms_norm"; }
+    int arity() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[1].dtype == F16 && a[0].shape.size() == 2 &&
+                       a[1].numel() == a[0].shape[1],
+                   "rms_norm: (x f16 [N,D], w f16 [D]) expected");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        return cacti_hip_rms_norm_fwd(aty[0].shape[0], aty[0].shape[1], a[0], a[1], eps, o[0], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        return c.adj_add({e.args[0], e.args[1]}, std::unique_ptr<ThunkSpec>(new RmsNormBwdSpec(eps)),
+                         {e.args[0], e.args[1], dy[0]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// MatrixMulThunkSpec src/thunk/op.rs:4284-4368 (2-d) and BlockMatrixMulThunkSpec :4719-4918
+// on [R, H*C] tensors (the reference's [B,S,H,C] with B = 1, flattened) whose H per-head
+// blocks are addressed by stride; H = 0 means one plain matrix.
+struct MatMulSpec : ThunkSpec {
+    bool ta, tb;
+    int64_t nblk;
+    bool blocked;
+    float alpha;
+    MatMulSpec(bool a, bool b, float al, int64_t h) : ta(a), tb(b), nblk(h), blocked(h > 0), alpha(al) {}
+    const char *name() const override { return blocked ? "block_matmul" : "matmul"; }
+    int arity() const override { return 2; }
+    struct Dims { int64_t H, M, N, K, lda, sa, ldb, sb, ldc, sc; };
+    int dims(const std::vector<CellType> &a, Dims &d) const
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[1].dtype == F16 && a[0].shape.size() == 2 &&
+                       a[1].shape.size() == 2,
+                   "%s: f16 operands of rank 2 expected", name());
+        d.H = blocked ? nblk : 1;
+        TY_REQUIRE(a[0].shape[1] % d.H == 0 && a[1].shape[1] % d.H == 0,
+                   "block_matmul: row length not divisible by the block count");
+        const int64_t ra = a[0].shape[0], ca = a[0].shape[1] / d.H;
+        const int64_t rb = a[1].shape[0], cb = a[1].shape[1] / d.H;
+        d.M = ta ? ca : ra;
+        d.K = ta ? ra : ca;
+        const int64_t kb = tb ? cb : rb;
+        d.N = tb ? rb : cb;
+        TY_REQUIRE(kb == d.K, "%s: inner dimensions %lld and %lld differ", name(), (long long)d.K,
+                   (long long)kb);
+        d.lda = d.H * ca; d.sa = ca;
+        d.ldb = d.H * cb; d.sb = cb;
+        d.ldc = d.H * d.N; d.sc = d.N;
+        return 0;
+    }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        Dims d;
+        int rc = dims(a, d);
+        if (rc) return rc;
+        o = {CellType({d.M, d.H * d.N}, F16)};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        Dims d;
+        int rc = dims(aty, d);
+        if (rc) return rc;
+        return cacti_hip_gemm_f16_strided_batched(ta, tb, d.H, d.M, d.N, d.K, alpha, a[0], d.lda,
+                                                  d.sa, a[1], d.ldb, d.sb, (acc & 1) ? 1.f : 0.f,
+                                                  o[0], d.ldc, d.sc, S(c));
+    }
+    std::unique_ptr<ThunkSpec> mm(bool x, bool y) const
+    {
+        return std::unique_ptr<ThunkSpec>(new MatMulSpec(x, y, alpha, nblk));
+    }
+    // the four transposition cases of pop_adj, src/thunk/op.rs:4335-4367 / :4882-4912:
+    // arg_adj[1] first, then arg_adj[0], both carrying o_scale
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        const CellPtr A = e.args[0], B = e.args[1], G = dy[0];
+        int rc;
+        if (!ta && !tb) {
+            if ((rc = c.adj_add({B}, mm(true, false), {A, G}))) return rc;      // A^T G
+            return c.adj_add({A}, mm(false, true), {G, B});                      // G B^T
+        }
+        if (!ta && tb) {
+            if ((rc = c.adj_add({B}, mm(true, false), {G, A}))) return rc;      // G^T A
+            return c.adj_add({A}, mm(false, false), {G, B});                     // G B
+        }
+        if (ta && !tb) {
+            if ((rc = c.adj_add({B}, mm(false, false), {A, G}))) return rc;     // A G
+            return c.adj_add({A}, mm(false, true), {B, G});                      // B G^T
+        }
+        if ((rc = c.adj_add({B}, mm(true, true), {G, A}))) return rc;           // G^T A^T
+        return c.adj_add({A}, mm(true, true), {B, G});                           // B^T G^T
+    }
+};
+
+// ---------------------------------------------------------------------------
+// RoPE (symplectic_embed src/librarium/llama.rs:463-465); cos/sin are const_ cells
+// x is [S, H*Dh] (the reference's [1,S,H,Dh] flattened); the head count rides in the spec.
+struct RopeBwdSpec : ThunkSpec {
+    int64_t H;
+    explicit RopeBwdSpec(int64_t h) : H(h) {}
+    const char *name() const override { return "rope_bwd"; }
+    int arity() const override { return 3; }                       // (dy, cos, sin) -> dx
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] % H == 0,
+                   "rope_bwd: dy f16 [S,H*Dh] expected");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        const auto &s = aty[0].shape;
+        return cacti_hip_rope_bwd(s[0], H, s[1] / H, a[0], a[1], a[2], o[0], acc & 1, S(c));
+    }
+};
+
+struct RopeSpec : ThunkSpec {
+    int64_t H;
+    explicit RopeSpec(int64_t h) : H(h) {}
+    const char *name() const override { return "rope"; }
+    int arity() const override { return 3; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] % H == 0 &&
+                       a[1].shape.size() == 2 && a[1].shape[0] >= a[0].shape[0] &&
+                       a[1].shape[1] == a[0].shape[1] / H && a[1] == a[2],
+                   "rope: (x f16 [S,H*Dh], cos [S,Dh], sin [S,Dh]) expected");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        const auto &s = aty[0].shape;
+        return cacti_hip_rope_fwd(s[0], H, s[1] / H, a[0], a[1], a[2], o[0], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        return c.adj_add({e.args[0]}, std::unique_ptr<ThunkSpec>(new RopeBwdSpec(H)),
+                         {dy[0], e.args[1], e.args[2]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// causal softmax over scores (src/librarium/llama.rs:501-505)
+struct CausalSoftmaxBwdSpec : ThunkSpec {
+    int64_t H;
+    explicit CausalSoftmaxBwdSpec(int64_t h) : H(h) {}
+    const char *name() const override { return "causal_softmax_bwd"; }
+    int arity() const override { return 2; }                       // (s16, dp16) -> ds16
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[1], "causal_softmax_bwd: shape mismatch");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        TY_REQUIRE(!(acc & 1), "causal_softmax_bwd: accumulate mode not staged on this path");
+        return cacti_hip_causal_softmax_bwd(aty[0].shape[0], H, a[0], a[1], o[0], S(c));
+    }
+};
+
+struct CausalSoftmaxSpec : ThunkSpec {
+    int64_t H;
+    explicit CausalSoftmaxSpec(int64_t h) : H(h) {}
+    const char *name() const override { return "causal_softmax"; }
+    int arity() const override { return 1; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] == H * a[0].shape[0],
+                   "causal_softmax: s16 f16 [S,H*S] expected");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        return cacti_hip_causal_softmax_fwd(aty[0].shape[0], H, a[0], o[0], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        return c.adj_add({e.args[0]}, std::unique_ptr<ThunkSpec>(new CausalSoftmaxBwdSpec(H)),
+                         {e.args[0], dy[0]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// SiLU gate (src/librarium/llama.rs:526-527)
+struct SiluGateBwdSpec : ThunkSpec {
+    const char *name() const override { return "silu_gate_bwd"; }
+    int arity() const override { return 3; }                       // (g, u, dh) -> dg, du
+    int nout() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[1] && a[0] == a[2], "silu_gate_bwd: shape mismatch");
+        o = {a[0], a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        return cacti_hip_silu_gate_bwd(aty[0].numel(), a[0], a[1], a[2], o[0], acc & 1, o[1],
+                                       (acc >> 1) & 1, S(c));
+    }
+};
+
+struct SiluGateSpec : ThunkSpec {
+    const char *name() const override { return "silu_gate"; }
+    int arity() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[1] && a[0].dtype == F16, "silu_gate: equal f16 shapes expected");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        return cacti_hip_silu_gate_fwd(aty[0].numel(), a[0], a[1], o[0], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        return c.adj_add({e.args[0], e.args[1]}, std::unique_ptr<ThunkSpec>(new SiluGateBwdSpec()),
+                         {e.args[0], e.args[1], dy[0]});
+    }
+};
+
+// ---------------------------------------------------------------------------
+// LM loss (src/librarium/llama.rs:541-546)
+struct SoftmaxCeBwdSpec : ThunkSpec {
+    const char *name() const override { return "softmax_ce_bwd"; }
+    int arity() const override { return 3; }                       // (logit, tok, dloss) -> dlogit
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].shape.size() == 2 && a[2].dtype == F32 && a[2].numel() == a[0].shape[0],
+                   "softmax_ce_bwd: (logit [N,V], tok, dloss f32 [N]) expected");
+        o = {a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        return cacti_hip_softmax_ce_bwd(aty[0].shape[0], aty[0].shape[1], a[0], a[1], a[2], o[0],
+                                        acc & 1, S(c));
+    }
+};
+
+struct SoftmaxCeSpec : ThunkSpec {
+    bool want_prob;
+    explicit SoftmaxCeSpec(bool p) : want_prob(p) {}
+    const char *name() const override { return "softmax_ce"; }
+    int arity() const override { return 2; }
+    int nout() const override { return want_prob ? 3 : 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[1].dtype == U16 &&
+                       a[1].numel() == a[0].shape[0],
+                   "softmax_ce: (logit f16 [N,V], tok u16 [N]) expected");
+        o = {CellType({a[0].shape[0]}, F32), CellType({a[0].shape[0]}, U16)};
+        if (want_prob) o.push_back(CellType(a[0].shape, F32));
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        return cacti_hip_softmax_ce_fwd(aty[0].shape[0], aty[0].shape[1], a[0], a[1],
+                                        want_prob ? o[2] : nullptr, o[0], o[1], c.status_ptr(), S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        if (!dy[0]) return 0;                    // only the loss output carries a gradient
+        return c.adj_add({e.args[0]}, std::unique_ptr<ThunkSpec>(new SoftmaxCeBwdSpec()),
+                         {e.args[0], e.args[1], dy[0]});
+    }
+};
+
+}  // namespace
+
+std::unique_ptr<ThunkSpec> make_embed() { return std::unique_ptr<ThunkSpec>(new EmbedSpec()); }
+std::unique_ptr<ThunkSpec> make_rms_norm(float eps)
+{
+    return std::unique_ptr<ThunkSpec>(new RmsNormSpec(eps));
+}
+std::unique_ptr<ThunkSpec> make_matmul(bool ta, bool tb, float alpha)
+{
+    return std::unique_ptr<ThunkSpec>(new MatMulSpec(ta, tb, alpha, 0));
+}
+std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int64_t H)
+{
+    return std::unique_ptr<ThunkSpec>(new MatMulSpec(ta, tb, alpha, H));
+}
+std::unique_ptr<ThunkSpec> make_rope(int64_t H) { return std::unique_ptr<ThunkSpec>(new RopeSpec(H)); }
+std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H)
+{
+    return std::unique_ptr<ThunkSpec>(new CausalSoftmaxSpec(H));
+}
+std::unique_ptr<ThunkSpec> make_add() { return std::unique_ptr<ThunkSpec>(new AddSpec()); }
+std::unique_ptr<ThunkSpec> make_copy() { return std::unique_ptr<ThunkSpec>(new CopySpec()); }
+std::unique_ptr<ThunkSpec> make_silu_gate()
+{
+    return std::unique_ptr<ThunkSpec>(new SiluGateSpec());
+}
+std::unique_ptr<ThunkSpec> make_softmax_ce(bool want_prob)
+{
+    return std::unique_ptr<ThunkSpec>(new SoftmaxCeSpec(want_prob));
+}
+
+}  // namespace cacti

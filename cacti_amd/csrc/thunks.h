@@ -1,0 +1,21 @@
+// Thunk specs of the LLaMA path: type inference, kernel dispatch through the C ABI, and
+// adjoint rules.  Forward specs stand for the reference's thunk chains
+// (src/librarium/llama.rs:420-548); each pop_adj stages the fused adjoint thunk(s) in the
+// order the reference's AD emits the corresponding contributions (src/spine.rs:447-690).
+#pragma once
+#include "runtime.h"
+
+namespace cacti {
+
+std::unique_ptr<ThunkSpec> make_embed();                              // (W, tok) -> y
+std::unique_ptr<ThunkSpec> make_rms_norm(float eps);                  // (x, w) -> y
+std::unique_ptr<ThunkSpec> make_matmul(bool ta, bool tb, float alpha);   // (a, b) -> c, 2-d
+std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int64_t H);   // [R,H*C]
+std::unique_ptr<ThunkSpec> make_rope(int64_t H);                      // (x [S,H*Dh], cos, sin) -> y
+std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H);            // (s16 [S,H*S]) -> p16
+std::unique_ptr<ThunkSpec> make_add();                                // (a, b) -> y
+std::unique_ptr<ThunkSpec> make_copy();                               // (x) -> y
+std::unique_ptr<ThunkSpec> make_silu_gate();                          // (g, u) -> h
+std::unique_ptr<ThunkSpec> make_softmax_ce(bool want_prob);           // (logit, tok) -> loss, amax[, prob]
+
+}  // namespace cacti

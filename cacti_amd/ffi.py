@@ -64,7 +64,49 @@ SIGNATURES = {
     "cacti_hip_embed_bwd": (ci, [i64, i64, i64, vp, vp, vp, ci, vp]),
     "cacti_hip_add_f16": (ci, [i64, vp, vp, vp, vp]),
     "cacti_hip_selftest_wave_reduce": (ci, [vp, vp]),
+    # ---- runtime (include/cacti_hip_runtime.h)
+    "cacti_ctx_create": (ci, [pvp, ci, sz, ci]),
+    "cacti_ctx_destroy": (ci, [vp]),
+    "cacti_ctx_stats": (ci, [vp, vp]),
+    "cacti_ctx_sync": (ci, [vp]),
+    "cacti_ctx_stream": (vp, [vp]),
+    "cacti_ctx_set_timing": (ci, [vp, ci]),
+    "cacti_ctx_timing_report": (ci, [vp, C.c_char_p, sz]),
+    "cacti_mempool_create": (ci, [pvp, C.c_uint64]),
+    "cacti_mempool_destroy": (ci, [vp]),
+    "cacti_mempool_alloc": (C.c_uint64, [vp, C.c_uint64]),
+    "cacti_mempool_free": (ci, [vp, C.c_uint64]),
+    "cacti_mempool_stats": (ci, [vp, C.POINTER(C.c_uint64)]),
+    "cacti_reset": (ci, [vp]),
+    "cacti_compile": (ci, [vp]),
+    "cacti_resume": (ci, [vp, C.POINTER(ci)]),
+    "cacti_resume_put": (ci, [vp, ci, vp, sz]),
+    "cacti_cell_bytes": (ci, [vp, ci, C.POINTER(sz)]),
+    "cacti_cell_get": (ci, [vp, ci, vp, sz]),
+    "cacti_log_len": (ci, [vp]),
+    "cacti_log_name": (C.c_char_p, [vp, ci]),
+    "cacti_llama_create": (ci, [vp, vp, pvp]),
+    "cacti_llama_destroy": (ci, [vp]),
+    "cacti_llama_num_params": (ci, [vp]),
+    "cacti_llama_param_info": (ci, [vp, ci, C.c_char_p, sz, C.POINTER(i64), C.POINTER(i64),
+                                    C.POINTER(ci), C.POINTER(ci)]),
+    "cacti_llama_param_put": (ci, [vp, ci, vp, sz]),
+    "cacti_llama_grad_get": (ci, [vp, ci, vp, sz]),
+    "cacti_llama_io_cells": (ci, [vp] + [C.POINTER(ci)] * 7),
+    "cacti_llama_stage": (ci, [vp, ci, ci]),
+    "cacti_llama_step": (ci, [vp, vp, vp, vp, ci, ci, vp]),
 }
+
+
+class LlamaCfg(C.Structure):
+    _fields_ = [("S", i64), ("D", i64), ("H", i64), ("Dh", i64), ("F", i64), ("V", i64),
+                ("L", i64), ("eps", f32)]
+
+
+class Stats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "pool_cap", "pool_used", "pool_peak", "pool_front", "n_alloc", "n_evict", "n_upload",
+        "bytes_d2h", "bytes_h2d", "n_soft_oom", "n_entries", "n_thunks_run", "host_bytes")]
 
 _lib = None
 

@@ -1,0 +1,192 @@
+"""Host-side handles for the runtime C ABI (include/cacti_hip_runtime.h): the device
+context with its capped pool and host spill, the spine calls, and the LLaMA step.
+
+Mirrors the reference's control flow (reset / stage / vadd_vjp / compile / resume /
+resume_put, examples/open_llama_3b_train.rs:203-531); arrays cross as numpy.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import ffi
+
+DONE, YIELD = 0, 1
+
+
+class MemPool:
+    """The pool's placement policy over a plain offset range (no GPU involved)."""
+
+    def __init__(self, cap):
+        self._p = C.c_void_p()
+        ffi.call("cacti_mempool_create", C.byref(self._p), cap)
+
+    def alloc(self, nbytes):
+        off = ffi.lib().cacti_mempool_alloc(self._p, nbytes)
+        return None if off == 2 ** 64 - 1 else off
+
+    def free(self, off):
+        ffi.call("cacti_mempool_free", self._p, off)
+
+    def stats(self):
+        out = (C.c_uint64 * 5)()
+        ffi.call("cacti_mempool_stats", self._p, out)
+        return dict(zip(("cap", "used", "peak", "front", "largest_free"), list(out)))
+
+    def __del__(self):
+        if getattr(self, "_p", None):
+            ffi.lib().cacti_mempool_destroy(self._p)
+            self._p = None
+
+
+class Ctx:
+    def __init__(self, dev=0, pool_bytes=0, host_pagelocked=True):
+        self._c = C.c_void_p()
+        ffi.call("cacti_ctx_create", C.byref(self._c), dev, pool_bytes, int(host_pagelocked))
+
+    def close(self):
+        if self._c:
+            ffi.lib().cacti_ctx_destroy(self._c)
+            self._c = None
+
+    def __del__(self):
+        self.close()
+
+    def stats(self):
+        s = ffi.Stats()
+        ffi.call("cacti_ctx_stats", self._c, C.byref(s))
+        return {n: getattr(s, n) for n, _ in ffi.Stats._fields_}
+
+    def sync(self):
+        ffi.call("cacti_ctx_sync", self._c)
+
+    @property
+    def stream(self):
+        return ffi.lib().cacti_ctx_stream(self._c)
+
+    def set_timing(self, on):
+        ffi.call("cacti_ctx_set_timing", self._c, int(on))
+
+    def timing_report(self):
+        buf = C.create_string_buffer(1 << 16)
+        ffi.call("cacti_ctx_timing_report", self._c, buf, len(buf))
+        out = {}
+        for line in buf.value.decode().splitlines():
+            name, cnt, ms = line.split()
+            out[name] = (int(cnt), float(ms))
+        return out
+
+    # ---- spine
+    def reset(self):
+        ffi.call("cacti_reset", self._c)
+
+    def compile(self):
+        ffi.call("cacti_compile", self._c)
+
+    def resume(self):
+        """Returns (DONE, None) or (YIELD, cell)."""
+        y = C.c_int(0)
+        rc = ffi.lib().cacti_resume(self._c, C.byref(y))
+        if rc < 0:
+            ffi.check(rc)
+        return (rc, y.value if rc == YIELD else None)
+
+    def resume_put(self, cell, arr):
+        arr = np.ascontiguousarray(arr)
+        ffi.call("cacti_resume_put", self._c, cell, arr.ctypes.data, arr.nbytes)
+
+    def cell_get(self, cell, dtype, shape):
+        out = np.empty(shape, dtype)
+        ffi.call("cacti_cell_get", self._c, cell, out.ctypes.data, out.nbytes)
+        return out
+
+    def log_names(self):
+        n = ffi.lib().cacti_log_len(self._c)
+        return [ffi.lib().cacti_log_name(self._c, i).decode() for i in range(n)]
+
+
+class Llama:
+    """Llama::{from, apply} + the training cycle (src/librarium/llama.rs:223-548)."""
+
+    def __init__(self, ctx, S, D, H, Dh, F, V, L, eps=1e-6):
+        self.ctx = ctx
+        self.cfg = ffi.LlamaCfg(S, D, H, Dh, F, V, L, eps)
+        self._m = C.c_void_p()
+        ffi.call("cacti_llama_create", ctx._c, C.byref(self.cfg), C.byref(self._m))
+        self.params = []          # (name, shape)
+        for i in range(ffi.lib().cacti_llama_num_params(self._m)):
+            name = C.create_string_buffer(64)
+            r, c = C.c_int64(), C.c_int64()
+            ffi.call("cacti_llama_param_info", self._m, i, name, 64, C.byref(r), C.byref(c), None,
+                     None)
+            shape = (r.value,) if name.value.endswith(b"norm") else (r.value, c.value)
+            self.params.append((name.value.decode(), shape))
+
+    def close(self):
+        if self._m:
+            ffi.lib().cacti_llama_destroy(self._m)
+            self._m = None
+
+    def put_param(self, i, arr):
+        arr = np.ascontiguousarray(arr, dtype=np.float16)
+        assert arr.shape == self.params[i][1], (arr.shape, self.params[i])
+        ffi.call("cacti_llama_param_put", self._m, i, arr.ctypes.data, arr.nbytes)
+
+    def put_params_flat(self, flat):
+        o = 0
+        for i, (_, shp) in enumerate(self.params):
+            n = int(np.prod(shp))
+            self.put_param(i, flat[o:o + n].reshape(shp))
+            o += n
+        assert o == flat.size
+
+    def grad(self, i):
+        out = np.empty(self.params[i][1], np.float16)
+        ffi.call("cacti_llama_grad_get", self._m, i, out.ctypes.data, out.nbytes)
+        return out
+
+    def grads(self):
+        return {name: self.grad(i) for i, (name, _) in enumerate(self.params)}
+
+    def io_cells(self):
+        v = [C.c_int(0) for _ in range(7)]
+        ffi.call("cacti_llama_io_cells", self._m, *[C.byref(x) for x in v])
+        return dict(zip(("tok", "lm_tok", "loss_scale", "logit", "loss", "amax", "prob"),
+                        [x.value for x in v]))
+
+    def stage(self, want_prob=False, want_grad=True):
+        ffi.call("cacti_llama_stage", self._m, int(want_prob), int(want_grad))
+
+    def step(self, tok, lm_tok, loss_scale, want_prob=False, want_grad=True, want_loss=True):
+        """One fwd + loss + bwd cycle; returns the per-position loss (f32 [S]) or None."""
+        tok = np.ascontiguousarray(tok, dtype=np.uint16)
+        lm_tok = np.ascontiguousarray(lm_tok, dtype=np.uint16)
+        loss_scale = np.ascontiguousarray(loss_scale, dtype=np.float32)
+        S = self.cfg.S
+        assert tok.size == S and lm_tok.size == S and loss_scale.size == S
+        loss = np.empty(S, np.float32) if want_loss else None
+        ffi.call("cacti_llama_step", self._m, tok.ctypes.data, lm_tok.ctypes.data,
+                 loss_scale.ctypes.data, int(want_prob), int(want_grad),
+                 loss.ctypes.data if want_loss else None)
+        return loss
+
+    def step_explicit(self, tok, lm_tok, loss_scale, want_prob=False, want_grad=True):
+        """The same cycle driven call by call, as the reference's example drives the spine."""
+        c = self.ctx
+        c.reset()
+        self.stage(want_prob, want_grad)
+        c.compile()
+        io = self.io_cells()
+        feed = {io["tok"]: np.asarray(tok, np.uint16), io["lm_tok"]: np.asarray(lm_tok, np.uint16),
+                io["loss_scale"]: np.asarray(loss_scale, np.float32)}
+        while True:
+            rc, cell = c.resume()
+            if rc == DONE:
+                break
+            c.resume_put(cell, feed[cell])
+        S, V = self.cfg.S, self.cfg.V
+        out = dict(loss=c.cell_get(io["loss"], np.float32, (S,)),
+                   logit=c.cell_get(io["logit"], np.float16, (S, V)),
+                   amax=c.cell_get(io["amax"], np.uint16, (S,)))
+        if want_prob:
+            out["prob"] = c.cell_get(io["prob"], np.float32, (S, V))
+        return out

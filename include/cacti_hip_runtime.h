@@ -1,0 +1,111 @@
+/*
+ * cacti_hip_runtime.h -- C ABI of the host runtime inside libcacti_gpu_hip_ffi.so:
+ * the HIP device context (pooled allocator + host spill), the spine
+ * (reset / compile / resume / resume_put) and the LLaMA step staged on it.
+ *
+ * The kernel-level entry points are in cacti_gpu_hip_ffi.h; this header is the
+ * layer a host program drives, with the reference's control flow:
+ *   reset(); stage...; vadd_vjp; compile(); resume() <-> resume_put(); read outputs
+ * (examples/open_llama_3b_train.rs:203-531).  Status codes as in cacti_gpu_hip_ffi.h.
+ * One thread per context (src/ctx.rs:21-29).
+ */
+#ifndef CACTI_HIP_RUNTIME_H
+#define CACTI_HIP_RUNTIME_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cacti_ctx cacti_ctx;
+typedef struct cacti_llama cacti_llama;
+
+/* LlamaConfig, src/librarium/llama.rs:28-105 (batch ubat_sz = 1, q_group = 1). */
+typedef struct {
+    int64_t S;   /* seq_cap          */
+    int64_t D;   /* num_head*head_dim */
+    int64_t H;   /* num_head         */
+    int64_t Dh;  /* head_dim         */
+    int64_t F;   /* mlp_inner_dim    */
+    int64_t V;   /* tok_dim          */
+    int64_t L;   /* num_layer        */
+    float eps;   /* rms_norm_eps     */
+} cacti_llama_cfg;
+
+typedef struct {
+    uint64_t pool_cap, pool_used, pool_peak, pool_front;
+    uint64_t n_alloc, n_evict, n_upload, bytes_d2h, bytes_h2d, n_soft_oom;
+    uint64_t n_entries, n_thunks_run, host_bytes;
+} cacti_stats;
+
+/* ---- device context: replaces NvGpuPCtx + NvGpuMemPool, src/pctx/nvgpu.rs:163-306,
+ * 1377-2002.  pool_bytes = 0 reserves 90.01 % of the device (src/ctx.rs:43); otherwise the
+ * cap in bytes (the CACTI_VMEM_SOFT_LIMIT analogue, src/pctx/nvgpu.rs:1434-1463).  The pool
+ * is ONE hipMalloc; when it is exhausted live cells are spilled to host memory
+ * (_try_soft_oom, src/pctx/nvgpu.rs:2004-2283) and re-uploaded on their next use.
+ * host_pagelocked: 1 = hipHostMalloc, 0 = malloc (CACTI_NVGPU_MEM_ALLOC, :995-1002). */
+int cacti_ctx_create(cacti_ctx **ctx, int dev, size_t pool_bytes, int host_pagelocked);
+int cacti_ctx_destroy(cacti_ctx *ctx);
+int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out);
+int cacti_ctx_sync(cacti_ctx *ctx);
+void *cacti_ctx_stream(cacti_ctx *ctx);                 /* the hipStream_t all work runs on */
+/* per-thunk wall times (CACTI_DEBUG_TIMING, src/ctx.rs:114-133): on = 1 syncs after every
+ * thunk; the report is text "name count total_ms" per line. */
+int cacti_ctx_set_timing(cacti_ctx *ctx, int on);
+int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap);
+
+/* ---- the pool's placement policy alone, over a plain offset range (no device memory is
+ * touched, so it can be exercised on a host without a GPU): first fit over the coalesced
+ * free regions, else bump the front cursor; 256-byte granules; freeing the last region
+ * retracts the cursor (src/pctx/nvgpu.rs:30, 1633-1655).  alloc returns the offset, or
+ * UINT64_MAX when the request does not fit. */
+typedef struct cacti_mempool cacti_mempool;
+int cacti_mempool_create(cacti_mempool **pool, uint64_t cap);
+int cacti_mempool_destroy(cacti_mempool *pool);
+uint64_t cacti_mempool_alloc(cacti_mempool *pool, uint64_t bytes);
+int cacti_mempool_free(cacti_mempool *pool, uint64_t offset);
+/* out[0..4] = cap, used, peak, front cursor, largest request that fits now */
+int cacti_mempool_stats(cacti_mempool *pool, uint64_t out[5]);
+
+/* ---- spine: src/ctx.rs:326-373, src/spine.rs:1193-1991 */
+int cacti_reset(cacti_ctx *ctx);
+int cacti_compile(cacti_ctx *ctx);
+/* returns 0 = ran to the end, 1 = yielded: *yield_cell must be supplied with
+ * cacti_resume_put before resuming; negative = error */
+int cacti_resume(cacti_ctx *ctx, int *yield_cell);
+int cacti_resume_put(cacti_ctx *ctx, int cell, const void *host, size_t bytes);
+int cacti_cell_bytes(cacti_ctx *ctx, int cell, size_t *bytes);
+int cacti_cell_get(cacti_ctx *ctx, int cell, void *host, size_t bytes);   /* with_mem, src/op.rs:2203 */
+/* number of log entries and the name of entry i ("matmul", "rms_norm_bwd", "unlive", ...) */
+int cacti_log_len(cacti_ctx *ctx);
+const char *cacti_log_name(cacti_ctx *ctx, int i);
+
+/* ---- model: Llama::{from, init_constants, apply}, src/librarium/llama.rs:223-548.
+ * Parameters (3 + 9 L tensors, f16) and their gradients are stable cells; order:
+ * embed, per layer {pre_norm, q, k, v, o, post_norm, gate, up, down}, head_norm, lm_head. */
+int cacti_llama_create(cacti_ctx *ctx, const cacti_llama_cfg *cfg, cacti_llama **model);
+int cacti_llama_destroy(cacti_llama *model);
+int cacti_llama_num_params(cacti_llama *model);
+int cacti_llama_param_info(cacti_llama *model, int i, char *name, size_t name_cap,
+                           int64_t *rows, int64_t *cols, int *param_cell, int *grad_cell);
+int cacti_llama_param_put(cacti_llama *model, int i, const void *host, size_t bytes);
+int cacti_llama_grad_get(cacti_llama *model, int i, void *host, size_t bytes);
+/* cells of the inputs (tok u16 [S], lm_tok u16 [S], loss_scale f32 [S]) and of the kept
+ * outputs of the last staged cycle (logit f16 [S,V], loss f32 [S], amax u16 [S],
+ * prob f32 [S,V] or 0) */
+int cacti_llama_io_cells(cacti_llama *model, int *tok, int *lm_tok, int *loss_scale, int *logit,
+                         int *loss, int *amax, int *prob);
+/* Stages one cycle on a freshly reset spine: mem_set_yield_ of the three inputs,
+ * Llama::apply, and (want_grad) sink.add(loss, loss_scale) + vadd_vjp over all parameters
+ * (examples/open_llama_3b_train.rs:350-389). */
+int cacti_llama_stage(cacti_llama *model, int want_prob, int want_grad);
+/* reset + stage + compile + resume/resume_put + sync; loss_out [S] f32 may be NULL. */
+int cacti_llama_step(cacti_llama *model, const uint16_t *tok, const uint16_t *lm_tok,
+                     const float *loss_scale, int want_prob, int want_grad, float *loss_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CACTI_HIP_RUNTIME_H */

@@ -9,9 +9,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _header_symbols():
-    txt = open(os.path.join(ROOT, "include", "cacti_gpu_hip_ffi.h")).read()
-    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
-    return sorted(set(re.findall(r"\b(cacti_\w+)\s*\(", txt)))
+    syms = set()
+    for h in ("cacti_gpu_hip_ffi.h", "cacti_hip_runtime.h"):
+        txt = open(os.path.join(ROOT, "include", h)).read()
+        txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+        syms |= set(re.findall(r"\b(cacti_\w+)\s*\(", txt))
+    return sorted(syms)
 
 
 def test_library_exports_every_declared_symbol():
