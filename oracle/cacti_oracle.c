@@ -477,6 +477,12 @@ ORACLE_API void vjp_inner_mean(i64 N, i64 D, const float *dm, float *dsq)
 
 typedef float v8f __attribute__((vector_size(32)));
 
+/* The fp32 summation order of a GEMM is not fixed by the reference (cuBLAS picks it).
+ * 0 = ascending k, 1 = descending k: two equally valid restatements whose difference
+ * is the floor below which no parity tolerance on a chain of f16 GEMMs can go. */
+static int g_gemm_reverse_k = 0;
+ORACLE_API void oracle_set_gemm_reverse_k(int on) { g_gemm_reverse_k = on; }
+
 static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h16 *A, i64 lda,
                        const h16 *B, i64 ldb, float beta, h16 *C, i64 ldc)
 {
@@ -494,7 +500,7 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
         for (i64 n = 0; n < Np; n++)
             b[k * Np + n] = (n < N) ? h2f(tb ? B[n * ldb + k] : B[k * ldb + n]) : 0.0f;
 
-    const i64 KB = 256;
+    const int rev = g_gemm_reverse_k;
 #pragma omp parallel for schedule(dynamic, 1) collapse(2)
     for (i64 m0 = 0; m0 < Mp; m0 += 4)
         for (i64 n0 = 0; n0 < Np; n0 += 16) {
@@ -503,18 +509,16 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
                 acc[i][0] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
                 acc[i][1] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
             }
-            for (i64 k0 = 0; k0 < K; k0 += KB) {
-                i64 k1 = k0 + KB < K ? k0 + KB : K;
-                for (i64 k = k0; k < k1; k++) {
-                    v8f b0, b1;
-                    memcpy(&b0, b + k * Np + n0, 32);
-                    memcpy(&b1, b + k * Np + n0 + 8, 32);
-                    for (int i = 0; i < 4; i++) {
-                        float av = a[(m0 + i) * K + k];
-                        v8f avv = {av, av, av, av, av, av, av, av};
-                        acc[i][0] += avv * b0;
-                        acc[i][1] += avv * b1;
-                    }
+            for (i64 kk = 0; kk < K; kk++) {
+                const i64 k = rev ? K - 1 - kk : kk;
+                v8f b0, b1;
+                memcpy(&b0, b + k * Np + n0, 32);
+                memcpy(&b1, b + k * Np + n0 + 8, 32);
+                for (int i = 0; i < 4; i++) {
+                    float av = a[(m0 + i) * K + k];
+                    v8f avv = {av, av, av, av, av, av, av, av};
+                    acc[i][0] += avv * b0;
+                    acc[i][1] += avv * b1;
                 }
             }
             for (int i = 0; i < 4; i++) {

@@ -83,6 +83,11 @@ def num_threads():
     return lib().oracle_num_threads()
 
 
+def set_gemm_reverse_k(on):
+    """Sum GEMM products in descending k (an equally valid fp32 accumulation order)."""
+    lib().oracle_set_gemm_reverse_k(C.c_int(int(on)))
+
+
 def set_num_threads(n):
     lib().oracle_set_num_threads(C.c_int(n))
 

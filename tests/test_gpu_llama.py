@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from tests.llama_ref import make_inputs
-from tests.util import assert_parity, rel_l2
+from tests.util import assert_parity, rel_l2, max_rel
 
 pytestmark = pytest.mark.gpu
 
@@ -18,15 +18,34 @@ def _model(cfg, pool_bytes=1 << 30, pagelocked=True):
     return ctx, m
 
 
-def _compare(oracle, cfg, m, out, ref, tag):
+def _order_floor(oracle, cfg, flat, tok, lm_tok, scale, ref):
+    """rel-L2 / max-rel between two equally valid restatements of the reference: the oracle
+    with its GEMMs summed in ascending and in descending k.  A chain of f16-rounded GEMMs
+    turns any change of fp32 summation order into independent f16 rounding flips, so this is
+    the floor for ANY implementation that does not share the oracle's order (cuBLAS and the
+    MFMA kernels alike); the gradient check is made relative to it."""
+    oracle.set_gemm_reverse_k(1)
+    try:
+        alt = oracle.llama_step(cfg, flat, tok, lm_tok, scale)
+    finally:
+        oracle.set_gemm_reverse_k(0)
+    a, b = oracle.split_params(cfg, ref["grad"]), oracle.split_params(cfg, alt["grad"])
+    return {n: (rel_l2(b[n], a[n]), max_rel(b[n], a[n])) for n in a}
+
+
+def _compare(oracle, cfg, m, ref, floor, tag):
     grads = m.grads()
     want = oracle.split_params(cfg, ref["grad"])
     assert len(grads) == 3 + 9 * cfg.L
-    worst = 0.0
+    worst = worst_ratio = 0.0
     for name, g in grads.items():
-        e2, _ = assert_parity(g, want[name], tag + ":" + name)
-        worst = max(worst, e2)
-    print("%s: worst gradient rel_l2 vs oracle %.3e" % (tag, worst), flush=True)
+        f2, fm = floor[name]
+        # north-star bar (1e-3 / 2e-2) where the order floor allows it, else 1.3 x the floor
+        e2, em = assert_parity(g, want[name], tag + ":" + name, l2=max(1e-3, 1.3 * f2),
+                               mx=max(2e-2, 1.5 * fm))
+        worst, worst_ratio = max(worst, e2), max(worst_ratio, e2 / f2)
+    print("%s: worst gradient rel_l2 vs oracle %.3e (%.2f x the summation-order floor)"
+          % (tag, worst, worst_ratio), flush=True)
 
 
 def test_tiny_llama_step_all_gradients(oracle):
@@ -40,7 +59,14 @@ def test_tiny_llama_step_all_gradients(oracle):
     assert_parity(out["logit"], ref["logit"], "logit")
     assert np.mean(out["amax"] == ref["amax"]) > 0.99       # ties in f16 logits may differ
     assert abs(out["prob"].sum(1) - 1).max() < 1e-4
-    _compare(oracle, cfg, m, out, ref, "healthy")
+    floor = _order_floor(oracle, cfg, flat, tok, lm_tok, scale, ref)
+    _compare(oracle, cfg, m, ref, floor, "healthy")
+    # and against exact arithmetic (fp64 autograd): no further from the truth than the oracle is
+    from tests.llama_ref import torch_step
+    _, g64, _ = torch_step(cfg, oracle.split_params(cfg, flat), tok, lm_tok, scale)
+    want = oracle.split_params(cfg, ref["grad"])
+    for name, g in m.grads().items():
+        assert rel_l2(g, g64[name]) <= 1.15 * rel_l2(want[name], g64[name]) + 1e-4, name
     names = ctx.log_names()
     assert names.count("yield_set") == 3 and "unlive" in names and "rms_norm_bwd" in names
     # a second cycle on the same context (reset GCs the first one's cells) gives the same result
@@ -115,7 +141,7 @@ def test_capped_pool_spills_and_matches(oracle, pagelocked):
 def test_pool_too_small_is_a_clean_error(oracle):
     from cacti_amd.ffi import CactiError
     cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=3)
-    ctx, m = _model(cfg, pool_bytes=3 << 20)                  # smaller than one thunk's working set
+    ctx, m = _model(cfg, pool_bytes=1 << 20)                  # smaller than one thunk's working set
     m.put_params_flat(flat)
     with pytest.raises(CactiError) as e:
         m.step(tok, lm_tok, scale)
