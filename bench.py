@@ -1,0 +1,326 @@
+#!/usr/bin/env python3
+"""bench.py -- fwd + loss + full-gradient bwd tokens/sec of the OpenLLaMA-3B-shaped fp16 step
+on one MI355X, with the roofline of the dominant kernel and the CPU port timed beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--pool-gb G] [--no-cpu-baseline]
+    python bench.py --workload adjoints      # HBM-bound adjoint kernels at 3B shapes
+    python bench.py --workload gemm          # every GEMM shape of the step, standalone
+
+Prints ONE JSON line on stdout.  A step = reset + stage + vadd_vjp + compile + resume of
+the 26-layer cycle (the reference's per-cycle control flow), inputs resident on the device
+except the 3 small input cells (tokens, labels, loss scale: 16 KiB) that are put every step.
+"""
+import argparse
+import json
+import os
+import re
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LLAMA_3B = dict(S=2048, D=3200, H=32, Dh=100, F=8640, V=32000, L=26, eps=1e-6)
+PEAK_MFMA_F16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
+PEAK_HBM_GBS = 8000.0              # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def synth_params(model, seed=0, std=0.02):
+    """Seeded synthetic weights ~N(0, std) (norm weights ~N(1, std)): one 2^26-element normal
+    block, read at a tensor-dependent offset with wrap-around (drawing 3.4e9 fresh normals on
+    the host would take minutes and changes nothing that is measured)."""
+    r = np.random.default_rng(seed)
+    n = 1 << 26
+    block = (r.standard_normal(n, dtype=np.float32) * std).astype(np.float16)
+    off = 0
+    for i, (name, shape) in enumerate(model.params):
+        cnt = int(np.prod(shape))
+        idx0 = (off * 7919) % n
+        if idx0 + cnt <= n:
+            w = block[idx0:idx0 + cnt]
+        else:
+            reps = (idx0 + cnt + n - 1) // n
+            w = np.tile(block, reps)[idx0:idx0 + cnt]
+        w = w.reshape(shape)
+        if name.endswith("norm"):
+            w = (w.astype(np.float32) + 1.0).astype(np.float16)
+        model.put_param(i, w)
+        off += cnt
+
+
+def synth_inputs(cfg, seed=1, grad_scale=1024.0):
+    r = np.random.default_rng(seed)
+    tok = r.integers(0, cfg["V"], cfg["S"]).astype(np.uint16)
+    lm_tok = np.concatenate([tok[1:], tok[:1]]).astype(np.uint16)
+    scale = np.full(cfg["S"], grad_scale / (cfg["S"] - 1), np.float32)   # train.rs:521-530
+    scale[0] = 0.0
+    return tok, lm_tok, scale
+
+
+GEMM_RE = re.compile(r"^(block_matmul|matmul)\[([NT])([NT]),(\d+)x(\d+)x(\d+)x(\d+)(,acc)?\]$")
+
+
+def gemm_flops(label):
+    m = GEMM_RE.match(label)
+    if not m:
+        return None
+    H, M, N, K = (int(m.group(i)) for i in (4, 5, 6, 7))
+    return 2.0 * H * M * N * K
+
+
+def kernel_symbol(label):
+    m = GEMM_RE.match(label)
+    ta, tb = m.group(2) == "T", m.group(3) == "T"
+    return "gemm_f16_kernel<TA=%d,TB=%d>" % (ta, tb)
+
+
+def cpu_baseline(cfg):
+    """The CPU port (the oracle) on a bounded sample of the same workload: one decoder layer
+    and the LM head + loss at full shapes, forward + backward, extrapolated to 26 layers."""
+    from oracle import oracle as o
+    from tests.llama_ref import make_inputs
+    times = {}
+    for L in (0, 1):
+        c = dict(cfg, L=L)
+        ocfg, flat, tok, lm_tok, scale = make_inputs(c, seed=0, norm_mean=1.0, grad_scale=1024.0)
+        t0 = time.time()
+        o.llama_step(ocfg, flat, tok, lm_tok, scale)
+        times[L] = time.time() - t0
+        log("cpu_baseline: oracle L=%d fwd+bwd %.2f s" % (L, times[L]))
+    layer = max(times[1] - times[0], 1e-9)
+    full = times[0] + cfg["L"] * layer
+    return {"value": cfg["S"] / full, "unit": "tokens/s", "cores": o.num_threads(), "kind": "port",
+            "sample": "oracle fwd+bwd of 1 of %d layers (%.2f s) and of embedding+LM head+loss "
+                      "(%.2f s) at full shapes, S=%d; step time extrapolated as head + %d x layer"
+                      % (cfg["L"], layer, times[0], cfg["S"], cfg["L"])}
+
+
+def run_step(args):
+    import torch
+    from cacti_amd.runtime import Ctx, Llama
+    cfg = dict(LLAMA_3B)
+    if args.layers is not None:
+        cfg["L"] = args.layers
+    pool = int(args.pool_gb * (1 << 30)) if args.pool_gb else 0
+    ctx = Ctx(0, pool, True)
+    model = Llama(ctx, **cfg)
+    t0 = time.time()
+    synth_params(model)
+    log("params staged on the host in %.1f s" % (time.time() - t0))
+    tok, lm_tok, scale = synth_inputs(cfg)
+    for _ in range(args.warmup):
+        model.step(tok, lm_tok, scale, want_loss=False)
+    ctx.sync()
+    torch.cuda.synchronize()
+    ctx.set_timing(0)
+    ctx.set_timing(2)
+    st0 = ctx.stats()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.step(tok, lm_tok, scale, want_loss=False)
+    ctx.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    rep = ctx.timing_report()
+    st1 = ctx.stats()
+    ctx.set_timing(0)
+    loss = model.step(tok, lm_tok, scale)
+    assert np.all(np.isfinite(loss)), "non-finite loss"
+    ms = dt / args.steps * 1e3
+    tokens_s = cfg["S"] * args.steps / dt
+
+    # per-label device time; the dominant GEMM kernel gives the roofline entry
+    by_sym = {}
+    kernels = []
+    for label, (cnt, tot_ms) in sorted(rep.items(), key=lambda kv: -kv[1][1]):
+        fl = gemm_flops(label)
+        ent = {"label": label, "launches": cnt, "avg_us": tot_ms / cnt * 1e3,
+               "total_ms_per_step": tot_ms / args.steps}
+        if fl is not None:
+            ent["tflops"] = fl / (tot_ms / cnt * 1e-3) / 1e12
+            if label.startswith("matmul"):
+                s = by_sym.setdefault(kernel_symbol(label), [0.0, 0.0, 0])
+                s[0] += fl * cnt
+                s[1] += tot_ms * 1e-3
+                s[2] += cnt
+        kernels.append(ent)
+    dev_ms = sum(v[1] for v in rep.values()) / args.steps
+    sym, (fl, sec, cnt) = max(by_sym.items(), key=lambda kv: kv[1][1])
+    achieved = fl / sec / 1e12
+    roofline = {"bound": "mfma", "kernel": sym, "launches_per_step": cnt // args.steps,
+                "avg_launch_us": sec / cnt * 1e6, "flops_per_launch": fl / cnt,
+                "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": None}
+    out = {
+        "metric": "fwd+bwd tokens/sec, 3B-shaped fp16 step, 1 GPU", "value": tokens_s,
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic (seeded N(0,0.02) weights, uniform token ids)",
+        "config": {"workload": "OpenLLaMA-3B-shaped full-gradient step: %d layers, hidden 3200, "
+                               "32 heads x 100, ffn 8640, vocab 32000, batch 1, seq 2048, "
+                               "fwd + softmax-CE loss + bwd" % cfg["L"],
+                   "pool_cap_bytes": st1["pool_cap"], "pool_peak_bytes": st1["pool_peak"],
+                   "spill_evictions_per_step": (st1["n_evict"] - st0["n_evict"]) / args.steps,
+                   "spill_d2h_bytes_per_step": (st1["bytes_d2h"] - st0["bytes_d2h"]) / args.steps},
+        "device_ms_per_step": dev_ms,
+        "roofline": roofline,
+        "kernels": kernels[:24],
+    }
+    model.close()
+    ctx.close()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(LLAMA_3B)
+    else:
+        out["cpu_baseline"] = None
+    return out
+
+
+def time_launches(fn, stream_sync, n_warm=3, n_iter=20):
+    """Average device time of fn(i) over n_iter back-to-back launches (torch events on the
+    current stream, which is the stream cacti_amd.ops launches on)."""
+    import torch
+    for i in range(n_warm):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(n_iter):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n_iter * 1e-3
+
+
+def run_adjoints(args):
+    """BASELINE config 2-4 kernels at 3B shapes; buffers rotate over > 256 MB so every launch
+    reads HBM, not the Infinity Cache."""
+    import torch
+    from cacti_amd import ops
+    N, D, H, Dh, F, V = 2048, 3200, 32, 100, 8640, 32000
+    g = torch.Generator(device="cuda").manual_seed(0)
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, device="cuda", generator=g) * std).half()
+
+    res = []
+
+    def add(name, sec, nbytes):
+        res.append({"kernel": name, "us": sec * 1e6, "algorithmic_bytes": nbytes,
+                    "achieved_GBs": nbytes / sec / 1e9, "frac_of_8TBs": nbytes / sec / 1e9 / PEAK_HBM_GBS})
+        log("%-22s %8.1f us  %7.1f GB/s  (%.1f%% of 8 TB/s)" % (name, sec * 1e6, nbytes / sec / 1e9,
+                                                             100 * nbytes / sec / 1e9 / PEAK_HBM_GBS))
+
+    R = 8
+    xs, dys, dxs = [rn(N, D) for _ in range(R)], [rn(N, D) for _ in range(R)], [rn(N, D) for _ in range(R)]
+    w = rn(D)
+    add("rms_norm_bwd", time_launches(lambda i: ops.rms_norm_bwd(xs[i % R], w, 1e-6, dys[i % R], dxs[i % R], None), None),
+        3 * 2 * N * D + 2 * 2 * D)
+    add("rms_norm_fwd", time_launches(lambda i: ops.rms_norm_fwd(xs[i % R], w, 1e-6), None), 2 * 2 * N * D + 2 * D)
+    cos, sin = ops.rope_tables(N, Dh)
+    q = [rn(N, H, Dh) for _ in range(12)]
+    add("rope_bwd", time_launches(lambda i: ops.rope_bwd(q[i % 12], cos, sin), None), 2 * 2 * N * H * Dh + 2 * 2 * N * Dh)
+    add("rope_fwd", time_launches(lambda i: ops.rope_fwd(q[i % 12], cos, sin), None), 2 * 2 * N * H * Dh + 2 * 2 * N * Dh)
+    del xs, dys, dxs, q
+    R = 3
+    gs, us, dhs = [rn(N, F) for _ in range(R)], [rn(N, F) for _ in range(R)], [rn(N, F) for _ in range(R)]
+    add("silu_gate_bwd", time_launches(lambda i: ops.silu_gate_bwd(gs[i % R], us[i % R], dhs[i % R]), None), 5 * 2 * N * F)
+    add("silu_gate_fwd", time_launches(lambda i: ops.silu_gate_fwd(gs[i % R], us[i % R]), None), 3 * 2 * N * F)
+    del gs, us, dhs
+    lg = [rn(N, V, std=2.0) for _ in range(3)]
+    tok = torch.randint(0, V, (N,), device="cuda").to(torch.int16)
+    sc = torch.full((N,), 1.0 / N, device="cuda")
+    add("softmax_ce_bwd", time_launches(lambda i: ops.softmax_ce_bwd(lg[i % 3], tok, sc), None), 2 * 2 * N * V)
+    add("softmax_ce_fwd(loss)", time_launches(lambda i: ops.softmax_ce_fwd(lg[i % 3], tok, want_prob=False), None), 2 * N * V)
+    del lg
+    s16 = [rn(N, H, N) for _ in range(2)]
+    dp = rn(N, H, N)
+    add("causal_softmax_fwd", time_launches(lambda i: ops.causal_softmax_fwd(s16[i % 2]), None, n_iter=10), 2 * 2 * N * H * N)
+    add("causal_softmax_bwd", time_launches(lambda i: ops.causal_softmax_bwd(s16[i % 2], dp), None, n_iter=10), 3 * 2 * N * H * N)
+    dom = max(res, key=lambda r: r["algorithmic_bytes"] if r["kernel"] == "silu_gate_bwd" else 0)
+    return {"metric": "HBM-bound adjoint kernels at OpenLLaMA-3B shapes", "value": dom["achieved_GBs"],
+            "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "dtype": "f16",
+            "config": {"workload": "adjoint microbench: RMSNorm [2048,3200], RoPE [2048,32,100], "
+                                   "SiLU-gate [2048,8640], softmax-CE [2048,32000], causal softmax [2048,32,2048]"},
+            "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["achieved_GBs"],
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_of_8TBs"], "traffic": None},
+            "kernels": res}
+
+
+def run_gemm(args):
+    """Every GEMM shape of the step, standalone: TFLOP/s per shape."""
+    import torch
+    from cacti_amd import ops
+    N, D, F, V, H, Dh = 2048, 3200, 8640, 32000, 32, 100
+    g = torch.Generator(device="cuda").manual_seed(0)
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, device="cuda", generator=g) * std).half()
+
+    res = []
+    shapes = [("proj fwd NT", False, True, (N, D), (D, D)), ("proj dgrad NN", False, False, (N, D), (D, D)),
+              ("proj wgrad TN", True, False, (N, D), (N, D)),
+              ("ffn-up fwd NT", False, True, (N, D), (F, D)), ("ffn-up dgrad NN", False, False, (N, F), (F, D)),
+              ("ffn-up wgrad TN", True, False, (N, F), (N, D)),
+              ("ffn-down fwd NT", False, True, (N, F), (D, F)), ("ffn-down dgrad NN", False, False, (N, D), (D, F)),
+              ("ffn-down wgrad TN", True, False, (N, D), (N, F)),
+              ("head fwd NT", False, True, (N, D), (V, D)), ("head dgrad NN", False, False, (N, V), (V, D)),
+              ("head wgrad TN", True, False, (N, V), (N, D))]
+    for name, ta, tb, sa, sb in shapes:
+        a, b = rn(*sa), rn(*sb, std=0.02)
+        M, K = (sa[1], sa[0]) if ta else sa
+        Nn = sb[0] if tb else sb[1]
+        out = torch.empty(M, Nn, device="cuda", dtype=torch.float16)
+        sec = time_launches(lambda i: ops.gemm(a, b, ta, tb, 1.0, 0.0, out), None, n_iter=10)
+        fl = 2.0 * M * Nn * K
+        res.append({"shape": name, "M": M, "N": Nn, "K": K, "us": sec * 1e6, "tflops": fl / sec / 1e12})
+        log("%-18s M=%5d N=%5d K=%5d %9.1f us %7.1f TFLOP/s" % (name, M, Nn, K, sec * 1e6, fl / sec / 1e12))
+    q, k, v = rn(N, H, Dh), rn(N, H, Dh), rn(N, H, Dh)
+    sec = time_launches(lambda i: ops.block_matmul_qk(q, k, 0.1), None, n_iter=5)
+    fl = 2.0 * H * N * N * Dh
+    res.append({"shape": "attn QK^T (32 blocks)", "us": sec * 1e6, "tflops": fl / sec / 1e12})
+    log("%-18s %9.1f us %7.1f TFLOP/s (dense)" % ("attn QK^T", sec * 1e6, fl / sec / 1e12))
+    p = rn(N, H, N)
+    sec = time_launches(lambda i: ops.block_matmul_pv(p, v), None, n_iter=5)
+    res.append({"shape": "attn PV (32 blocks)", "us": sec * 1e6, "tflops": fl / sec / 1e12})
+    log("%-18s %9.1f us %7.1f TFLOP/s (dense)" % ("attn PV", sec * 1e6, fl / sec / 1e12))
+    best = max(r["tflops"] for r in res)
+    return {"metric": "GEMM shapes of the 3B step, standalone", "value": best, "unit": "TFLOP/s",
+            "n_gpus": 1, "higher_is_better": True, "dtype": "f16",
+            "config": {"workload": "f16 GEMM, fp32 accumulate, f16 out"},
+            "roofline": {"bound": "mfma", "achieved": best, "peak": PEAK_MFMA_F16_TFLOPS,
+                         "unit": "TFLOP/s", "frac": best / PEAK_MFMA_F16_TFLOPS, "traffic": None},
+            "kernels": res}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--pool-gb", type=float, default=0.0,
+                    help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
+    ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm"], default="step")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
+            "has no collective); --gpus %d is not supported" % args.gpus)
+        sys.exit(2)
+    if args.workload == "step":
+        out = run_step(args)
+    elif args.workload == "adjoints":
+        out = run_adjoints(args)
+    else:
+        out = run_gemm(args)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -98,7 +98,8 @@ CACTI_API void *cacti_ctx_stream(cacti_ctx *ctx) { return (void *)ctx->c.stream(
 
 CACTI_API int cacti_ctx_set_timing(cacti_ctx *ctx, int on)
 {
-    ctx->c.set_timing(on != 0);
+    ctx->c.set_timing(on);
+    if (!on) ctx->c.clear_timings();
     return 0;
 }
 
@@ -107,6 +108,8 @@ CACTI_API int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap)
     CACTI_REQUIRE(ctx && buf && cap > 0, CACTI_E_INVALID, "timing_report: null pointer");
     size_t n = 0;
     buf[0] = 0;
+    int rc = ctx->c.collect_timings();
+    if (rc) return rc;
     for (auto &kv : ctx->c.timings()) {
         int w = snprintf(buf + n, cap - n, "%s %llu %.4f\n", kv.first.c_str(),
                          (unsigned long long)kv.second.second, kv.second.first);

@@ -94,6 +94,10 @@ Ctx::~Ctx()
 {
     if (stream_) hipStreamSynchronize(stream_);
     for (auto &c : cells_) host_free(c);
+    for (auto &e : ev_pool_) {
+        hipEventDestroy(e.first);
+        hipEventDestroy(e.second);
+    }
     if (ev0_) hipEventDestroy(ev0_);
     if (ev1_) hipEventDestroy(ev1_);
     if (base_) hipFree(base_);
@@ -541,15 +545,27 @@ int Ctx::run_entry(const Entry &e)
         // resolve pointers only now: eviction during allocation cannot move pinned cells
         for (CellPtr a : e.args) ap.push_back(dev_ptr(cells_[a].voff));
         for (CellPtr o : e.outs) op.push_back(dev_ptr(cells_[o].voff));
-        if (timing_) hipEventRecord(ev0_, stream_);
+        hipEvent_t e0 = ev0_, e1 = ev1_;
+        if (timing_ == 2) {
+            if (ev_keys_.size() == ev_pool_.size()) {
+                hipEvent_t a, b;
+                hipEventCreate(&a);
+                hipEventCreate(&b);
+                ev_pool_.emplace_back(a, b);
+            }
+            e0 = ev_pool_[ev_keys_.size()].first;
+            e1 = ev_pool_[ev_keys_.size()].second;
+            ev_keys_.push_back(sp.key(aty, e.acc_mask));
+        }
+        if (timing_) hipEventRecord(e0, stream_);
         rc = sp.run(*this, aty, ap.data(), oty, op.data(), e.acc_mask,
                     ws_off == kNoOffset ? nullptr : dev_ptr(ws_off), ws_bytes);
-        if (timing_ && !rc) {
-            hipEventRecord(ev1_, stream_);
-            hipEventSynchronize(ev1_);
+        if (timing_) hipEventRecord(e1, stream_);
+        if (timing_ == 1 && !rc) {
+            hipEventSynchronize(e1);
             float ms = 0;
-            hipEventElapsedTime(&ms, ev0_, ev1_);
-            auto &t = times_[sp.name()];
+            hipEventElapsedTime(&ms, e0, e1);
+            auto &t = times_[sp.key(aty, e.acc_mask)];
             t.first += ms;
             t.second++;
         }
@@ -564,6 +580,20 @@ int Ctx::run_entry(const Entry &e)
     for (CellPtr a : e.args) cells_[a].pin--;
     for (CellPtr o : e.outs) cells_[o].pin--;
     return rc;
+}
+
+int Ctx::collect_timings()
+{
+    CACTI_HIP(hipStreamSynchronize(stream_));
+    for (size_t i = 0; i < ev_keys_.size(); i++) {
+        float ms = 0;
+        if (hipEventElapsedTime(&ms, ev_pool_[i].first, ev_pool_[i].second) != hipSuccess) continue;
+        auto &t = times_[ev_keys_[i]];
+        t.first += ms;
+        t.second++;
+    }
+    ev_keys_.clear();
+    return 0;
 }
 
 int Ctx::resume(CellPtr *yield_cell)

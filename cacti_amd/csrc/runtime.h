@@ -96,6 +96,8 @@ struct ThunkSpec {
     virtual int nout() const { return 1; }
     virtual int out_ty(const std::vector<CellType> &arg, std::vector<CellType> &out) const = 0;
     virtual size_t workspace(const std::vector<CellType> &) const { return 0; }
+    // label under which launches are grouped in the timing report (name + shape for GEMMs)
+    virtual std::string key(const std::vector<CellType> &, uint32_t) const { return name(); }
     virtual int run(Ctx &ctx, const std::vector<CellType> &aty, void *const *a,
                     const std::vector<CellType> &oty, void *const *o, uint32_t acc_mask,
                     void *ws, size_t ws_bytes) const = 0;
@@ -167,7 +169,11 @@ class Ctx {
     const std::vector<Entry> &log() const { return log_; }
     const ThunkSpec &thunk(int i) const { return *thunks_[i]; }
     const char *entry_name(size_t i) const;
-    void set_timing(bool on) { timing_ = on; }
+    // 0 = off; 1 = sync after every thunk; 2 = event pairs recorded without syncing and read
+    // back by collect_timings() (measures each launch inside an undisturbed run)
+    void set_timing(int mode) { timing_ = mode; }
+    int collect_timings();
+    void clear_timings() { times_.clear(); }
     const std::map<std::string, std::pair<double, uint64_t>> &timings() const { return times_; }
 
    private:
@@ -195,7 +201,9 @@ class Ctx {
     // statistics
     uint64_t n_alloc_ = 0, n_evict_ = 0, n_upload_ = 0, bytes_d2h_ = 0, bytes_h2d_ = 0,
              n_soft_oom_ = 0, n_run_ = 0, host_bytes_ = 0;
-    bool timing_ = false;
+    int timing_ = 0;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> ev_pool_;
+    std::vector<std::string> ev_keys_;
     std::map<std::string, std::pair<double, uint64_t>> times_;
     hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
 };

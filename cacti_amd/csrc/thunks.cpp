@@ -209,6 +209,16 @@ struct MatMulSpec : ThunkSpec {
                                                   d.sa, a[1], d.ldb, d.sb, (acc & 1) ? 1.f : 0.f,
                                                   o[0], d.ldc, d.sc, S(c));
     }
+    std::string key(const std::vector<CellType> &aty, uint32_t acc) const override
+    {
+        Dims d;
+        if (dims(aty, d)) return name();
+        char buf[128];
+        snprintf(buf, sizeof(buf), "%s[%c%c,%lldx%lldx%lldx%lld%s]", name(), ta ? 'T' : 'N',
+                 tb ? 'T' : 'N', (long long)d.H, (long long)d.M, (long long)d.N, (long long)d.K,
+                 (acc & 1) ? ",acc" : "");
+        return buf;
+    }
     std::unique_ptr<ThunkSpec> mm(bool x, bool y) const
     {
         return std::unique_ptr<ThunkSpec>(new MatMulSpec(x, y, alpha, nblk));

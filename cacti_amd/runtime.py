@@ -63,15 +63,16 @@ class Ctx:
     def stream(self):
         return ffi.lib().cacti_ctx_stream(self._c)
 
-    def set_timing(self, on):
-        ffi.call("cacti_ctx_set_timing", self._c, int(on))
+    def set_timing(self, mode):
+        """0 off (clears totals), 1 sync per thunk, 2 event pairs without syncing."""
+        ffi.call("cacti_ctx_set_timing", self._c, int(mode))
 
     def timing_report(self):
-        buf = C.create_string_buffer(1 << 16)
+        buf = C.create_string_buffer(1 << 18)
         ffi.call("cacti_ctx_timing_report", self._c, buf, len(buf))
         out = {}
         for line in buf.value.decode().splitlines():
-            name, cnt, ms = line.split()
+            name, cnt, ms = line.rsplit(" ", 2)
             out[name] = (int(cnt), float(ms))
         return out
 

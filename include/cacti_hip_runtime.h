@@ -51,8 +51,11 @@ int cacti_ctx_destroy(cacti_ctx *ctx);
 int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out);
 int cacti_ctx_sync(cacti_ctx *ctx);
 void *cacti_ctx_stream(cacti_ctx *ctx);                 /* the hipStream_t all work runs on */
-/* per-thunk wall times (CACTI_DEBUG_TIMING, src/ctx.rs:114-133): on = 1 syncs after every
- * thunk; the report is text "name count total_ms" per line. */
+/* per-thunk device times (CACTI_DEBUG_TIMING, src/ctx.rs:114-133).  mode 1 syncs after
+ * every thunk; mode 2 records a HIP event pair around every launch without syncing and
+ * reads them back in the report, so a run is measured undisturbed; 0 switches timing off
+ * and clears the totals.  The report is text, one "label count total_ms" line per label;
+ * GEMM labels carry the transposes and nblk x M x N x K. */
 int cacti_ctx_set_timing(cacti_ctx *ctx, int on);
 int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap);
 

@@ -486,24 +486,34 @@ ORACLE_API void oracle_set_gemm_reverse_k(int on) { g_gemm_reverse_k = on; }
 static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h16 *A, i64 lda,
                        const h16 *B, i64 ldb, float beta, h16 *C, i64 ldc)
 {
-    /* pack op(A) as f32 [M,K] and op(B) as f32 [K,Np] with Np a multiple of 16 */
-    i64 Np = (N + 15) / 16 * 16;
-    float *a = (float *)aligned_alloc(64, (size_t)((M + 3) / 4 * 4) * (size_t)K * 4 + 64);
+    /* pack op(A) as f32 panels of 4 rows [Mp/4][K][4] and op(B) as f32 panels of 16
+     * columns [Np/16][K][16], so the inner loop streams contiguous memory */
+    const i64 Np = (N + 15) / 16 * 16, Mp = (M + 3) / 4 * 4;
+    float *a = (float *)aligned_alloc(64, (size_t)Mp * (size_t)K * 4 + 64);
     float *b = (float *)aligned_alloc(64, (size_t)K * (size_t)Np * 4 + 64);
-    i64 Mp = (M + 3) / 4 * 4;
 #pragma omp parallel for schedule(static)
-    for (i64 m = 0; m < Mp; m++)
+    for (i64 mp = 0; mp < Mp / 4; mp++)
         for (i64 k = 0; k < K; k++)
-            a[m * K + k] = (m < M) ? h2f(ta ? A[k * lda + m] : A[m * lda + k]) : 0.0f;
+            for (int i = 0; i < 4; i++) {
+                const i64 m = mp * 4 + i;
+                a[(mp * K + k) * 4 + i] = (m < M) ? h2f(ta ? A[k * lda + m] : A[m * lda + k]) : 0.0f;
+            }
 #pragma omp parallel for schedule(static)
-    for (i64 k = 0; k < K; k++)
-        for (i64 n = 0; n < Np; n++)
-            b[k * Np + n] = (n < N) ? h2f(tb ? B[n * ldb + k] : B[k * ldb + n]) : 0.0f;
+    for (i64 np = 0; np < Np / 16; np++)
+        for (i64 k = 0; k < K; k++)
+            for (int j = 0; j < 16; j++) {
+                const i64 n = np * 16 + j;
+                b[(np * K + k) * 16 + j] = (n < N) ? h2f(tb ? B[n * ldb + k] : B[k * ldb + n]) : 0.0f;
+            }
 
     const int rev = g_gemm_reverse_k;
-#pragma omp parallel for schedule(dynamic, 1) collapse(2)
-    for (i64 m0 = 0; m0 < Mp; m0 += 4)
-        for (i64 n0 = 0; n0 < Np; n0 += 16) {
+#pragma omp parallel for schedule(dynamic, 1)
+    for (i64 np = 0; np < Np / 16; np++) {
+        const float *bp = b + np * K * 16;
+        const i64 n0 = np * 16;
+        for (i64 mp = 0; mp < Mp / 4; mp++) {
+            const float *ap = a + mp * K * 4;
+            const i64 m0 = mp * 4;
             v8f acc[4][2];
             for (int i = 0; i < 4; i++) {
                 acc[i][0] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
@@ -512,20 +522,20 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
             for (i64 kk = 0; kk < K; kk++) {
                 const i64 k = rev ? K - 1 - kk : kk;
                 v8f b0, b1;
-                memcpy(&b0, b + k * Np + n0, 32);
-                memcpy(&b1, b + k * Np + n0 + 8, 32);
+                memcpy(&b0, bp + k * 16, 32);
+                memcpy(&b1, bp + k * 16 + 8, 32);
                 for (int i = 0; i < 4; i++) {
-                    float av = a[(m0 + i) * K + k];
-                    v8f avv = {av, av, av, av, av, av, av, av};
+                    const float av = ap[k * 4 + i];
+                    const v8f avv = {av, av, av, av, av, av, av, av};
                     acc[i][0] += avv * b0;
                     acc[i][1] += avv * b1;
                 }
             }
             for (int i = 0; i < 4; i++) {
-                i64 m = m0 + i;
+                const i64 m = m0 + i;
                 if (m >= M) break;
                 for (int j = 0; j < 16; j++) {
-                    i64 n = n0 + j;
+                    const i64 n = n0 + j;
                     if (n >= N) break;
                     float v = alpha * acc[i][j >> 3][j & 7];
                     if (beta != 0.0f) v += beta * h2f(C[m * ldc + n]);
@@ -533,6 +543,7 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
                 }
             }
         }
+    }
     free(a);
     free(b);
 }
