@@ -14,22 +14,11 @@
 // The MFMA is issued with the B fragment as first operand, so a lane ends up with 4
 // consecutive columns of one row of C per accumulator group and stores 8 bytes at a time.
 #include "common.h"
+#include "gemm_internal.h"
 
 using namespace cacti;
 
 namespace {
-
-struct GemmArgs {
-    int64_t M, N, K;
-    float alpha, beta;
-    const half_t *A;
-    int64_t lda, sa;
-    const half_t *B;
-    int64_t ldb, sb;
-    half_t *C;
-    int64_t ldc, sc;
-    int tiles_m, tiles_n;
-};
 
 template <int VEC> struct VecT;
 template <> struct VecT<8> { typedef uint4 type; };
@@ -166,14 +155,17 @@ __global__ void __launch_bounds__(NT) gemm_f16_kernel(GemmArgs p)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    const int nk = (int)((p.K + BK - 1) / BK);
-    la.load(A, p.lda, m0, p.M, 0, p.K);
-    lb.load(B, p.ldb, n0, p.N, 0, p.K);
-    la.store(As[0]);
-    lb.store(Bs[0]);
+    int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;
+    if (p.tri == 1 && n0 > m0 + BM - 1) return;               // uniform for the block
+    if (p.tri == 2) nk = min(nk, (int)((m0 + BM + BK - 1) / BK));
+    if (p.tri == 3) kt0 = (int)(m0 / BK);
+    la.load(A, p.lda, m0, p.M, (int64_t)kt0 * BK, p.K);
+    lb.load(B, p.ldb, n0, p.N, (int64_t)kt0 * BK, p.K);
+    la.store(As[kt0 & 1]);
+    lb.store(Bs[kt0 & 1]);
     __syncthreads();
 
-    for (int kt = 0; kt < nk; kt++) {
+    for (int kt = kt0; kt < nk; kt++) {
         const int cur = kt & 1;
         if (kt + 1 < nk) {
             la.load(A, p.lda, m0, p.M, (int64_t)(kt + 1) * BK, p.K);
@@ -262,12 +254,17 @@ inline bool mult(int64_t v, int64_t a) { return v % a == 0; }
 
 }  // namespace
 
-CACTI_API int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N,
-                                                 int64_t K, float alpha, const void *A, int64_t lda,
-                                                 int64_t stride_a, const void *B, int64_t ldb,
-                                                 int64_t stride_b, float beta, void *C, int64_t ldc,
-                                                 int64_t stride_c, void *stream)
+CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nblk, int64_t M,
+                                                     int64_t N, int64_t K, float alpha, const void *A,
+                                                     int64_t lda, int64_t stride_a, const void *B,
+                                                     int64_t ldb, int64_t stride_b, float beta,
+                                                     void *C, int64_t ldc, int64_t stride_c, int tri,
+                                                     void *stream)
 {
+    CACTI_REQUIRE(tri >= 0 && tri <= 3, CACTI_E_INVALID, "gemm: tri must be 0..3");
+    CACTI_REQUIRE(tri == 0 || (tri == 1 && M == N) || (tri == 2 && !ta && M == K) ||
+                      (tri == 3 && ta && M == K),
+                  CACTI_E_INVALID, "gemm: tri=%d needs a square (sequence x sequence) operand", tri);
     CACTI_REQUIRE(A && B && C, CACTI_E_INVALID, "gemm: null operand");
     CACTI_REQUIRE(M > 0 && N > 0 && K > 0 && nblk > 0 && nblk <= 65535, CACTI_E_INVALID,
                   "gemm: bad shape M=%lld N=%lld K=%lld nblk=%lld", (long long)M, (long long)N,
@@ -284,6 +281,7 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, i
     p.C = (half_t *)C; p.ldc = ldc; p.sc = stride_c;
     p.tiles_m = (int)((M + BM - 1) / BM);
     p.tiles_n = (int)((N + BN - 1) / BN);
+    p.tri = tri;
     CACTI_REQUIRE((int64_t)p.tiles_m * p.tiles_n < (1LL << 31), CACTI_E_NOTIMPL, "gemm: too many tiles");
 
     // widest vector every operand supports: contiguous extent, leading dimension,
@@ -300,10 +298,21 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, i
         }
     }
     hipStream_t st = (hipStream_t)stream;
+    if (vec >= 4) return gemm_mfma_launch(ta, tb, p, nblk, vec, -1, st);
     if (!ta && !tb) return launch_vec<false, false>(vec, p, nblk, st);
     if (!ta && tb) return launch_vec<false, true>(vec, p, nblk, st);
     if (ta && !tb) return launch_vec<true, false>(vec, p, nblk, st);
     return launch_vec<true, true>(vec, p, nblk, st);
+}
+
+CACTI_API int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N,
+                                                 int64_t K, float alpha, const void *A, int64_t lda,
+                                                 int64_t stride_a, const void *B, int64_t ldb,
+                                                 int64_t stride_b, float beta, void *C, int64_t ldc,
+                                                 int64_t stride_c, void *stream)
+{
+    return cacti_hip_gemm_f16_strided_batched_tri(ta, tb, nblk, M, N, K, alpha, A, lda, stride_a, B,
+                                                  ldb, stride_b, beta, C, ldc, stride_c, 0, stream);
 }
 
 CACTI_API int cacti_hip_gemm_f16(int ta, int tb, int64_t M, int64_t N, int64_t K, float alpha,

@@ -1,0 +1,35 @@
+// Shared between the generic GEMM kernel (any alignment) and the 16-byte-aligned fast path.
+#pragma once
+#include "common.h"
+
+namespace cacti {
+
+struct GemmArgs {
+    int64_t M, N, K;
+    float alpha, beta;
+    const half_t *A;
+    int64_t lda, sa;
+    const half_t *B;
+    int64_t ldb, sb;
+    half_t *C;
+    int64_t ldc, sc;
+    int tiles_m, tiles_n;
+    // triangular structure of square attention operands (0 = none):
+    //  1: only the lower triangle (n <= m) of C is wanted: tiles wholly above it are skipped
+    //     and left unwritten;
+    //  2: op(A) = A is lower triangular (zero for k > m): the k loop stops at the tile's
+    //     last row;
+    //  3: op(A) = A^T with A lower triangular (zero for k < m): the k loop starts at the
+    //     tile's first row.
+    // For 2 and 3 the entries of A above the diagonal must be zero up to the next multiple
+    // of 256 columns; beyond that they are never read.
+    int tri;
+};
+constexpr int kTriPad = 256;
+
+// tile < 0: chosen by shape
+// align = 8 (16-byte aligned operands) or 4 (8-byte aligned, e.g. head_dim 100)
+int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align, int tile,
+                     hipStream_t st);
+
+}  // namespace cacti

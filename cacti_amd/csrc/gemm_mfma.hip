@@ -1,0 +1,368 @@
+// Fast path of the f16 GEMM for operands whose rows are at least 8-byte aligned (every
+// projection, LM-head and attention GEMM of the step; head_dim 100 gives 8-byte alignment).
+//
+//   C[M,N] = alpha op(A) op(B) + beta C,   f16 in, fp32 MFMA accumulate, f16 out.
+//
+// Block tile BM x BN x 64, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN) patch of
+// 32 x 32 accumulators fed by v_mfma_f32_32x32x16_f16.
+//
+// LDS layout (both operands): [row][64 k] = 128 bytes per row, no padding; the 16-byte
+// k-chunk q of row r sits at chunk position q ^ f(r), f(r) = ((r >> 3) ^ (r & 6)) & 7.
+// With this swizzle (a) the 16-byte MFMA operand reads of 16 consecutive rows, (b) the
+// 16-byte writes of a k-contiguous global row and (c) the writes of the register
+// transpose (8 rows apart per lane) all touch 16 distinct bank groups.
+//
+// An operand whose k index is not contiguous in memory (A^T, or B not transposed) is
+// loaded as 8 k-rows x 8 tile-rows per lane with fully coalesced 16-byte loads, transposed
+// in registers with 32 v_perm_b32, and written as 8 16-byte rows: the MFMA read path is
+// identical for NN / NT / TN / TT.
+//
+// Global loads of k-tile t+1 are issued before the MFMAs of tile t and stored into the
+// other LDS buffer afterwards: one barrier per 64-deep k tile.  Workgroups are numbered so
+// that the 8 XCDs (round-robin dispatch) each walk a contiguous band of tiles and reuse
+// the operand panels in their own L2.
+#include "common.h"
+#include "gemm_internal.h"
+
+using namespace cacti;
+
+namespace {
+
+constexpr int BK = 64;
+
+__device__ __forceinline__ int swz(int r) { return ((r >> 3) ^ (r & 6)) & 7; }
+
+// 16-byte chunk q (0..7) of tile row r
+__device__ __forceinline__ int lds_off(int r, int q) { return r * BK + ((q ^ swz(r)) << 3); }
+
+// ---- global -> registers -> LDS ---------------------------------------------
+// k-contiguous operand (memory [row][k]): chunk c -> row c / 8, k-chunk c % 8
+// 8 halves at p: one 16-byte load (AL = 8) or two 8-byte loads (AL = 4: operands that are
+// only 8-byte aligned, e.g. the per-head blocks of a head_dim-100 tensor); `n` = number of
+// valid halves from p on (a multiple of AL), the rest reads as zero
+template <int AL>
+__device__ __forceinline__ uint4 load8(const half_t *p, int64_t n)
+{
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (AL == 8) {
+        if (n > 0) v = *reinterpret_cast<const uint4 *>(p);
+    } else {
+        if (n > 0) {
+            const uint2 lo = *reinterpret_cast<const uint2 *>(p);
+            v.x = lo.x;
+            v.y = lo.y;
+        }
+        if (n > 4) {
+            const uint2 hi = *reinterpret_cast<const uint2 *>(p + 4);
+            v.z = hi.x;
+            v.w = hi.y;
+        }
+    }
+    return v;
+}
+
+template <int ROWS, int NT, int AL>
+struct LoadKC {
+    static constexpr int ITEMS = ROWS * 8;
+    static constexpr int NL = (ITEMS + NT - 1) / NT;
+    uint4 st[NL];
+    __device__ __forceinline__ void load(const half_t *base, int64_t ld, int64_t row0, int64_t R,
+                                         int64_t k0, int64_t K)
+    {
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            const int c = threadIdx.x + it * NT;
+            const int row = c >> 3, kc = c & 7;
+            const int64_t gr = row0 + row, gk = k0 + kc * 8;
+            const bool on = (ITEMS % NT == 0 || c < ITEMS) && gr < R;
+            st[it] = load8<AL>(base + gr * ld + gk, on ? K - gk : 0);
+        }
+    }
+    __device__ __forceinline__ void store(half_t *lds)
+    {
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            const int c = threadIdx.x + it * NT;
+            const int row = c >> 3, kc = c & 7;
+            if (ITEMS % NT == 0 || c < ITEMS)
+                *reinterpret_cast<uint4 *>(lds + lds_off(row, kc)) = st[it];
+        }
+    }
+};
+
+// k-strided operand (memory [k][row]): item c -> row chunk c % (ROWS/8), k group c / (ROWS/8);
+// an item is 8 k x 8 rows.  T0 = first thread that takes part (lets two strided operands
+// use disjoint halves of the block).
+template <int ROWS, int NT, int T0, int AL>
+struct LoadKS {
+    static constexpr int RC = ROWS / 8;
+    static constexpr int ITEMS = RC * 8;
+    static constexpr int NTH = NT - T0 >= ITEMS ? ITEMS : NT;      // threads taking part
+    static constexpr int TB = NT - T0 >= ITEMS ? T0 : 0;
+    static constexpr int NL = (ITEMS + NTH - 1) / NTH;
+    uint4 st[NL][8];
+    __device__ __forceinline__ bool mine(int it, int &c) const
+    {
+        const int t = (int)threadIdx.x - TB;
+        c = t + it * NTH;
+        return t >= 0 && t < NTH && c < ITEMS;
+    }
+    __device__ __forceinline__ void load(const half_t *base, int64_t ld, int64_t row0, int64_t R,
+                                         int64_t k0, int64_t K)
+    {
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            int c;
+            const bool on = mine(it, c);
+            const int rc = c % RC, kq = c / RC;
+            const int64_t gr = row0 + rc * 8;
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) {
+                const int64_t gk = k0 + kq * 8 + kk;
+                st[it][kk] = load8<AL>(base + gk * ld + gr, (on && gk < K) ? R - gr : 0);
+            }
+        }
+    }
+    __device__ __forceinline__ void store(half_t *lds)
+    {
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            int c;
+            if (!mine(it, c)) continue;
+            const int rc = c % RC, kq = c / RC;
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(&st[it][0]);   // [kk][4 words]
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                // row j of the 8 x 8 block: halves (k = 0..7) = word j/2, half j%2 of each k row
+                const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+                uint4 o;
+                o.x = __builtin_amdgcn_perm(w[1 * 4 + (j >> 1)], w[0 * 4 + (j >> 1)], sel);
+                o.y = __builtin_amdgcn_perm(w[3 * 4 + (j >> 1)], w[2 * 4 + (j >> 1)], sel);
+                o.z = __builtin_amdgcn_perm(w[5 * 4 + (j >> 1)], w[4 * 4 + (j >> 1)], sel);
+                o.w = __builtin_amdgcn_perm(w[7 * 4 + (j >> 1)], w[6 * 4 + (j >> 1)], sel);
+                *reinterpret_cast<uint4 *>(lds + lds_off(rc * 8 + j, kq)) = o;
+            }
+        }
+    }
+};
+
+template <bool STRIDED, int ROWS, int NT, int T0, int AL> struct Loader;
+template <int ROWS, int NT, int T0, int AL>
+struct Loader<false, ROWS, NT, T0, AL> : LoadKC<ROWS, NT, AL> {};
+template <int ROWS, int NT, int T0, int AL>
+struct Loader<true, ROWS, NT, T0, AL> : LoadKS<ROWS, NT, T0, AL> {};
+
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL>
+__global__ void __launch_bounds__(WM * WN * 64)
+gemm_mfma_kernel(GemmArgs p)
+{
+    constexpr int NT = WM * WN * 64;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;          // 32x32 tiles per wave
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    half_t *As = reinterpret_cast<half_t *>(smem_raw);            // [2][BM*BK]
+    half_t *Bs = As + 2 * BM * BK;                                // [2][BN*BK]
+
+    // XCD-aware numbering: dispatch order i lands on XCD i % 8; give each XCD a contiguous
+    // band of the tile sequence, and walk tiles m-fastest so one weight panel is shared
+    const int nb = gridDim.x;
+    int bid = blockIdx.x;
+    {
+        const int per = nb >> 3, rem = nb & 7;
+        const int xcd = bid & 7, idx = bid >> 3;
+        bid = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    }
+    const int tm = bid % p.tiles_m, tn = bid / p.tiles_m;
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    const int64_t bz = blockIdx.z;
+    const half_t *A = p.A + bz * p.sa;
+    const half_t *B = p.B + bz * p.sb;
+    half_t *C = p.C + bz * p.sc;
+
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int wm = wid % WM, wn = wid / WM;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    // when both operands are strided they use disjoint halves of the block
+    Loader<TA, BM, NT, 0, AL> la;
+    Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL> lb;
+
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;
+    if (p.tri == 1 && n0 > m0 + BM - 1) return;                   // uniform for the block
+    if (p.tri == 2) nk = min(nk, (int)((m0 + BM + BK - 1) / BK));
+    if (p.tri == 3) kt0 = (int)(m0 / BK);
+    la.load(A, p.lda, m0, p.M, (int64_t)kt0 * BK, p.K);
+    lb.load(B, p.ldb, n0, p.N, (int64_t)kt0 * BK, p.K);
+    la.store(As + (kt0 & 1) * BM * BK);
+    lb.store(Bs + (kt0 & 1) * BN * BK);
+    __syncthreads();
+
+    // per-lane row offsets and swizzles of the operand fragments
+    const int ar0 = wm * (BM / WM) + l32, br0 = wn * (BN / WN) + l32;
+    const int asw = swz(ar0), bsw = swz(br0);                     // row + 32 i flips bit 2
+
+    for (int kt = kt0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {
+            la.load(A, p.lda, m0, p.M, (int64_t)(kt + 1) * BK, p.K);
+            lb.load(B, p.ldb, n0, p.N, (int64_t)(kt + 1) * BK, p.K);
+        }
+        const half_t *as = As + cur * BM * BK + ar0 * BK;
+        const half_t *bs = Bs + cur * BN * BK + br0 * BK;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            const int q = ks * 2 + lh;
+            half8_t af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                af[i] = *reinterpret_cast<const half8_t *>(
+                    as + i * 32 * BK + ((q ^ asw ^ ((i & 1) << 2)) << 3));
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                bf[j] = *reinterpret_cast<const half8_t *>(
+                    bs + j * 32 * BK + ((q ^ bsw ^ ((j & 1) << 2)) << 3));
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] =
+                        __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            la.store(As + (cur ^ 1) * BM * BK);
+            lb.store(Bs + (cur ^ 1) * BN * BK);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue through LDS (the operand buffers are free after the last barrier): a lane
+    // holds row m = .. + l32 and, per accumulator group q, the 4 consecutive columns
+    // n = .. + 8 q + 4 lh + {0..3}, i.e. 8 bytes in each of 32 different rows of C; staged as
+    // Cs[row][BN] (16-byte chunks swizzled by the row) the tile leaves as whole contiguous
+    // rows, 16 bytes per lane.  With beta the old C tile is staged the same way first, so
+    // alpha acc + beta C is still rounded to f16 exactly once.
+    half_t *Cs = reinterpret_cast<half_t *>(smem_raw);
+    constexpr int CPRC = BN / 8;                                  // 16-byte chunks per row
+    const bool has_beta = p.beta != 0.f;
+    if (has_beta) {
+        for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
+            const int row = c / CPRC, cc = c % CPRC;
+            const int64_t m = m0 + row, n = n0 + cc * 8;
+            const uint4 v = load8<AL>(C + m * p.ldc + n, m < p.M ? p.N - n : 0);
+            *reinterpret_cast<uint4 *>(Cs + row * BN + ((cc ^ (row & (CPRC - 1))) << 3)) = v;
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int row = wm * (BM / WM) + i * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int col = wn * (BN / WN) + j * 32 + q * 8 + lh * 4;
+                half_t *sp = Cs + row * BN + ((((col >> 3) ^ (row & (CPRC - 1))) << 3) | (col & 4));
+                half4_t o;
+                if (has_beta) {
+                    const half4_t old = *reinterpret_cast<const half4_t *>(sp);
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        o[r] = f2h(p.alpha * acc[i][j][q * 4 + r] + p.beta * h2f(old[r]));
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) o[r] = f2h(p.alpha * acc[i][j][q * 4 + r]);
+                }
+                *reinterpret_cast<half4_t *>(sp) = o;
+            }
+        }
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
+        const int row = c / CPRC, cc = c % CPRC;
+        const int64_t m = m0 + row, n = n0 + cc * 8;
+        if (m >= p.M || n >= p.N) continue;
+        const uint4 v = *reinterpret_cast<const uint4 *>(Cs + row * BN + ((cc ^ (row & (CPRC - 1))) << 3));
+        half_t *cp = C + m * p.ldc + n;
+        if (AL == 8) {
+            *reinterpret_cast<uint4 *>(cp) = v;
+        } else {
+            *reinterpret_cast<uint2 *>(cp) = make_uint2(v.x, v.y);
+            if (p.N - n > 4) *reinterpret_cast<uint2 *>(cp + 4) = make_uint2(v.z, v.w);
+        }
+    }
+}
+
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL>
+int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
+{
+    p.tiles_m = (int)((p.M + BM - 1) / BM);
+    p.tiles_n = (int)((p.N + BN - 1) / BN);
+    const size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(half_t);
+    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL>;
+    static bool attr_set = false;                 // one flag per instantiation
+    if (!attr_set) {
+        CACTI_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)smem));
+        attr_set = true;
+    }
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)nblk), block(WM * WN * 64);
+    hipLaunchKernelGGL(kern, grid, block, smem, st, p);
+    return launch_status("gemm_mfma");
+}
+
+template <bool TA, bool TB>
+int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
+{
+    if (align < 8) {                              // 8-byte aligned operands: one tile shape
+        return launch_cfg<TA, TB, 128, 128, 2, 2, 4>(p, nblk, st);
+    }
+    switch (tile) {
+        case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8>(p, nblk, st);
+        case 1: return launch_cfg<TA, TB, 256, 128, 4, 2, 8>(p, nblk, st);
+        case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8>(p, nblk, st);
+        default: return launch_cfg<TA, TB, 256, 256, 2, 2, 8>(p, nblk, st);
+    }
+}
+
+}  // namespace
+
+namespace cacti {
+
+// tile: 0 = 128x128 (4 waves), 1 = 256x128 (8 waves), 2 = 256x256 (8 waves), 3 = 256x256
+// (4 waves); -1 = pick by shape
+int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align, int tile,
+                     hipStream_t st)
+{
+    if (tile < 0) {
+        static int forced = -2;
+        if (forced == -2) {
+            const char *e = getenv("CACTI_GEMM_TILE");
+            forced = e ? atoi(e) : -1;
+        }
+        if (forced >= 0) {
+            tile = forced;
+        } else {
+            // measured on MI355X at the step's shapes: the double-transpose (TN) case is
+            // bound by its loaders and prefers the largest wave tile; the others prefer
+            // 128 x 128 (two blocks per CU) unless 256 x 256 tiles still fill the chip
+            // several times over
+            const int64_t big = ((p.M + 255) / 256) * ((p.N + 255) / 256) * nblk;
+            if (ta && !tb) tile = (p.M >= 256 && p.N >= 256) ? 3 : 0;
+            else if (!ta && tb) tile = big >= 768 ? 2 : 0;
+            else tile = 0;
+        }
+    }
+    if (!ta && !tb) return launch_tile<false, false>(tile, align, p, nblk, st);
+    if (!ta && tb) return launch_tile<false, true>(tile, align, p, nblk, st);
+    if (ta && !tb) return launch_tile<true, false>(tile, align, p, nblk, st);
+    return launch_tile<true, true>(tile, align, p, nblk, st);
+}
+
+}  // namespace cacti

@@ -321,9 +321,9 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
         TRY(ap(c, make_rope(g.H), {k, m->cos, m->sin}, &kr));
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.v}, &v));
-        TRY(ap(c, make_block_matmul(false, true, alpha, g.H), {qr, kr}, &s16));
+        TRY(ap(c, make_causal_scores(alpha, g.H), {qr, kr}, &s16));
         TRY(ap(c, make_causal_softmax(g.H), {s16}, &p16));
-        TRY(ap(c, make_block_matmul(false, false, 1.f, g.H), {p16, v}, &attn));
+        TRY(ap(c, make_causal_pv(g.H), {p16, v}, &attn));
         TRY(ap(c, make_matmul(false, true, 1.f), {attn, w.o}, &o));
         TRY(ap(c, make_add(), {stream, o}, &x1));
         TRY(ap(c, make_rms_norm(g.eps), {x1, w.post_norm}, &post));

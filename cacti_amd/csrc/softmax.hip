@@ -56,11 +56,14 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
         }
     sum = wave_sum(sum);
     half_t *orow = out + row * S;
+    // columns written: j <= i, then zeros to the next multiple of 256 (the triangular GEMMs
+    // read no further); the rest of the row is left untouched
+    const int wchunk = min(nchunk, ((i + 256) & ~255) >> 3);
     if (!BWD) {
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int ch = c * 64 + lane;
-            if (ch < nchunk) {
+            if (ch < wchunk) {
                 h8 o;
 #pragma unroll
                 for (int k = 0; k < 8; k++) o.v[k] = f2h(e[c][k] / sum);
@@ -89,7 +92,7 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
         for (int c = 0; c < CH; c++) {
             const int ch = c * 64 + lane;
             const int j0 = ch * 8;
-            if (ch < nchunk) {
+            if (ch < wchunk) {
                 h8 o;
 #pragma unroll
                 for (int k = 0; k < 8; k++) {

@@ -161,12 +161,21 @@ struct RmsNormSpec : ThunkSpec {
 // MatrixMulThunkSpec src/thunk/op.rs:4284-4368 (2-d) and BlockMatrixMulThunkSpec :4719-4918
 // on [R, H*C] tensors (the reference's [B,S,H,C] with B = 1, flattened) whose H per-head
 // blocks are addressed by stride; H = 0 means one plain matrix.
+//
+// `causal` marks the two products of causal attention (scores = a Q K^T whose upper
+// triangle the mask discards: CAUSAL_OUT; P V with P lower triangular: CAUSAL_A) so that
+// the discarded half is not computed; the adjoint rules carry the structure along
+// (dP = dO V^T is only needed below the diagonal; dV = P^T dO, dQ = a dS K, dK = a dS^T Q
+// have a triangular first operand).
+enum { CAUSAL_NONE = 0, CAUSAL_OUT = 1, CAUSAL_A = 2 };
 struct MatMulSpec : ThunkSpec {
     bool ta, tb;
     int64_t nblk;
     bool blocked;
     float alpha;
-    MatMulSpec(bool a, bool b, float al, int64_t h) : ta(a), tb(b), nblk(h), blocked(h > 0), alpha(al) {}
+    int causal;
+    MatMulSpec(bool a, bool b, float al, int64_t h, int cz = CAUSAL_NONE)
+        : ta(a), tb(b), nblk(h), blocked(h > 0), alpha(al), causal(cz) {}
     const char *name() const override { return blocked ? "block_matmul" : "matmul"; }
     int arity() const override { return 2; }
     struct Dims { int64_t H, M, N, K, lda, sa, ldb, sb, ldc, sc; };
@@ -205,9 +214,11 @@ struct MatMulSpec : ThunkSpec {
         Dims d;
         int rc = dims(aty, d);
         if (rc) return rc;
-        return cacti_hip_gemm_f16_strided_batched(ta, tb, d.H, d.M, d.N, d.K, alpha, a[0], d.lda,
-                                                  d.sa, a[1], d.ldb, d.sb, (acc & 1) ? 1.f : 0.f,
-                                                  o[0], d.ldc, d.sc, S(c));
+        const int tri = causal == CAUSAL_OUT ? 1 : causal == CAUSAL_A ? (ta ? 3 : 2) : 0;
+        return cacti_hip_gemm_f16_strided_batched_tri(ta, tb, d.H, d.M, d.N, d.K, alpha, a[0],
+                                                      d.lda, d.sa, a[1], d.ldb, d.sb,
+                                                      (acc & 1) ? 1.f : 0.f, o[0], d.ldc, d.sc, tri,
+                                                      S(c));
     }
     std::string key(const std::vector<CellType> &aty, uint32_t acc) const override
     {
@@ -219,9 +230,9 @@ struct MatMulSpec : ThunkSpec {
                  (acc & 1) ? ",acc" : "");
         return buf;
     }
-    std::unique_ptr<ThunkSpec> mm(bool x, bool y) const
+    std::unique_ptr<ThunkSpec> mm(bool x, bool y, int cz = CAUSAL_NONE) const
     {
-        return std::unique_ptr<ThunkSpec>(new MatMulSpec(x, y, alpha, nblk));
+        return std::unique_ptr<ThunkSpec>(new MatMulSpec(x, y, alpha, nblk, cz));
     }
     // the four transposition cases of pop_adj, src/thunk/op.rs:4335-4367 / :4882-4912:
     // arg_adj[1] first, then arg_adj[0], both carrying o_scale
@@ -229,6 +240,16 @@ struct MatMulSpec : ThunkSpec {
     {
         const CellPtr A = e.args[0], B = e.args[1], G = dy[0];
         int rc;
+        if (causal == CAUSAL_OUT) {              // C = a A B^T, only tril(C) is used: G = tril
+            TY_REQUIRE(!ta && tb, "causal scores product must be A B^T");
+            if ((rc = c.adj_add({B}, mm(true, false, CAUSAL_A), {G, A}))) return rc;   // G^T A
+            return c.adj_add({A}, mm(false, false, CAUSAL_A), {G, B});                  // G B
+        }
+        if (causal == CAUSAL_A) {                // C = A B with A = tril
+            TY_REQUIRE(!ta && !tb, "causal probability product must be A B");
+            if ((rc = c.adj_add({B}, mm(true, false, CAUSAL_A), {A, G}))) return rc;   // A^T G
+            return c.adj_add({A}, mm(false, true, CAUSAL_OUT), {G, B});                 // tril(G B^T)
+        }
         if (!ta && !tb) {
             if ((rc = c.adj_add({B}, mm(true, false), {A, G}))) return rc;      // A^T G
             return c.adj_add({A}, mm(false, true), {G, B});                      // G B^T
@@ -445,6 +466,14 @@ std::unique_ptr<ThunkSpec> make_matmul(bool ta, bool tb, float alpha)
 std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int64_t H)
 {
     return std::unique_ptr<ThunkSpec>(new MatMulSpec(ta, tb, alpha, H));
+}
+std::unique_ptr<ThunkSpec> make_causal_scores(float alpha, int64_t H)
+{
+    return std::unique_ptr<ThunkSpec>(new MatMulSpec(false, true, alpha, H, CAUSAL_OUT));
+}
+std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H)
+{
+    return std::unique_ptr<ThunkSpec>(new MatMulSpec(false, false, 1.f, H, CAUSAL_A));
 }
 std::unique_ptr<ThunkSpec> make_rope(int64_t H) { return std::unique_ptr<ThunkSpec>(new RopeSpec(H)); }
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H)

@@ -11,6 +11,9 @@ std::unique_ptr<ThunkSpec> make_embed();                              // (W, tok
 std::unique_ptr<ThunkSpec> make_rms_norm(float eps);                  // (x, w) -> y
 std::unique_ptr<ThunkSpec> make_matmul(bool ta, bool tb, float alpha);   // (a, b) -> c, 2-d
 std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int64_t H);   // [R,H*C]
+// the two block products of causal attention, computed on the lower triangle only
+std::unique_ptr<ThunkSpec> make_causal_scores(float alpha, int64_t H);   // (q, k) -> a q k^T
+std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H);                    // (p16, v) -> p16 v
 std::unique_ptr<ThunkSpec> make_rope(int64_t H);                      // (x [S,H*Dh], cos, sin) -> y
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H);            // (s16 [S,H*S]) -> p16
 std::unique_ptr<ThunkSpec> make_add();                                // (a, b) -> y

@@ -43,6 +43,8 @@ SIGNATURES = {
     "cacti_hip_gemm_f16": (ci, [ci, ci, i64, i64, i64, f32, vp, i64, vp, i64, f32, vp, i64, vp]),
     "cacti_hip_gemm_f16_strided_batched": (ci, [ci, ci, i64, i64, i64, i64, f32, vp, i64, i64, vp,
                                                 i64, i64, f32, vp, i64, i64, vp]),
+    "cacti_hip_gemm_f16_strided_batched_tri": (ci, [ci, ci, i64, i64, i64, i64, f32, vp, i64, i64,
+                                                    vp, i64, i64, f32, vp, i64, i64, ci, vp]),
     "cacti_hip_gemm_colmajor_f16": (ci, [ci, ci, ci, ci, ci, C.POINTER(f32), vp, ci, vp, ci,
                                          C.POINTER(f32), vp, ci, vp]),
     "cacti_hip_accumulate_1d_f32": (ci, [vp, vp, i64, vp]),

@@ -47,27 +47,32 @@ def gemm(a, b, ta=False, tb=False, alpha=1.0, beta=0.0, out=None):
     return out
 
 
-def gemm_strided_batched(ta, tb, nblk, M, N, K, alpha, a, lda, sa, b, ldb, sb, beta, c, ldc, sc):
-    ffi.call("cacti_hip_gemm_f16_strided_batched", int(ta), int(tb), nblk, M, N, K, alpha,
-             a.data_ptr(), lda, sa, b.data_ptr(), ldb, sb, beta, c.data_ptr(), ldc, sc, _stream())
+def gemm_strided_batched(ta, tb, nblk, M, N, K, alpha, a, lda, sa, b, ldb, sb, beta, c, ldc, sc,
+                         tri=0):
+    """tri: 0 dense; 1 only tril(C) wanted (rest unwritten); 2 A = tril; 3 A^T with A = tril."""
+    ffi.call("cacti_hip_gemm_f16_strided_batched_tri", int(ta), int(tb), nblk, M, N, K, alpha,
+             a.data_ptr(), lda, sa, b.data_ptr(), ldb, sb, beta, c.data_ptr(), ldc, sc, int(tri),
+             _stream())
     return c
 
 
-def block_matmul_qk(q, k, alpha):
-    """S16[i,h,j] = f16(alpha q[i,h,:] . k[j,h,:]) on [S,H,Dh] tensors (src/librarium/llama.rs:501)."""
+def block_matmul_qk(q, k, alpha, causal=False):
+    """S16[i,h,j] = f16(alpha q[i,h,:] . k[j,h,:]) on [S,H,Dh] tensors (src/librarium/llama.rs:501).
+    causal: only the tiles touching j <= i are computed; the rest of S16 is left unwritten."""
     S, H, Dh = q.shape
     s16 = torch.empty((S, H, S), dtype=F16, device=q.device)
     return gemm_strided_batched(False, True, H, S, S, Dh, alpha, q, H * Dh, Dh, k, H * Dh, Dh, 0.0,
-                                s16, H * S, S)
+                                s16, H * S, S, tri=1 if causal else 0)
 
 
-def block_matmul_pv(p16, v):
-    """O[i,h,:] = f16(sum_j p16[i,h,j] v[j,h,:]) (src/librarium/llama.rs:506)."""
+def block_matmul_pv(p16, v, causal=False):
+    """O[i,h,:] = f16(sum_j p16[i,h,j] v[j,h,:]) (src/librarium/llama.rs:506).
+    causal: p16 is lower triangular (as the causal softmax writes it)."""
     S, H, _ = p16.shape
     Dh = v.shape[2]
     o = torch.empty((S, H, Dh), dtype=F16, device=v.device)
     return gemm_strided_batched(False, False, H, S, Dh, S, 1.0, p16, H * S, S, v, H * Dh, Dh, 0.0, o,
-                                H * Dh, Dh)
+                                H * Dh, Dh, tri=2 if causal else 0)
 
 
 # ---------------------------------------------------------------- fused thunks
@@ -141,7 +146,9 @@ def causal_softmax_fwd(s16):
     _chk(s16)
     S, H, S2 = s16.shape
     assert S == S2
-    p = torch.empty_like(s16)
+    # the kernel writes j <= i and zeros only up to the next multiple of 256 columns:
+    # start from zeros so that dense consumers may read the whole row
+    p = torch.zeros_like(s16)
     ffi.call("cacti_hip_causal_softmax_fwd", S, H, s16.data_ptr(), p.data_ptr(), _stream())
     return p
 
@@ -149,7 +156,7 @@ def causal_softmax_fwd(s16):
 def causal_softmax_bwd(s16, dp16):
     _chk(s16), _chk(dp16)
     S, H, _ = s16.shape
-    ds = torch.empty_like(s16)
+    ds = torch.zeros_like(s16)
     ffi.call("cacti_hip_causal_softmax_bwd", S, H, s16.data_ptr(), dp16.data_ptr(), ds.data_ptr(),
              _stream())
     return ds

@@ -102,6 +102,23 @@ int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, 
                                        int64_t stride_b, float beta, void *C, int64_t ldc,
                                        int64_t stride_c, void *stream);
 
+/* The same with the triangular structure of causal attention made explicit, so that the
+ * half of each sequence x sequence product that the causal mask discards is never computed:
+ *   tri = 0  none (identical to the call above);
+ *   tri = 1  only the lower triangle (column <= row) of C is wanted (M == N): tiles wholly
+ *            above the diagonal are skipped and their part of C is left UNWRITTEN
+ *            (S = a Q K^T and dP = dO V^T feed the causal softmax, which never reads there);
+ *   tri = 2  A is lower triangular, not transposed (M == K): O = P V, dQ = a dS K;
+ *   tri = 3  A is lower triangular, transposed (M == K): dV = P^T dO, dK = a dS^T Q.
+ * For 2 and 3 the entries of A above the diagonal must be zero up to the next multiple of
+ * 256 columns (the causal softmax kernels write them so); beyond that A is not read.
+ * The reference computes these products densely (src/thunk/op.rs:5027-5471). */
+int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nblk, int64_t M, int64_t N,
+                                           int64_t K, float alpha, const void *A, int64_t lda,
+                                           int64_t stride_a, const void *B, int64_t ldb,
+                                           int64_t stride_b, float beta, void *C, int64_t ldc,
+                                           int64_t stride_c, int tri, void *stream);
+
 /* Column-major, cuBLAS-shaped form with host alpha/beta pointers, the call the
  * reference makes (cublas_gemm, cacti_gpu_cu_ffi/src/lib.rs:727-791; row-major
  * callers pass the operands swapped, src/thunk/op.rs:4469-4491).  tr_* = 0 (N)
@@ -164,7 +181,10 @@ int cacti_hip_silu_gate_bwd(int64_t n, const void *g, const void *u, const void 
  * (Cast, BlockTriElemAffineFutThunkSpec op.rs:4189-4278, InnerSoftmaxFutThunkSpec
  * :3257-3383), and its adjoint dS16 = f16(tril(T - (sum_j T) P')), T = P' * f32(dP16),
  * P' recomputed in fp32 (InnerSoftmaxPostAdjFutThunkSpec :3386-3457).
- * s16, p16, dp16, ds16: [S,H,S] f16 (row i, head, column j).  S % 8 == 0, S <= 16384. */
+ * s16, p16, dp16, ds16: [S,H,S] f16 (row i, head, column j).  S % 8 == 0, S <= 8192.
+ * Inputs are read only at j <= i; outputs are written at j <= i and as zeros from there to
+ * the next multiple of 256 columns (what the tri = 2 / 3 GEMMs read); entries further right
+ * are left untouched. */
 int cacti_hip_causal_softmax_fwd(int64_t S, int64_t H, const void *s16, void *p16, void *stream);
 int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const void *dp16,
                                  void *ds16, void *stream);

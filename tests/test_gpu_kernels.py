@@ -137,20 +137,35 @@ def test_silu_gate(ops, oracle, shape):
 
 
 # ---------------------------------------------------------------- causal softmax
-@pytest.mark.parametrize("S,H", [(128, 4), (512, 3), (8, 1), (2048, 2)])
+@pytest.mark.parametrize("S,H", [(128, 4), (512, 3), (8, 1), (2048, 2), (640, 2)])
 def test_causal_softmax(ops, oracle, S, H):
     say("causal_softmax", S, H)
     r = rng(500 + S)
     s16, dp = randn16(r, (S, H, S), 2.0), randn16(r, (S, H, S), 3.0)
+    # the kernels read j <= i only (entries above the diagonal may hold anything) and write
+    # j <= i plus zeros up to the next multiple of 256 columns; the rest stays untouched
+    i, j = np.arange(S)[:, None, None], np.arange(S)[None, None, :]
+    upper = np.broadcast_to(j > i, s16.shape)
+    written = np.broadcast_to(j < np.minimum(S, (i + 256) // 256 * 256), s16.shape)
+    junk = s16.copy(); junk[upper] = np.float16(np.nan)
     wp = oracle.causal_softmax_fwd(s16)
-    gp = host(ops.causal_softmax_fwd(dev(s16)))
-    assert_parity(gp, wp, "p16")
-    iu = np.triu_indices(S, 1)
-    assert np.all(gp[iu[0], :, iu[1]] == 0)
+    out = torch.full((S, H, S), 7.0, dtype=torch.float16, device="cuda")
+    from cacti_amd import ffi
+    dj = dev(junk)
+    ffi.call("cacti_hip_causal_softmax_fwd", S, H, dj.data_ptr(), out.data_ptr(),
+             torch.cuda.current_stream().cuda_stream)
+    gp = host(out)
+    assert np.all(gp[~written] == 7.0) and np.all(gp[written & upper] == 0)
+    assert_parity(np.where(written, gp, 0), wp, "p16")
     wds = oracle.causal_softmax_bwd(s16, dp)
-    gds = host(ops.causal_softmax_bwd(dev(s16), dev(dp)))
-    assert_parity(gds, wds, "ds16")
-    assert np.all(gds[iu[0], :, iu[1]] == 0)
+    djp = dp.copy(); djp[upper] = np.float16(np.nan)
+    ddp = dev(djp)
+    out = torch.full((S, H, S), 7.0, dtype=torch.float16, device="cuda")
+    ffi.call("cacti_hip_causal_softmax_bwd", S, H, dj.data_ptr(), ddp.data_ptr(), out.data_ptr(),
+             torch.cuda.current_stream().cuda_stream)
+    gds = host(out)
+    assert np.all(gds[~written] == 7.0) and np.all(gds[written & upper] == 0)
+    assert_parity(np.where(written, gds, 0), wds, "ds16")
 
 
 # ---------------------------------------------------------------- softmax cross-entropy
@@ -305,30 +320,34 @@ def test_gemm_colmajor_entry(ops, oracle):
 
 
 # ---------------------------------------------------------------- attention block
-@pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100)])
-def test_attention_block_via_thunks(ops, oracle, S, H, Dh):
-    """Q K^T -> causal softmax -> P V and the adjoint, composed as the reference stages them."""
-    say("attention", S, H, Dh)
+@pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100), (1024, 2, 100)])
+@pytest.mark.parametrize("tri", [False, True])
+def test_attention_block_via_thunks(ops, oracle, S, H, Dh, tri):
+    """Q K^T -> causal softmax -> P V and the adjoint, composed as the reference stages them;
+    tri: the products skip the half that the causal mask discards."""
+    say("attention", S, H, Dh, tri)
     r = rng(1000 + S)
     alpha = float(np.float32(1.0) / np.sqrt(np.float32(Dh)))
     q, k, v, dO = (randn16(r, (S, H, Dh)) for _ in range(4))
     ws16, wp16, wo = oracle.attention_fwd(q, k, v, alpha)
     dq_, dk_, dv_ = oracle.attention_bwd(q, k, v, dO, alpha)
     Q, K_, V_, DO = dev(q), dev(k), dev(v), dev(dO)
-    s16 = ops.block_matmul_qk(Q, K_, alpha)
-    assert_parity(host(s16), ws16, "s16")
+    low = np.broadcast_to(np.arange(S)[:, None, None] >= np.arange(S)[None, None, :], ws16.shape)
+    s16 = ops.block_matmul_qk(Q, K_, alpha, causal=tri)
+    assert_parity(np.where(low, host(s16), 0), np.where(low, ws16, 0), "s16")
     p16 = ops.causal_softmax_fwd(s16)
-    assert_parity(host(p16), wp16, "p16")
-    o = ops.block_matmul_pv(p16, V_)
+    assert_parity(np.where(low, host(p16), 0), wp16, "p16")
+    o = ops.block_matmul_pv(p16, V_, causal=tri)
     assert_parity(host(o), wo, "o")
     ld, lds = H * Dh, H * S
     dv = torch.empty_like(V_); dp = torch.empty_like(s16)
     dq = torch.empty_like(Q); dk = torch.empty_like(Q)
-    ops.gemm_strided_batched(True, False, H, S, Dh, S, 1.0, p16, lds, S, DO, ld, Dh, 0.0, dv, ld, Dh)
-    ops.gemm_strided_batched(False, True, H, S, S, Dh, 1.0, DO, ld, Dh, V_, ld, Dh, 0.0, dp, lds, S)
+    t1, t2, t3 = (1, 2, 3) if tri else (0, 0, 0)
+    ops.gemm_strided_batched(True, False, H, S, Dh, S, 1.0, p16, lds, S, DO, ld, Dh, 0.0, dv, ld, Dh, t3)
+    ops.gemm_strided_batched(False, True, H, S, S, Dh, 1.0, DO, ld, Dh, V_, ld, Dh, 0.0, dp, lds, S, t1)
     ds = ops.causal_softmax_bwd(s16, dp)
-    ops.gemm_strided_batched(True, False, H, S, Dh, S, alpha, ds, lds, S, Q, ld, Dh, 0.0, dk, ld, Dh)
-    ops.gemm_strided_batched(False, False, H, S, Dh, S, alpha, ds, lds, S, K_, ld, Dh, 0.0, dq, ld, Dh)
+    ops.gemm_strided_batched(True, False, H, S, Dh, S, alpha, ds, lds, S, Q, ld, Dh, 0.0, dk, ld, Dh, t3)
+    ops.gemm_strided_batched(False, False, H, S, Dh, S, alpha, ds, lds, S, K_, ld, Dh, 0.0, dq, ld, Dh, t2)
     assert_parity(host(dv), dv_, "dv")
     assert_parity(host(dq), dq_, "dq")
     assert_parity(host(dk), dk_, "dk")
