@@ -7,18 +7,24 @@
 // 32 x 32 accumulators fed by v_mfma_f32_32x32x16_f16.
 //
 // LDS layout (both operands): [row][64 k] = 128 bytes per row, no padding; the 16-byte
-// k-chunk q of row r sits at chunk position q ^ f(r), f(r) = ((r >> 3) ^ (r & 6)) & 7.
-// With this swizzle (a) the 16-byte MFMA operand reads of 16 consecutive rows, (b) the
+// k-chunk q of row r sits at chunk position q ^ f(r), f(r) = (r ^ (r >> 3)) & 7.
+// With this swizzle (a) the 16-byte MFMA operand reads of 8 consecutive rows, (b) the
 // 16-byte writes of a k-contiguous global row and (c) the writes of the register
-// transpose (8 rows apart per lane) all touch 16 distinct bank groups.
+// transpose (lanes 8 rows apart) each cover all eight 16-byte bank groups of a 128-byte
+// LDS line, and 16 consecutive rows also spread over both halves of a 256-byte line.
 //
 // An operand whose k index is not contiguous in memory (A^T, or B not transposed) is
 // loaded as 8 k-rows x 8 tile-rows per lane with fully coalesced 16-byte loads, transposed
 // in registers with 32 v_perm_b32, and written as 8 16-byte rows: the MFMA read path is
 // identical for NN / NT / TN / TT.
 //
-// Global loads of k-tile t+1 are issued before the MFMAs of tile t and stored into the
-// other LDS buffer afterwards: one barrier per 64-deep k tile.  Workgroups are numbered so
+// The main loop has no branch: every lane's global offsets (32-bit, relative to the tile
+// origin, clamped into the operand) are computed once, a k step only moves a uniform base
+// pointer.  Rows beyond the edge read a duplicate of the last rows (they only feed outputs
+// that are never stored); a k tail is zeroed with selects (KTAIL instantiations only).
+// With STAGES = 2 the global loads of k tile t+2 are issued before the MFMAs of tile t and
+// stored to LDS after the MFMAs of tile t+1 (two register stages + double-buffered LDS);
+// STAGES = 1 looks one tile ahead.  One barrier per k tile.  Workgroups are numbered so
 // that the 8 XCDs (round-robin dispatch) each walk a contiguous band of tiles and reuse
 // the operand panels in their own L2.
 #include "common.h"
@@ -30,18 +36,30 @@ namespace {
 
 constexpr int BK = 64;
 
-__device__ __forceinline__ int swz(int r) { return ((r >> 3) ^ (r & 6)) & 7; }
+__device__ __forceinline__ int swz(int r) { return ((r >> 3) ^ r) & 7; }
 
 // 16-byte chunk q (0..7) of tile row r
 __device__ __forceinline__ int lds_off(int r, int q) { return r * BK + ((q ^ swz(r)) << 3); }
 
-// ---- global -> registers -> LDS ---------------------------------------------
-// k-contiguous operand (memory [row][k]): chunk c -> row c / 8, k-chunk c % 8
-// 8 halves at p: one 16-byte load (AL = 8) or two 8-byte loads (AL = 4: operands that are
-// only 8-byte aligned, e.g. the per-head blocks of a head_dim-100 tensor); `n` = number of
-// valid halves from p on (a multiple of AL), the rest reads as zero
+__device__ __forceinline__ const half_t *at(const half_t *base, uint32_t byte_off)
+{
+    return reinterpret_cast<const half_t *>(reinterpret_cast<const char *>(base) + byte_off);
+}
+
+// 8 halves as one 16-byte load (AL = 8) or two 8-byte loads (AL = 4: operands that are only
+// 8-byte aligned, whose extents are multiples of 4); off1 = offset of the second half
 template <int AL>
-__device__ __forceinline__ uint4 load8(const half_t *p, int64_t n)
+__device__ __forceinline__ uint4 ld8(const half_t *base, uint32_t off0, uint32_t off1)
+{
+    if (AL == 8) return *reinterpret_cast<const uint4 *>(at(base, off0));
+    const uint2 lo = *reinterpret_cast<const uint2 *>(at(base, off0));
+    const uint2 hi = *reinterpret_cast<const uint2 *>(at(base, off1));
+    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+}
+
+// old C tile for the beta path: zero outside the matrix
+template <int AL>
+__device__ __forceinline__ uint4 load8_guarded(const half_t *p, int64_t n)
 {
     uint4 v = make_uint4(0, 0, 0, 0);
     if (AL == 8) {
@@ -61,24 +79,54 @@ __device__ __forceinline__ uint4 load8(const half_t *p, int64_t n)
     return v;
 }
 
-template <int ROWS, int NT, int AL>
+// ---- k-contiguous operand (memory [row][k]): chunk c -> row c / 8, k-chunk c % 8 ----------
+template <int ROWS, int NT, int AL, bool KTAIL>
 struct LoadKC {
     static constexpr int ITEMS = ROWS * 8;
     static constexpr int NL = (ITEMS + NT - 1) / NT;
-    uint4 st[NL];
-    __device__ __forceinline__ void load(const half_t *base, int64_t ld, int64_t row0, int64_t R,
-                                         int64_t k0, int64_t K)
+    uint32_t off[NL];              // byte offset of the chunk from (row0, k = 0)
+    int64_t ld, K;
+
+    // rows_left = R - row0 > 0
+    __device__ __forceinline__ void init(int64_t ld_, int64_t rows_left, int64_t K_)
     {
+        ld = ld_;
+        K = K_;
 #pragma unroll
         for (int it = 0; it < NL; it++) {
             const int c = threadIdx.x + it * NT;
-            const int row = c >> 3, kc = c & 7;
-            const int64_t gr = row0 + row, gk = k0 + kc * 8;
-            const bool on = (ITEMS % NT == 0 || c < ITEMS) && gr < R;
-            st[it] = load8<AL>(base + gr * ld + gk, on ? K - gk : 0);
+            int row = (c >> 3) % ROWS;
+            const int kc = c & 7;
+            if (row >= rows_left) row = (int)rows_left - 1;
+            off[it] = (uint32_t)((row * ld + kc * 8) * 2);
         }
     }
-    __device__ __forceinline__ void store(half_t *lds)
+    // origin = &op[row0][0]
+    __device__ __forceinline__ void load(uint4 *st, const half_t *origin, int64_t k0) const
+    {
+        const half_t *base = origin + k0;
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            if (!KTAIL) {
+                st[it] = ld8<AL>(base, off[it], off[it] + 8);
+            } else {
+                const int kc = (threadIdx.x + it * NT) & 7;
+                const int left = (int)(K - k0) - kc * 8;        // valid halves from this chunk on
+                // clamp both halves back into the row; zero what lies beyond K
+                const uint32_t back0 = left >= AL ? 0 : (uint32_t)(AL - left) * 2;
+                const uint32_t back1 = left >= 8 ? 0 : (uint32_t)(8 - (left > 4 ? left : 4)) * 2;
+                uint4 v = ld8<AL>(base, off[it] - back0, off[it] + 8 - back0 - back1);
+                if (AL == 8) {
+                    if (left <= 0) v = make_uint4(0, 0, 0, 0);
+                } else {
+                    if (left <= 0) { v.x = 0; v.y = 0; }
+                    if (left <= 4) { v.z = 0; v.w = 0; }
+                }
+                st[it] = v;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(const uint4 *st, half_t *lds) const
     {
 #pragma unroll
         for (int it = 0; it < NL; it++) {
@@ -88,49 +136,84 @@ struct LoadKC {
                 *reinterpret_cast<uint4 *>(lds + lds_off(row, kc)) = st[it];
         }
     }
+    static constexpr int NREG = NL;
 };
 
-// k-strided operand (memory [k][row]): item c -> row chunk c % (ROWS/8), k group c / (ROWS/8);
-// an item is 8 k x 8 rows.  T0 = first thread that takes part (lets two strided operands
-// use disjoint halves of the block).
-template <int ROWS, int NT, int T0, int AL>
+// ---- k-strided operand (memory [k][row]): item c -> row chunk c % (ROWS/8), k group
+// c / (ROWS/8); an item is 8 k x 8 rows.  T0 = first thread that takes part (lets two
+// strided operands use disjoint halves of the block).
+template <int ROWS, int NT, int T0, int AL, bool KTAIL>
 struct LoadKS {
     static constexpr int RC = ROWS / 8;
     static constexpr int ITEMS = RC * 8;
     static constexpr int NTH = NT - T0 >= ITEMS ? ITEMS : NT;      // threads taking part
     static constexpr int TB = NT - T0 >= ITEMS ? T0 : 0;
     static constexpr int NL = (ITEMS + NTH - 1) / NTH;
-    uint4 st[NL][8];
-    __device__ __forceinline__ bool mine(int it, int &c) const
+    uint32_t off[NL], off1[NL];    // byte offset of the item's first k row from (k = 0, row0)
+    uint32_t ldb2;                 // ld in bytes
+    int64_t ld, K;
+
+    __device__ __forceinline__ int item(int it) const
+    {
+        const int t = ((int)threadIdx.x - TB + NT) % NT;           // non-members wrap harmlessly
+        return (t + it * NTH) % ITEMS;
+    }
+    __device__ __forceinline__ bool mine(int it) const
     {
         const int t = (int)threadIdx.x - TB;
-        c = t + it * NTH;
-        return t >= 0 && t < NTH && c < ITEMS;
+        return t >= 0 && t < NTH && t + it * NTH < ITEMS;
     }
-    __device__ __forceinline__ void load(const half_t *base, int64_t ld, int64_t row0, int64_t R,
-                                         int64_t k0, int64_t K)
+    __device__ __forceinline__ void init(int64_t ld_, int64_t rows_left, int64_t K_)
     {
+        ld = ld_;
+        K = K_;
+        ldb2 = (uint32_t)(ld_ * 2);
 #pragma unroll
         for (int it = 0; it < NL; it++) {
-            int c;
-            const bool on = mine(it, c);
+            const int c = item(it);
             const int rc = c % RC, kq = c / RC;
-            const int64_t gr = row0 + rc * 8;
+            // clamp the row chunk(s) into the operand (rows_left is a multiple of AL)
+            int r0 = rc * 8, r1 = rc * 8 + 4;
+            if (AL == 8) {
+                if (r0 > rows_left - 8) r0 = (int)rows_left - 8;
+            } else {
+                if (r0 > rows_left - 4) r0 = (int)rows_left - 4;
+                if (r1 > rows_left - 4) r1 = (int)rows_left - 4;
+            }
+            off[it] = (uint32_t)(((int64_t)kq * 8 * ld + r0) * 2);
+            off1[it] = (uint32_t)(((int64_t)kq * 8 * ld + r1) * 2);
+        }
+    }
+    // origin = &op[0][row0]
+    __device__ __forceinline__ void load(uint4 *st, const half_t *origin, int64_t k0) const
+    {
+        const half_t *base = origin + k0 * ld;
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            if (!mine(it)) continue;          // whole wavefronts: a uniform skip, not a lane mask
+            const int kq = item(it) / RC;
 #pragma unroll
             for (int kk = 0; kk < 8; kk++) {
-                const int64_t gk = k0 + kq * 8 + kk;
-                st[it][kk] = load8<AL>(base + gk * ld + gr, (on && gk < K) ? R - gr : 0);
+                if (!KTAIL) {
+                    st[it * 8 + kk] = ld8<AL>(base, off[it] + kk * ldb2, off1[it] + kk * ldb2);
+                } else {
+                    const int left = (int)(K - k0) - (kq * 8 + kk);   // > 0 iff this k row exists
+                    const uint32_t back = left > 0 ? 0 : (uint32_t)(1 - left) * ldb2;
+                    uint4 v = ld8<AL>(base, off[it] + kk * ldb2 - back, off1[it] + kk * ldb2 - back);
+                    if (left <= 0) v = make_uint4(0, 0, 0, 0);
+                    st[it * 8 + kk] = v;
+                }
             }
         }
     }
-    __device__ __forceinline__ void store(half_t *lds)
+    __device__ __forceinline__ void store(const uint4 *st, half_t *lds) const
     {
 #pragma unroll
         for (int it = 0; it < NL; it++) {
-            int c;
-            if (!mine(it, c)) continue;
+            if (!mine(it)) continue;
+            const int c = item(it);
             const int rc = c % RC, kq = c / RC;
-            const uint32_t *w = reinterpret_cast<const uint32_t *>(&st[it][0]);   // [kk][4 words]
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(st + it * 8);   // [kk][4 words]
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 // row j of the 8 x 8 block: halves (k = 0..7) = word j/2, half j%2 of each k row
@@ -144,16 +227,21 @@ struct LoadKS {
             }
         }
     }
+    static constexpr int NREG = NL * 8;
 };
 
-template <bool STRIDED, int ROWS, int NT, int T0, int AL> struct Loader;
-template <int ROWS, int NT, int T0, int AL>
-struct Loader<false, ROWS, NT, T0, AL> : LoadKC<ROWS, NT, AL> {};
-template <int ROWS, int NT, int T0, int AL>
-struct Loader<true, ROWS, NT, T0, AL> : LoadKS<ROWS, NT, T0, AL> {};
+template <bool STRIDED, int ROWS, int NT, int T0, int AL, bool KTAIL> struct Loader;
+template <int ROWS, int NT, int T0, int AL, bool KTAIL>
+struct Loader<false, ROWS, NT, T0, AL, KTAIL> : LoadKC<ROWS, NT, AL, KTAIL> {};
+template <int ROWS, int NT, int T0, int AL, bool KTAIL>
+struct Loader<true, ROWS, NT, T0, AL, KTAIL> : LoadKS<ROWS, NT, T0, AL, KTAIL> {};
 
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL>
-__global__ void __launch_bounds__(WM * WN * 64)
+// waves per SIMD the register allocation must leave room for: two 128 x 128 blocks (or one
+// 8-wave block) per CU, one 4-wave 256 x 256 block
+constexpr int min_waves(int bm, int bn, int nwaves) { return (bm * bn <= 128 * 128 || nwaves == 8) ? 2 : 1; }
+
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
+__global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN))
 gemm_mfma_kernel(GemmArgs p)
 {
     constexpr int NT = WM * WN * 64;
@@ -173,18 +261,32 @@ gemm_mfma_kernel(GemmArgs p)
     }
     const int tm = bid % p.tiles_m, tn = bid / p.tiles_m;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+
+    int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;
+    if (p.tri == 1 && n0 > m0 + BM - 1) return;                   // uniform for the block
+    if (p.tri == 2) nk = min(nk, (int)((m0 + BM + BK - 1) / BK));
+    if (p.tri == 3) kt0 = (int)(m0 / BK);
+
     const int64_t bz = blockIdx.z;
     const half_t *A = p.A + bz * p.sa;
     const half_t *B = p.B + bz * p.sb;
     half_t *C = p.C + bz * p.sc;
+    // tile origins: &op[row0][0] for a k-contiguous operand, &op[0][row0] for a strided one
+    const half_t *Ao = TA ? A + m0 : A + m0 * p.lda;
+    const half_t *Bo = TB ? B + n0 * p.ldb : B + n0;
 
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int wm = wid % WM, wn = wid / WM;
     const int l32 = lane & 31, lh = lane >> 5;
 
     // when both operands are strided they use disjoint halves of the block
-    Loader<TA, BM, NT, 0, AL> la;
-    Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL> lb;
+    typedef Loader<TA, BM, NT, 0, AL, KTAIL> LA;
+    typedef Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL, KTAIL> LB;
+    LA la;
+    LB lb;
+    la.init(p.lda, p.M - m0, p.K);
+    lb.init(p.ldb, p.N - n0, p.K);
+    uint4 ra[STAGES][LA::NREG], rb[STAGES][LB::NREG];
 
     float16_t acc[TM][TN];
 #pragma unroll
@@ -194,26 +296,15 @@ gemm_mfma_kernel(GemmArgs p)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;
-    if (p.tri == 1 && n0 > m0 + BM - 1) return;                   // uniform for the block
-    if (p.tri == 2) nk = min(nk, (int)((m0 + BM + BK - 1) / BK));
-    if (p.tri == 3) kt0 = (int)(m0 / BK);
-    la.load(A, p.lda, m0, p.M, (int64_t)kt0 * BK, p.K);
-    lb.load(B, p.ldb, n0, p.N, (int64_t)kt0 * BK, p.K);
-    la.store(As + (kt0 & 1) * BM * BK);
-    lb.store(Bs + (kt0 & 1) * BN * BK);
-    __syncthreads();
-
     // per-lane row offsets and swizzles of the operand fragments
     const int ar0 = wm * (BM / WM) + l32, br0 = wn * (BN / WN) + l32;
     const int asw = swz(ar0), bsw = swz(br0);                     // row + 32 i flips bit 2
 
-    for (int kt = kt0; kt < nk; kt++) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {
-            la.load(A, p.lda, m0, p.M, (int64_t)(kt + 1) * BK, p.K);
-            lb.load(B, p.ldb, n0, p.N, (int64_t)(kt + 1) * BK, p.K);
-        }
+    // loads past the last tile re-read the last one; their LDS copy is never used
+    auto tile_k = [&](int kt) __attribute__((always_inline)) {
+        return (int64_t)(kt < nk ? kt : nk - 1) * BK;
+    };
+    auto compute = [&](int cur) __attribute__((always_inline)) {
         const half_t *as = As + cur * BM * BK + ar0 * BK;
         const half_t *bs = Bs + cur * BN * BK + br0 * BK;
 #pragma unroll
@@ -235,11 +326,45 @@ gemm_mfma_kernel(GemmArgs p)
                     acc[i][j] =
                         __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) {
-            la.store(As + (cur ^ 1) * BM * BK);
-            lb.store(Bs + (cur ^ 1) * BN * BK);
-        }
+    };
+
+    if (STAGES == 2) {
+        la.load(ra[0], Ao, tile_k(kt0));
+        lb.load(rb[0], Bo, tile_k(kt0));
+        la.load(ra[STAGES - 1], Ao, tile_k(kt0 + 1));
+        lb.load(rb[STAGES - 1], Bo, tile_k(kt0 + 1));
+        la.store(ra[0], As + (kt0 & 1) * BM * BK);
+        lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
         __syncthreads();
+        for (int kt = kt0; kt < nk; kt += 2) {
+            la.load(ra[0], Ao, tile_k(kt + 2));
+            lb.load(rb[0], Bo, tile_k(kt + 2));
+            compute(kt & 1);
+            la.store(ra[STAGES - 1], As + ((kt + 1) & 1) * BM * BK);
+            lb.store(rb[STAGES - 1], Bs + ((kt + 1) & 1) * BN * BK);
+            __syncthreads();
+            if (kt + 1 >= nk) break;
+            la.load(ra[STAGES - 1], Ao, tile_k(kt + 3));
+            lb.load(rb[STAGES - 1], Bo, tile_k(kt + 3));
+            compute((kt + 1) & 1);
+            la.store(ra[0], As + (kt & 1) * BM * BK);
+            lb.store(rb[0], Bs + (kt & 1) * BN * BK);
+            __syncthreads();
+        }
+    } else {
+        la.load(ra[0], Ao, tile_k(kt0));
+        lb.load(rb[0], Bo, tile_k(kt0));
+        la.store(ra[0], As + (kt0 & 1) * BM * BK);
+        lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
+        __syncthreads();
+        for (int kt = kt0; kt < nk; kt++) {
+            la.load(ra[0], Ao, tile_k(kt + 1));
+            lb.load(rb[0], Bo, tile_k(kt + 1));
+            compute(kt & 1);
+            la.store(ra[0], As + ((kt + 1) & 1) * BM * BK);
+            lb.store(rb[0], Bs + ((kt + 1) & 1) * BN * BK);
+            __syncthreads();
+        }
     }
 
     // Epilogue through LDS (the operand buffers are free after the last barrier): a lane
@@ -255,7 +380,7 @@ gemm_mfma_kernel(GemmArgs p)
         for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
             const int row = c / CPRC, cc = c % CPRC;
             const int64_t m = m0 + row, n = n0 + cc * 8;
-            const uint4 v = load8<AL>(C + m * p.ldc + n, m < p.M ? p.N - n : 0);
+            const uint4 v = load8_guarded<AL>(C + m * p.ldc + n, m < p.M ? p.N - n : 0);
             *reinterpret_cast<uint4 *>(Cs + row * BN + ((cc ^ (row & (CPRC - 1))) << 3)) = v;
         }
         __syncthreads();
@@ -299,13 +424,13 @@ gemm_mfma_kernel(GemmArgs p)
     }
 }
 
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL>
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
 int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 {
     p.tiles_m = (int)((p.M + BM - 1) / BM);
     p.tiles_n = (int)((p.N + BN - 1) / BN);
     const size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(half_t);
-    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL>;
+    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES>;
     static bool attr_set = false;                 // one flag per instantiation
     if (!attr_set) {
         CACTI_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -317,17 +442,23 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
     return launch_status("gemm_mfma");
 }
 
+// register stages per layout: a strided operand stages 8 x 16 bytes per lane, so two
+// stages only pay where the accumulators leave room
 template <bool TA, bool TB>
 int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
 {
+    constexpr int S0 = (!TA && TB) ? 2 : 1;       // 128 x 128: two stages only if no operand is strided
+    const bool ktail = (p.K % BK) != 0;
     if (align < 8) {                              // 8-byte aligned operands: one tile shape
-        return launch_cfg<TA, TB, 128, 128, 2, 2, 4>(p, nblk, st);
+        return ktail ? launch_cfg<TA, TB, 128, 128, 2, 2, 4, true, 1>(p, nblk, st)
+                     : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, 1>(p, nblk, st);
     }
+    if (ktail) return launch_cfg<TA, TB, 128, 128, 2, 2, 8, true, 1>(p, nblk, st);
     switch (tile) {
-        case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8>(p, nblk, st);
-        case 1: return launch_cfg<TA, TB, 256, 128, 4, 2, 8>(p, nblk, st);
-        case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8>(p, nblk, st);
-        default: return launch_cfg<TA, TB, 256, 256, 2, 2, 8>(p, nblk, st);
+        case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8, false, S0>(p, nblk, st);
+        case 1: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 1>(p, nblk, st);
+        case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1>(p, nblk, st);
+        default: return launch_cfg<TA, TB, 256, 256, 2, 2, 8, false, 1>(p, nblk, st);
     }
 }
 
@@ -349,14 +480,11 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
         if (forced >= 0) {
             tile = forced;
         } else {
-            // measured on MI355X at the step's shapes: the double-transpose (TN) case is
-            // bound by its loaders and prefers the largest wave tile; the others prefer
-            // 128 x 128 (two blocks per CU) unless 256 x 256 tiles still fill the chip
-            // several times over
+            // measured on MI355X at the step's shapes: 128 x 128 (two blocks per CU) wins
+            // everywhere except the k-contiguous (NT) case when 256 x 256 tiles still fill
+            // the chip several times over (the LM-head forward)
             const int64_t big = ((p.M + 255) / 256) * ((p.N + 255) / 256) * nblk;
-            if (ta && !tb) tile = (p.M >= 256 && p.N >= 256) ? 3 : 0;
-            else if (!ta && tb) tile = big >= 768 ? 2 : 0;
-            else tile = 0;
+            tile = (!ta && tb && big >= 768) ? 3 : 0;
         }
     }
     if (!ta && !tb) return launch_tile<false, false>(tile, align, p, nblk, st);
