@@ -93,7 +93,7 @@ CACTI_API int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out)
     return 0;
 }
 
-CACTI_API int cacti_ctx_sync(cacti_ctx *ctx) { return ctx->c.sync(); }
+CACTI_API int cacti_ctx_sync(cacti_ctx *ctx) { return ctx->c.check_status(); }
 CACTI_API void *cacti_ctx_stream(cacti_ctx *ctx) { return (void *)ctx->c.stream(); }
 
 CACTI_API int cacti_ctx_set_timing(cacti_ctx *ctx, int on)
@@ -377,7 +377,10 @@ CACTI_API int cacti_llama_step(cacti_llama *m, const uint16_t *tok, const uint16
         else if (y == m->in_loss_scale) TRY(c.resume_put(y, loss_scale, S * 4));
         else CACTI_REQUIRE(false, CACTI_E_STATE, "llama_step: unexpected yield of cell %d", y);
     }
+    // Without a loss read-back the call returns with the cycle still running on the stream
+    // (the next cycle's staging then overlaps it); an out-of-range token id is reported by
+    // the next synchronizing call (cacti_ctx_sync, or a step that reads the loss).
+    if (!loss_out) return 0;
     TRY(c.check_status());
-    if (loss_out) TRY(c.cell_get(m->out_loss, loss_out, S * 4));
-    return c.sync();
+    return c.cell_get(m->out_loss, loss_out, S * 4);
 }

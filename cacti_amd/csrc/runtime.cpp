@@ -176,8 +176,24 @@ int Ctx::host_alloc(Cell &c)
     return 0;
 }
 
+// wait until no in-flight copy reads or writes the cell's host buffer
+static void host_quiesce(Cell &c)
+{
+    if (c.h_busy) hipEventSynchronize(c.h_busy);
+}
+static void host_mark_busy(Cell &c, hipStream_t st)
+{
+    if (!c.h_busy) hipEventCreateWithFlags(&c.h_busy, hipEventDisableTiming);
+    hipEventRecord(c.h_busy, st);
+}
+
 void Ctx::host_free(Cell &c)
 {
+    if (c.h_busy) {
+        hipEventSynchronize(c.h_busy);
+        hipEventDestroy(c.h_busy);
+        c.h_busy = nullptr;
+    }
     if (!c.hptr) return;
     if (host_pagelocked_) hipHostFree(c.hptr); else free(c.hptr);
     host_bytes_ -= std::max<size_t>(c.ty.bytes(), 1);
@@ -193,11 +209,7 @@ int Ctx::cell_free_all(CellPtr ci)
         c.voff = kNoOffset;
     }
     c.v_valid = false;
-    if (c.hptr) {
-        // a host buffer may still be the source or target of an in-flight copy
-        if (stream_) hipStreamSynchronize(stream_);
-        host_free(c);
-    }
+    if (c.hptr || c.h_busy) host_free(c);     // waits for in-flight copies of this cell only
     return 0;
 }
 
@@ -208,7 +220,7 @@ int Ctx::cell_put(CellPtr ci, const void *host, size_t bytes)
     CACTI_REQUIRE(bytes == c.ty.bytes(), CACTI_E_INVALID, "cell_put: %zu bytes given, cell %s has %zu",
                   bytes, c.name.c_str(), c.ty.bytes());
     // an earlier upload from this host buffer may still be in flight
-    CACTI_HIP(hipStreamSynchronize(stream_));
+    host_quiesce(c);
     int rc = host_alloc(c);
     if (rc) return rc;
     memcpy(c.hptr, host, bytes);
@@ -230,7 +242,7 @@ int Ctx::cell_get(CellPtr ci, void *host, size_t bytes)
         return 0;
     }
     CACTI_REQUIRE(c.h_valid, CACTI_E_STATE, "cell_get: cell %s holds no value", c.name.c_str());
-    CACTI_HIP(hipStreamSynchronize(stream_));
+    host_quiesce(c);
     memcpy(host, c.hptr, bytes);
     return 0;
 }
@@ -247,6 +259,7 @@ int Ctx::evict(CellPtr ci)
         CACTI_HIP(hipMemcpyAsync(c.hptr, dev_ptr(c.voff), c.ty.bytes(), hipMemcpyDeviceToHost,
                                  stream_));
         if (!host_pagelocked_) CACTI_HIP(hipStreamSynchronize(stream_));
+        host_mark_busy(c, stream_);
         c.h_valid = true;
         bytes_d2h_ += c.ty.bytes();
     }
@@ -312,6 +325,7 @@ int Ctx::ensure_vmem(CellPtr ci, bool need_value)
                       d.name.c_str());
         CACTI_HIP(hipMemcpyAsync(dev_ptr(d.voff), d.hptr, d.ty.bytes(), hipMemcpyHostToDevice,
                                  stream_));
+        host_mark_busy(d, stream_);
         d.v_valid = true;
         n_upload_++;
         bytes_h2d_ += d.ty.bytes();

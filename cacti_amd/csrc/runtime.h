@@ -75,6 +75,7 @@ struct Cell {
     void *hptr = nullptr;    // Mem replica (host)
     bool v_valid = false, h_valid = false;
     int pin = 0;
+    hipEvent_t h_busy = nullptr;   // recorded after the last copy that touches hptr
 };
 
 struct Stats {

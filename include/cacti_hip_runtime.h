@@ -49,7 +49,7 @@ typedef struct {
 int cacti_ctx_create(cacti_ctx **ctx, int dev, size_t pool_bytes, int host_pagelocked);
 int cacti_ctx_destroy(cacti_ctx *ctx);
 int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out);
-int cacti_ctx_sync(cacti_ctx *ctx);
+int cacti_ctx_sync(cacti_ctx *ctx);      /* stream sync + token-range status check */
 void *cacti_ctx_stream(cacti_ctx *ctx);                 /* the hipStream_t all work runs on */
 /* per-thunk device times (CACTI_DEBUG_TIMING, src/ctx.rs:114-133).  mode 1 syncs after
  * every thunk; mode 2 records a HIP event pair around every launch without syncing and
@@ -104,7 +104,10 @@ int cacti_llama_io_cells(cacti_llama *model, int *tok, int *lm_tok, int *loss_sc
  * Llama::apply, and (want_grad) sink.add(loss, loss_scale) + vadd_vjp over all parameters
  * (examples/open_llama_3b_train.rs:350-389). */
 int cacti_llama_stage(cacti_llama *model, int want_prob, int want_grad);
-/* reset + stage + compile + resume/resume_put + sync; loss_out [S] f32 may be NULL. */
+/* reset + stage + compile + resume/resume_put.  With loss_out [S] f32 the call syncs, checks
+ * the token-range status and copies the loss back; with loss_out = NULL it returns while the
+ * cycle still runs on the stream (results and a CACTI_E_INDEX status are then observed by the
+ * next synchronizing call: cacti_ctx_sync, cacti_cell_get, cacti_llama_grad_get). */
 int cacti_llama_step(cacti_llama *model, const uint16_t *tok, const uint16_t *lm_tok,
                      const float *loss_scale, int want_prob, int want_grad, float *loss_out);
 
