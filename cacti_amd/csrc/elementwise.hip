@@ -110,6 +110,63 @@ rope_kernel(int64_t S, int H, int Dh, int tok_per_block, const half_t *__restric
 }
 
 // ---------------------------------------------------------------------------
+// RoPE without LDS, for head dimensions that are multiples of 4 (Dh/2 even, so an aligned
+// pair of halves never straddles the middle of a head).  A lane owns the pair (d, d+1) of the
+// left half AND its partner pair (d + Dh/2, ..) of the right half: it reads both, then writes
+// both, so no lane reads what another lane writes and the kernel may run in place.  All
+// accesses are 4 bytes per lane and consecutive across lanes.
+template <bool BWD>
+__global__ void __launch_bounds__(kThreads)
+rope_pair_kernel(int64_t S, int H, int Dh, const half_t *__restrict__ in,
+                 const half_t *__restrict__ cos16, const half_t *__restrict__ sin16, half_t *out,
+                 int acc)
+{
+    const int hf = Dh / 2, pph = hf / 2;            // pairs per half head
+    const int64_t per_tok = (int64_t)H * pph, total = S * per_tok;
+    for (int64_t it = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; it < total;
+         it += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t s = it / per_tok;
+        const int r = (int)(it - s * per_tok);
+        const int h = r / pph, d = (r - h * pph) * 2;
+        const int64_t eL = (s * H + h) * Dh + d, eR = eL + hf;
+        const int64_t tL = s * Dh + d, tR = tL + hf;
+        const half2_t xL = *reinterpret_cast<const half2_t *>(in + eL);
+        const half2_t xR = *reinterpret_cast<const half2_t *>(in + eR);
+        const half2_t cL = *reinterpret_cast<const half2_t *>(cos16 + tL);
+        const half2_t cR = *reinterpret_cast<const half2_t *>(cos16 + tR);
+        const half2_t sL = *reinterpret_cast<const half2_t *>(sin16 + tL);
+        const half2_t sR = *reinterpret_cast<const half2_t *>(sin16 + tR);
+        half2_t oL, oR, qL, qR;
+        if (BWD && acc) {
+            qL = *reinterpret_cast<const half2_t *>(out + eL);
+            qR = *reinterpret_cast<const half2_t *>(out + eR);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const float xl = h2f(xL[i]), xr = h2f(xR[i]);
+            if (!BWD) {
+                // a + f16(-x_r sin) == a - f16(x_r sin): rounding is symmetric in sign
+                oL[i] = f2h(rnd16(xl * h2f(cL[i])) - rnd16(xr * h2f(sL[i])));
+                oR[i] = f2h(rnd16(xr * h2f(cR[i])) + rnd16(xl * h2f(sR[i])));
+            } else {
+                const float dl = rnd16(xr * h2f(sR[i]));        // drx_r = f16(dy sin) at d + Dh/2
+                const float tl = rnd16(xl * h2f(sL[i]));        // drx_l; enters dx_r negated
+                const float c2l = rnd16(xl * h2f(cL[i])), c2r = rnd16(xr * h2f(cR[i]));
+                if (acc) {
+                    oL[i] = f2h(rnd16(h2f(qL[i]) + dl) + c2l);
+                    oR[i] = f2h(rnd16(h2f(qR[i]) - tl) + c2r);
+                } else {
+                    oL[i] = f2h(dl + c2l);
+                    oR[i] = f2h(c2r - tl);
+                }
+            }
+        }
+        *reinterpret_cast<half2_t *>(out + eL) = oL;
+        *reinterpret_cast<half2_t *>(out + eR) = oR;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // SiLU gate.  forward: y = f16(g / (1 + exp(-g))); h = f16(y u).
 __global__ void __launch_bounds__(kThreads)
 silu_gate_fwd_kernel(int64_t nchunk, const half_t *__restrict__ g, const half_t *__restrict__ u,
@@ -287,6 +344,19 @@ static int rope_launch(bool bwd, int64_t S, int64_t H, int64_t Dh, const void *i
     CACTI_REQUIRE(aligned(in, 16) && aligned(out, 16), CACTI_E_INVALID,
                   "rope: tensors must be 16-byte aligned");
     const int64_t row = H * Dh;
+    if (Dh % 4 == 0 && aligned(c, 4) && aligned(s, 4)) {
+        const int64_t items = S * H * (Dh / 4);
+        const int grid = grid_for(items, kThreads, 4096);
+        if (bwd)
+            hipLaunchKernelGGL(rope_pair_kernel<true>, dim3(grid), dim3(kThreads), 0,
+                               (hipStream_t)stream, S, (int)H, (int)Dh, (const half_t *)in,
+                               (const half_t *)c, (const half_t *)s, (half_t *)out, acc);
+        else
+            hipLaunchKernelGGL(rope_pair_kernel<false>, dim3(grid), dim3(kThreads), 0,
+                               (hipStream_t)stream, S, (int)H, (int)Dh, (const half_t *)in,
+                               (const half_t *)c, (const half_t *)s, (half_t *)out, 0);
+        return launch_status("rope");
+    }
     int tok = 2;
     size_t smem = (size_t)tok * (row + 2 * Dh) * 2;
     if (smem > 64 * 1024) {

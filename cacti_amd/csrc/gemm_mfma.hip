@@ -251,7 +251,7 @@ gemm_mfma_kernel(GemmArgs p)
     half_t *Bs = As + 2 * BM * BK;                                // [2][BN*BK]
 
     // XCD-aware numbering: dispatch order i lands on XCD i % 8; give each XCD a contiguous
-    // band of the tile sequence, and walk tiles m-fastest so one weight panel is shared
+    // band of the tile sequence
     const int nb = gridDim.x;
     int bid = blockIdx.x;
     {
@@ -259,7 +259,14 @@ gemm_mfma_kernel(GemmArgs p)
         const int xcd = bid & 7, idx = bid >> 3;
         bid = xcd * per + (xcd < rem ? xcd : rem) + idx;
     }
-    const int tm = bid % p.tiles_m, tn = bid / p.tiles_m;
+    // within the band, tiles are walked in groups of 8 tile rows x all tile columns, row
+    // fastest: the ~64 blocks resident on an XCD then form an 8 x 8 patch of C and each
+    // operand panel fetched into its L2 is shared by 8 blocks
+    constexpr int GM = 8;
+    const int per_group = GM * p.tiles_n;
+    const int first_m = (bid / per_group) * GM;
+    const int gsz = min(GM, p.tiles_m - first_m);
+    const int tm = first_m + (bid % per_group) % gsz, tn = (bid % per_group) / gsz;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
     int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;

@@ -41,7 +41,8 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         }
     }
     ss = wave_sum(ss);
-    const float r = sqrtf(ss / (float)D + eps);
+    // one exact division per row; x * (1/r) differs from x / r by at most one fp32 ulp
+    const float rinv = 1.0f / sqrtf(ss / (float)D + eps);
     half_t *yr = y + n * D;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
@@ -49,7 +50,7 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         if (ch < nchunk) {
             h8 wv = ld8(w + ch * 8), o;
 #pragma unroll
-            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv.v[i]) * (h2f(xv[c].v[i]) / r));
+            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv.v[i]) * (h2f(xv[c].v[i]) * rinv));
             st8(yr + ch * 8, o);
         }
     }
@@ -59,10 +60,10 @@ template <int CH>
 __global__ void __launch_bounds__(kThreads)
 rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t *__restrict__ w,
                     float eps, const half_t *__restrict__ dy, half_t *dx, int dx_acc,
-                    float *__restrict__ dw_part)
+                    float *__restrict__ dw_part, int wide_lds)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    float *sdw = reinterpret_cast<float *>(smem_raw);     // [D]
+    float *sdw = reinterpret_cast<float *>(smem_raw);     // [kWaves][D] (wide_lds) or [D]
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int64_t n = (int64_t)blockIdx.x * kWaves + wid;
     const int nchunk = D / 8;
@@ -99,6 +100,7 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         }
         ss = wave_sum(ss);
         const float r = sqrtf(ss / (float)D + eps);
+        const float rinv = 1.0f / r;              // x * rinv: within one fp32 ulp of x / r
         float sdx = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
@@ -108,11 +110,11 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     float xf = h2f(xv[c].v[i]), du = h2f(gv[c].v[i]);
-                    float t = xf / r;
+                    float t = xf * rinv;
                     dwp[c][i] = rnd16(du * t);
                     float dt = du * h2f(wv.v[i]);
                     sdx += dt * xf;
-                    gv[c].v[i] = f2h(dt / r);           // c1, kept in place of dy
+                    gv[c].v[i] = f2h(dt * rinv);        // c1, kept in place of dy
                     // dt is needed no further: c2 depends only on the row sum
                 }
             }
@@ -141,7 +143,29 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         }
     }
 
-    // block partial of dw: waves add their rows into LDS one after another
+    // block partial of dw (rows summed in wave order either way, so the result does not
+    // depend on the LDS mode): with room for one [D] row per wave every wave stores its row
+    // at once and the columns are summed after a single barrier ...
+    if (wide_lds) {
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * 64 + lane;
+            if (ch < nchunk) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) sdw[wid * D + ch * 8 + i] = dwp[c][i];
+            }
+        }
+        __syncthreads();
+        float *dst = dw_part + (int64_t)blockIdx.x * D;
+        for (int i = threadIdx.x; i < D; i += blockDim.x) {
+            float a = sdw[i];
+#pragma unroll
+            for (int wv = 1; wv < kWaves; wv++) a += sdw[wv * D + i];
+            dst[i] = a;
+        }
+        return;
+    }
+    // ... otherwise the waves add their rows into one LDS row one after another
     for (int wv = 0; wv < kWaves; wv++) {
         if (wid == wv) {
 #pragma unroll
@@ -195,8 +219,18 @@ template <int CH>
 void launch_bwd(int64_t N, int D, const half_t *x, const half_t *w, float eps, const half_t *dy,
                 half_t *dx, int dx_acc, float *part, hipStream_t st)
 {
-    hipLaunchKernelGGL(rms_norm_bwd_kernel<CH>, dim3((unsigned)((N + kWaves - 1) / kWaves)),
-                       dim3(kThreads), (size_t)D * 4, st, N, D, x, w, eps, dy, dx, dx_acc, part);
+    const size_t wide = (size_t)kWaves * D * 4;
+    const int wide_lds = wide <= 144 * 1024;
+    const size_t smem = wide_lds ? wide : (size_t)D * 4;
+    auto kern = rms_norm_bwd_kernel<CH>;
+    static bool attr_set = false;                 // one flag per instantiation
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  144 * 1024);
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(kThreads), smem, st,
+                       N, D, x, w, eps, dy, dx, dx_acc, part, wide_lds);
 }
 
 }  // namespace
