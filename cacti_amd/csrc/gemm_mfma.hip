@@ -105,9 +105,10 @@ struct LoadKC {
     __device__ __forceinline__ void load(uint4 *st, const half_t *origin, int64_t k0) const
     {
         const half_t *base = origin + k0;
+        const bool whole = !KTAIL || k0 + BK <= K;     // uniform: only the last k tile has a tail
 #pragma unroll
         for (int it = 0; it < NL; it++) {
-            if (!KTAIL) {
+            if (whole) {
                 st[it] = ld8<AL>(base, off[it], off[it] + 8);
             } else {
                 const int kc = (threadIdx.x + it * NT) & 7;
@@ -194,7 +195,7 @@ struct LoadKS {
             const int kq = item(it) / RC;
 #pragma unroll
             for (int kk = 0; kk < 8; kk++) {
-                if (!KTAIL) {
+                if (!KTAIL || k0 + BK <= K) {
                     st[it * 8 + kk] = ld8<AL>(base, off[it] + kk * ldb2, off1[it] + kk * ldb2);
                 } else {
                     const int left = (int)(K - k0) - (kq * 8 + kk);   // > 0 iff this k row exists
@@ -238,7 +239,10 @@ struct Loader<true, ROWS, NT, T0, AL, KTAIL> : LoadKS<ROWS, NT, T0, AL, KTAIL> {
 
 // waves per SIMD the register allocation must leave room for: two 128 x 128 blocks (or one
 // 8-wave block) per CU, one 4-wave 256 x 256 block
-constexpr int min_waves(int bm, int bn, int nwaves) { return (bm * bn <= 128 * 128 || nwaves == 8) ? 2 : 1; }
+constexpr int min_waves(int bm, int bn, int nwaves)
+{
+    return bm * bn <= 64 * 128 ? 3 : (bm * bn <= 128 * 128 || nwaves == 8) ? 2 : 1;
+}
 
 template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
 __global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN))
@@ -250,8 +254,10 @@ gemm_mfma_kernel(GemmArgs p)
     half_t *As = reinterpret_cast<half_t *>(smem_raw);            // [2][BM*BK]
     half_t *Bs = As + 2 * BM * BK;                                // [2][BN*BK]
 
-    // XCD-aware numbering: dispatch order i lands on XCD i % 8; give each XCD a contiguous
-    // band of the tile sequence
+    // XCD-aware numbering over the flattened (block of the batch, tile) sequence: dispatch
+    // order i lands on XCD i % 8; give each XCD a contiguous band.  With a batch that is a
+    // multiple of 8 an XCD then owns whole blocks of the batch, which also balances the
+    // triangular modes (their work per tile row grows or shrinks along M).
     const int nb = gridDim.x;
     int bid = blockIdx.x;
     {
@@ -259,14 +265,19 @@ gemm_mfma_kernel(GemmArgs p)
         const int xcd = bid & 7, idx = bid >> 3;
         bid = xcd * per + (xcd < rem ? xcd : rem) + idx;
     }
-    // within the band, tiles are walked in groups of 8 tile rows x all tile columns, row
-    // fastest: the ~64 blocks resident on an XCD then form an 8 x 8 patch of C and each
-    // operand panel fetched into its L2 is shared by 8 blocks
+    const int tiles = p.tiles_m * p.tiles_n;
+    const int64_t bz = bid / tiles;
+    bid -= (int)bz * tiles;
+    // within a block of the batch, tiles are walked in groups of 8 tile rows x all tile
+    // columns, row fastest: the ~64 blocks resident on an XCD then form an 8 x 8 patch of C
+    // and each operand panel fetched into its L2 is shared by 8 blocks
     constexpr int GM = 8;
     const int per_group = GM * p.tiles_n;
     const int first_m = (bid / per_group) * GM;
     const int gsz = min(GM, p.tiles_m - first_m);
-    const int tm = first_m + (bid % per_group) % gsz, tn = (bid % per_group) / gsz;
+    int tm = first_m + (bid % per_group) % gsz;
+    const int tn = (bid % per_group) / gsz;
+    if (p.tri == 2) tm = p.tiles_m - 1 - tm;                      // longest k ranges first
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
     int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;
@@ -274,7 +285,6 @@ gemm_mfma_kernel(GemmArgs p)
     if (p.tri == 2) nk = min(nk, (int)((m0 + BM + BK - 1) / BK));
     if (p.tri == 3) kt0 = (int)(m0 / BK);
 
-    const int64_t bz = blockIdx.z;
     const half_t *A = p.A + bz * p.sa;
     const half_t *B = p.B + bz * p.sb;
     half_t *C = p.C + bz * p.sc;
@@ -365,11 +375,18 @@ gemm_mfma_kernel(GemmArgs p)
         lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
         __syncthreads();
         for (int kt = kt0; kt < nk; kt++) {
-            la.load(ra[0], Ao, tile_k(kt + 1));
-            lb.load(rb[0], Bo, tile_k(kt + 1));
+            // short-K instantiations skip the load past the last tile (a third of their
+            // traffic when K spans two tiles); the long-K ones keep the loop branch-free
+            const bool more = !KTAIL || kt + 1 < nk;
+            if (more) {
+                la.load(ra[0], Ao, tile_k(kt + 1));
+                lb.load(rb[0], Bo, tile_k(kt + 1));
+            }
             compute(kt & 1);
-            la.store(ra[0], As + ((kt + 1) & 1) * BM * BK);
-            lb.store(rb[0], Bs + ((kt + 1) & 1) * BN * BK);
+            if (more) {
+                la.store(ra[0], As + ((kt + 1) & 1) * BM * BK);
+                lb.store(rb[0], Bs + ((kt + 1) & 1) * BN * BK);
+            }
             __syncthreads();
         }
     }
@@ -444,7 +461,10 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
                                       (int)smem));
         attr_set = true;
     }
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)nblk), block(WM * WN * 64);
+    const int64_t nwg = (int64_t)p.tiles_m * p.tiles_n * nblk;
+    CACTI_REQUIRE(nwg < (int64_t)1 << 31, CACTI_E_NOTIMPL, "gemm: %lld workgroups exceed the grid limit",
+                  (long long)nwg);
+    dim3 grid((unsigned)nwg), block(WM * WN * 64);
     hipLaunchKernelGGL(kern, grid, block, smem, st, p);
     return launch_status("gemm_mfma");
 }
@@ -456,7 +476,10 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
 {
     constexpr int S0 = (!TA && TB) ? 2 : 1;       // 128 x 128: two stages only if no operand is strided
     const bool ktail = (p.K % BK) != 0;
-    if (align < 8) {                              // 8-byte aligned operands: one tile shape
+    if (align < 8) {                              // 8-byte aligned operands (the attention blocks)
+        if (tile == 4)
+            return ktail ? launch_cfg<TA, TB, 64, 128, 2, 2, 4, true, 1>(p, nblk, st)
+                         : launch_cfg<TA, TB, 64, 128, 2, 2, 4, false, 1>(p, nblk, st);
         return ktail ? launch_cfg<TA, TB, 128, 128, 2, 2, 4, true, 1>(p, nblk, st)
                      : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, 1>(p, nblk, st);
     }

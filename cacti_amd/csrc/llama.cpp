@@ -103,6 +103,13 @@ CACTI_API int cacti_ctx_set_timing(cacti_ctx *ctx, int on)
     return 0;
 }
 
+CACTI_API int cacti_ctx_set_timing_filter(cacti_ctx *ctx, const char *label_prefix, int every)
+{
+    CACTI_REQUIRE(ctx && every >= 1, CACTI_E_INVALID, "set_timing_filter: null context or every < 1");
+    ctx->c.set_timing_filter(label_prefix ? label_prefix : "", every);
+    return 0;
+}
+
 CACTI_API int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap)
 {
     CACTI_REQUIRE(ctx && buf && cap > 0, CACTI_E_INVALID, "timing_report: null pointer");

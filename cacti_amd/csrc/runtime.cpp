@@ -560,7 +560,16 @@ int Ctx::run_entry(const Entry &e)
         for (CellPtr a : e.args) ap.push_back(dev_ptr(cells_[a].voff));
         for (CellPtr o : e.outs) op.push_back(dev_ptr(cells_[o].voff));
         hipEvent_t e0 = ev0_, e1 = ev1_;
-        if (timing_ == 2) {
+        int timing = timing_;
+        std::string key;
+        if (timing == 2) {
+            key = sp.key(aty, e.acc_mask);
+            if (!timing_filter_.empty() && key.compare(0, timing_filter_.size(), timing_filter_) != 0)
+                timing = 0;
+            else if (timing_seen_++ % (uint64_t)timing_every_ != 0)
+                timing = 0;
+        }
+        if (timing == 2) {
             if (ev_keys_.size() == ev_pool_.size()) {
                 hipEvent_t a, b;
                 hipEventCreate(&a);
@@ -569,13 +578,13 @@ int Ctx::run_entry(const Entry &e)
             }
             e0 = ev_pool_[ev_keys_.size()].first;
             e1 = ev_pool_[ev_keys_.size()].second;
-            ev_keys_.push_back(sp.key(aty, e.acc_mask));
+            ev_keys_.push_back(key);
         }
-        if (timing_) hipEventRecord(e0, stream_);
+        if (timing) hipEventRecord(e0, stream_);
         rc = sp.run(*this, aty, ap.data(), oty, op.data(), e.acc_mask,
                     ws_off == kNoOffset ? nullptr : dev_ptr(ws_off), ws_bytes);
-        if (timing_) hipEventRecord(e1, stream_);
-        if (timing_ == 1 && !rc) {
+        if (timing) hipEventRecord(e1, stream_);
+        if (timing == 1 && !rc) {
             hipEventSynchronize(e1);
             float ms = 0;
             hipEventElapsedTime(&ms, e0, e1);

@@ -173,6 +173,12 @@ class Ctx {
     // 0 = off; 1 = sync after every thunk; 2 = event pairs recorded without syncing and read
     // back by collect_timings() (measures each launch inside an undisturbed run)
     void set_timing(int mode) { timing_ = mode; }
+    void set_timing_filter(const std::string &prefix, int every)
+    {
+        timing_filter_ = prefix;
+        timing_every_ = every;
+        timing_seen_ = 0;
+    }
     int collect_timings();
     void clear_timings() { times_.clear(); }
     const std::map<std::string, std::pair<double, uint64_t>> &timings() const { return times_; }
@@ -203,6 +209,9 @@ class Ctx {
     uint64_t n_alloc_ = 0, n_evict_ = 0, n_upload_ = 0, bytes_d2h_ = 0, bytes_h2d_ = 0,
              n_soft_oom_ = 0, n_run_ = 0, host_bytes_ = 0;
     int timing_ = 0;
+    std::string timing_filter_;
+    int timing_every_ = 1;
+    uint64_t timing_seen_ = 0;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> ev_pool_;
     std::vector<std::string> ev_keys_;
     std::map<std::string, std::pair<double, uint64_t>> times_;

@@ -16,6 +16,28 @@ namespace {
 //  InnerSoftmaxPostAdj :3386-3457.)
 constexpr int kRowsPerBlock = 4;
 
+// e / sum for 0 <= e <= 1 <= sum without the general division sequence: y approximates 1 / sum
+// to within an ulp (one Newton step on v_rcp_f32), q0 = e y is within an ulp of the quotient,
+// and one residual correction rounds it to the nearest float (Markstein's theorem; it holds
+// for every divisor whose significand is not all ones, which is enough to agree with IEEE
+// division on all but a vanishing fraction of inputs, and the f16 rounding that follows
+// absorbs those).
+struct RowDivide {
+    float d, y;
+    __device__ explicit RowDivide(float sum) : d(sum)
+    {
+        const float y0 = __builtin_amdgcn_rcpf(sum);
+        y = __builtin_fmaf(__builtin_fmaf(-sum, y0, 1.0f), y0, y0);
+    }
+    __device__ float operator()(float e) const
+    {
+        const float q0 = e * y;
+        return __builtin_fmaf(__builtin_fmaf(-q0, d, e), y, q0);
+    }
+};
+
+// A wave owns one row and holds it in registers; chunk c covers columns [512 c, 512 c + 512)
+// (8 per lane), and chunks wholly above the diagonal are skipped (i is uniform in the wave).
 template <int CH, bool BWD>
 __global__ void __launch_bounds__(kRowsPerBlock * 64)
 causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
@@ -27,14 +49,18 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
     const int i = (int)(row / H);                 // query position
     const int nchunk = (int)(S / 8);
     const half_t *sr = s16 + row * S;
+    const half_t *gr = BWD ? dp16 + row * S : nullptr;
     float e[CH][8];
+    h8 g[CH];
     float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
+        if (c * 512 > i) continue;
         const int ch = c * 64 + lane;
         const int j0 = ch * 8;
         if (ch < nchunk && j0 <= i) {
             h8 v = ld8(sr + j0);
+            if (BWD) g[c] = ld8(gr + j0);
 #pragma unroll
             for (int k = 0; k < 8; k++) {
                 e[c][k] = (j0 + k <= i) ? h2f(v.v[k]) : -INFINITY;
@@ -42,19 +68,25 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
             }
         } else {
 #pragma unroll
-            for (int k = 0; k < 8; k++) e[c][k] = -INFINITY;
+            for (int k = 0; k < 8; k++) {
+                e[c][k] = -INFINITY;
+                if (BWD) g[c].v[k] = (half_t)0.f;
+            }
         }
     }
     mx = wave_max(mx);
     float sum = 0.f;
 #pragma unroll
-    for (int c = 0; c < CH; c++)
+    for (int c = 0; c < CH; c++) {
+        if (c * 512 > i) continue;
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             e[c][k] = expf(e[c][k] - mx);         // exp(-inf) = 0 above the diagonal
             sum += e[c][k];
         }
+    }
     sum = wave_sum(sum);
+    const RowDivide div(sum);
     half_t *orow = out + row * S;
     // columns written: j <= i, then zeros to the next multiple of 256 (the triangular GEMMs
     // read no further); the rest of the row is left untouched
@@ -62,34 +94,31 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
     if (!BWD) {
 #pragma unroll
         for (int c = 0; c < CH; c++) {
+            if (c * 512 > i) continue;
             const int ch = c * 64 + lane;
             if (ch < wchunk) {
                 h8 o;
 #pragma unroll
-                for (int k = 0; k < 8; k++) o.v[k] = f2h(e[c][k] / sum);
+                for (int k = 0; k < 8; k++) o.v[k] = f2h(div(e[c][k]));
                 st8(orow + ch * 8, o);
             }
         }
     } else {
-        const half_t *gr = dp16 + row * S;
-        h8 g[CH];
         float tsum = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
-            const int ch = c * 64 + lane;
-            const int j0 = ch * 8;
-            const bool ld = ch < nchunk && j0 <= i;
-            if (ld) g[c] = ld8(gr + j0);
+            if (c * 512 > i) continue;
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                const float p = e[c][k] / sum;          // 0 above the diagonal
+                const float p = div(e[c][k]);           // 0 above the diagonal
                 e[c][k] = p;
-                if (ld && j0 + k <= i) tsum += p * h2f(g[c].v[k]);
+                if ((c * 64 + lane) * 8 + k <= i) tsum += p * h2f(g[c].v[k]);
             }
         }
         tsum = wave_sum(tsum);
 #pragma unroll
         for (int c = 0; c < CH; c++) {
+            if (c * 512 > i) continue;
             const int ch = c * 64 + lane;
             const int j0 = ch * 8;
             if (ch < wchunk) {
@@ -97,12 +126,8 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
 #pragma unroll
                 for (int k = 0; k < 8; k++) {
                     const float p = e[c][k];
-                    if (j0 + k <= i) {
-                        const float t = p * h2f(g[c].v[k]);
-                        o.v[k] = f2h(t - tsum * p);
-                    } else {
-                        o.v[k] = (half_t)0.f;
-                    }
+                    const float t = p * h2f(g[c].v[k]);
+                    o.v[k] = (j0 + k <= i) ? f2h(t - tsum * p) : (half_t)0.f;
                 }
                 st8(orow + ch * 8, o);
             }

@@ -73,6 +73,7 @@ SIGNATURES = {
     "cacti_ctx_sync": (ci, [vp]),
     "cacti_ctx_stream": (vp, [vp]),
     "cacti_ctx_set_timing": (ci, [vp, ci]),
+    "cacti_ctx_set_timing_filter": (ci, [vp, C.c_char_p, ci]),
     "cacti_ctx_timing_report": (ci, [vp, C.c_char_p, sz]),
     "cacti_mempool_create": (ci, [pvp, C.c_uint64]),
     "cacti_mempool_destroy": (ci, [vp]),

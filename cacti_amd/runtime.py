@@ -67,6 +67,11 @@ class Ctx:
         """0 off (clears totals), 1 sync per thunk, 2 event pairs without syncing."""
         ffi.call("cacti_ctx_set_timing", self._c, int(mode))
 
+    def set_timing_filter(self, prefix, every=1):
+        """Mode 2 then times only every `every`-th launch whose label starts with prefix
+        ('' = all labels)."""
+        ffi.call("cacti_ctx_set_timing_filter", self._c, (prefix or "").encode(), int(every))
+
     def timing_report(self):
         buf = C.create_string_buffer(1 << 18)
         ffi.call("cacti_ctx_timing_report", self._c, buf, len(buf))

@@ -55,8 +55,13 @@ void *cacti_ctx_stream(cacti_ctx *ctx);                 /* the hipStream_t all w
  * every thunk; mode 2 records a HIP event pair around every launch without syncing and
  * reads them back in the report, so a run is measured undisturbed; 0 switches timing off
  * and clears the totals.  The report is text, one "label count total_ms" line per label;
- * GEMM labels carry the transposes and nblk x M x N x K. */
+ * GEMM labels carry the transposes and nblk x M x N x K.  A filter restricts mode 2 to the
+ * launches whose label starts with the given text (an event pair costs a few microseconds
+ * of stream time per launch, about 10 % of a whole step when every launch carries one);
+ * NULL or "" matches every launch; of the matching launches every `every`-th is timed
+ * (1 = all). */
 int cacti_ctx_set_timing(cacti_ctx *ctx, int on);
+int cacti_ctx_set_timing_filter(cacti_ctx *ctx, const char *label_prefix, int every);
 int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap);
 
 /* ---- the pool's placement policy alone, over a plain offset range (no device memory is
