@@ -24,6 +24,7 @@ struct GemmArgs {
     // For 2 and 3 the entries of A above the diagonal must be zero up to the next multiple
     // of 256 columns; beyond that they are never read.
     int tri;
+    int gm, xcd;          // tile walk: rows per group; 1 = XCD-banded numbering
 };
 constexpr int kTriPad = 256;
 

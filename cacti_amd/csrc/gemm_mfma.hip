@@ -237,12 +237,24 @@ struct Loader<false, ROWS, NT, T0, AL, KTAIL> : LoadKC<ROWS, NT, AL, KTAIL> {};
 template <int ROWS, int NT, int T0, int AL, bool KTAIL>
 struct Loader<true, ROWS, NT, T0, AL, KTAIL> : LoadKS<ROWS, NT, T0, AL, KTAIL> {};
 
+// scheduling pattern of one k step: NM MFMAs with NR LDS reads spread evenly between them
+template <int NM, int NR, int R>
+struct SchedStep {
+    static __device__ __forceinline__ void run()
+    {
+        __builtin_amdgcn_sched_group_barrier(0x008, (NM * (R + 1)) / NR - (NM * R) / NR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        SchedStep<NM, NR, R + 1>::run();
+    }
+};
+template <int NM, int NR>
+struct SchedStep<NM, NR, NR> {
+    static __device__ __forceinline__ void run() {}
+};
+
 // waves per SIMD the register allocation must leave room for: two 128 x 128 blocks (or one
 // 8-wave block) per CU, one 4-wave 256 x 256 block
-constexpr int min_waves(int bm, int bn, int nwaves)
-{
-    return bm * bn <= 64 * 128 ? 3 : (bm * bn <= 128 * 128 || nwaves == 8) ? 2 : 1;
-}
+constexpr int min_waves(int bm, int bn, int nwaves) { return (bm * bn <= 128 * 128 || nwaves == 8) ? 2 : 1; }
 
 template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
 __global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN))
@@ -260,7 +272,7 @@ gemm_mfma_kernel(GemmArgs p)
     // triangular modes (their work per tile row grows or shrinks along M).
     const int nb = gridDim.x;
     int bid = blockIdx.x;
-    {
+    if (p.xcd) {
         const int per = nb >> 3, rem = nb & 7;
         const int xcd = bid & 7, idx = bid >> 3;
         bid = xcd * per + (xcd < rem ? xcd : rem) + idx;
@@ -271,7 +283,7 @@ gemm_mfma_kernel(GemmArgs p)
     // within a block of the batch, tiles are walked in groups of 8 tile rows x all tile
     // columns, row fastest: the ~64 blocks resident on an XCD then form an 8 x 8 patch of C
     // and each operand panel fetched into its L2 is shared by 8 blocks
-    constexpr int GM = 8;
+    const int GM = p.gm;
     const int per_group = GM * p.tiles_n;
     const int first_m = (bid / per_group) * GM;
     const int gsz = min(GM, p.tiles_m - first_m);
@@ -321,27 +333,54 @@ gemm_mfma_kernel(GemmArgs p)
     auto tile_k = [&](int kt) __attribute__((always_inline)) {
         return (int64_t)(kt < nk ? kt : nk - 1) * BK;
     };
+    // MFMAs of k step ks run while the operand fragments of step ks + 1 are in flight from
+    // LDS (two fragment sets): the wait before a step's MFMAs leaves the next step's reads
+    // outstanding
     auto compute = [&](int cur) __attribute__((always_inline)) {
         const half_t *as = As + cur * BM * BK + ar0 * BK;
         const half_t *bs = Bs + cur * BN * BK + br0 * BK;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ks++) {
+        // fragment double-buffering costs (TM + TN) * 4 registers: used where it fits without
+        // spilling (16-byte aligned operands, all but the 8-wave 256 x 256 tile)
+        constexpr bool PIPE = AL == 8 && !(BM * BN == 256 * 256 && WM * WN == 8);
+        half8_t af[PIPE ? 2 : 1][TM], bf[PIPE ? 2 : 1][TN];
+        auto frags = [&](int set, int ks) __attribute__((always_inline)) {
             const int q = ks * 2 + lh;
-            half8_t af[TM], bf[TN];
 #pragma unroll
             for (int i = 0; i < TM; i++)
-                af[i] = *reinterpret_cast<const half8_t *>(
+                af[set][i] = *reinterpret_cast<const half8_t *>(
                     as + i * 32 * BK + ((q ^ asw ^ ((i & 1) << 2)) << 3));
 #pragma unroll
             for (int j = 0; j < TN; j++)
-                bf[j] = *reinterpret_cast<const half8_t *>(
+                bf[set][j] = *reinterpret_cast<const half8_t *>(
                     bs + j * 32 * BK + ((q ^ bsw ^ ((j & 1) << 2)) << 3));
+        };
+        if (PIPE) frags(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ks++) {
+            const int cur_set = PIPE ? (ks & 1) : 0;
+            if (!PIPE) frags(0, ks);
+            else if (ks + 1 < BK / 16) frags((ks + 1) & 1, ks + 1);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] =
-                        __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[cur_set][j], af[cur_set][i],
+                                                                       acc[i][j], 0, 0, 0);
+        }
+        if (PIPE) {
+            // pin that order for the instruction scheduler (it would otherwise sink each read
+            // to just before its use): the first fragment set, then per k step its MFMAs
+            // with the next step's LDS reads spread between them
+            constexpr int NM = TM * TN, NR = TM + TN;
+            // with one register stage the global loads of the next tile (same scheduling region
+            // when no operand is strided) must go first, so that their latency overlaps the
+            // whole k tile; with two stages they are a tile ahead anyway and are left to the
+            // scheduler (measured: pinning them first costs 5 %)
+            if (STAGES == 1) __builtin_amdgcn_sched_group_barrier(0x020, LA::NREG + LB::NREG, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
+#pragma unroll
+            for (int ks = 0; ks + 1 < BK / 16; ks++) SchedStep<NM, NR, 0>::run();
+            __builtin_amdgcn_sched_group_barrier(0x008, NM, 0);
         }
     };
 
@@ -353,19 +392,23 @@ gemm_mfma_kernel(GemmArgs p)
         la.store(ra[0], As + (kt0 & 1) * BM * BK);
         lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
         __syncthreads();
-        for (int kt = kt0; kt < nk; kt += 2) {
+        int kt = kt0;
+        for (; kt + 1 < nk; kt += 2) {
             la.load(ra[0], Ao, tile_k(kt + 2));
             lb.load(rb[0], Bo, tile_k(kt + 2));
             compute(kt & 1);
             la.store(ra[STAGES - 1], As + ((kt + 1) & 1) * BM * BK);
             lb.store(rb[STAGES - 1], Bs + ((kt + 1) & 1) * BN * BK);
             __syncthreads();
-            if (kt + 1 >= nk) break;
             la.load(ra[STAGES - 1], Ao, tile_k(kt + 3));
             lb.load(rb[STAGES - 1], Bo, tile_k(kt + 3));
             compute((kt + 1) & 1);
             la.store(ra[0], As + (kt & 1) * BM * BK);
             lb.store(rb[0], Bs + (kt & 1) * BN * BK);
+            __syncthreads();
+        }
+        if (kt < nk) {                            // odd number of k tiles: the last one is in LDS
+            compute(kt & 1);
             __syncthreads();
         }
     } else {
@@ -477,9 +520,6 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
     constexpr int S0 = (!TA && TB) ? 2 : 1;       // 128 x 128: two stages only if no operand is strided
     const bool ktail = (p.K % BK) != 0;
     if (align < 8) {                              // 8-byte aligned operands (the attention blocks)
-        if (tile == 4)
-            return ktail ? launch_cfg<TA, TB, 64, 128, 2, 2, 4, true, 1>(p, nblk, st)
-                         : launch_cfg<TA, TB, 64, 128, 2, 2, 4, false, 1>(p, nblk, st);
         return ktail ? launch_cfg<TA, TB, 128, 128, 2, 2, 4, true, 1>(p, nblk, st)
                      : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, 1>(p, nblk, st);
     }
@@ -501,6 +541,18 @@ namespace cacti {
 int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align, int tile,
                      hipStream_t st)
 {
+    GemmArgs q = p;
+    {
+        static int gm = 0, xcd = -1;
+        if (!gm) {
+            const char *e = getenv("CACTI_GEMM_GM");
+            gm = e ? atoi(e) : 8;
+            e = getenv("CACTI_GEMM_XCD");
+            xcd = e ? atoi(e) : 1;
+        }
+        q.gm = gm;
+        q.xcd = xcd;
+    }
     if (tile < 0) {
         static int forced = -2;
         if (forced == -2) {
@@ -517,10 +569,10 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             tile = (!ta && tb && big >= 768) ? 3 : 0;
         }
     }
-    if (!ta && !tb) return launch_tile<false, false>(tile, align, p, nblk, st);
-    if (!ta && tb) return launch_tile<false, true>(tile, align, p, nblk, st);
-    if (ta && !tb) return launch_tile<true, false>(tile, align, p, nblk, st);
-    return launch_tile<true, true>(tile, align, p, nblk, st);
+    if (!ta && !tb) return launch_tile<false, false>(tile, align, q, nblk, st);
+    if (!ta && tb) return launch_tile<false, true>(tile, align, q, nblk, st);
+    if (ta && !tb) return launch_tile<true, false>(tile, align, q, nblk, st);
+    return launch_tile<true, true>(tile, align, q, nblk, st);
 }
 
 }  // namespace cacti
