@@ -78,14 +78,13 @@ def gemm_flops(label):
 def kernel_symbol(label):
     """Name of the HIP kernel instantiation a dense GEMM label runs on, as rocprofv3 prints it
     (the tile choice mirrors gemm_mfma_launch: 256 x 256 for k-contiguous operands when that
-    still gives 768 tiles, else 128 x 128; two register stages only for NT)."""
+    still gives 768 tiles, else 128 x 128 with two register stages)."""
     m = GEMM_RE.match(label)
     ta, tb = m.group(2) == "T", m.group(3) == "T"
     H, M, N = int(m.group(4)), int(m.group(5)), int(m.group(6))
-    nt = not ta and tb
     big = ((M + 255) // 256) * ((N + 255) // 256) * H
-    tile = "256, 256, 2, 2, 8, false, 1" if nt and big >= 768 else \
-           "128, 128, 2, 2, 8, false, %d" % (2 if nt else 1)
+    tile = "256, 256, 2, 2, 8, false, 1" if (not ta and tb and big >= 768) else \
+           "128, 128, 2, 2, 8, false, 2"
     return "gemm_mfma_kernel<%s, %s, %s>" % (str(ta).lower(), str(tb).lower(), tile)
 
 

@@ -30,6 +30,8 @@
 #include "common.h"
 #include "gemm_internal.h"
 
+#include <type_traits>
+
 using namespace cacti;
 
 namespace {
@@ -231,6 +233,147 @@ struct LoadKS {
     static constexpr int NREG = NL * 8;
 };
 
+// ---- both operands k-strided (A^T and B), square block tile with exactly one 8 k x 8 rows
+// item per lane: the first half of the block takes A items, the second half B items.  Which
+// operand a wave works on only changes its base pointer, leading dimension and LDS target, so
+// the load / transpose / store sequence is one straight line for the whole block (no branch
+// splits the k loop into several scheduling regions).
+template <int BT, int NT, int AL, bool KTAIL>
+struct LoadKS2 {
+    static_assert(2 * BT == NT, "one item per lane");
+    static constexpr int RC = BT / 8;
+    uint32_t off, off1, ldb2;
+    const half_t *origin;
+    int64_t ld, K;
+    int lds_extra;                 // halves from the A stage buffer to this lane's operand buffer
+    int rc, kq;
+
+    __device__ __forceinline__ void init(const half_t *Ao, int64_t lda, int64_t rows_a,
+                                         const half_t *Bo, int64_t ldb, int64_t rows_b, int64_t K_)
+    {
+        const bool is_b = threadIdx.x >= BT;
+        const int c = threadIdx.x - (is_b ? BT : 0);
+        const int64_t rows_left = is_b ? rows_b : rows_a;
+        origin = is_b ? Bo : Ao;
+        ld = is_b ? ldb : lda;
+        lds_extra = is_b ? 2 * BT * BK : 0;
+        K = K_;
+        ldb2 = (uint32_t)(ld * 2);
+        rc = c % RC;
+        kq = c / RC;
+        int r0 = rc * 8, r1 = rc * 8 + 4;
+        if (AL == 8) {
+            if (r0 > rows_left - 8) r0 = (int)rows_left - 8;
+        } else {
+            if (r0 > rows_left - 4) r0 = (int)rows_left - 4;
+            if (r1 > rows_left - 4) r1 = (int)rows_left - 4;
+        }
+        off = (uint32_t)(((int64_t)kq * 8 * ld + r0) * 2);
+        off1 = (uint32_t)(((int64_t)kq * 8 * ld + r1) * 2);
+    }
+    __device__ __forceinline__ void load(uint4 *st, const half_t *, int64_t k0) const
+    {
+        const half_t *base = origin + k0 * ld;
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) {
+            if (!KTAIL || k0 + BK <= K) {
+                st[kk] = ld8<AL>(base, off + kk * ldb2, off1 + kk * ldb2);
+            } else {
+                const int left = (int)(K - k0) - (kq * 8 + kk);
+                const uint32_t back = left > 0 ? 0 : (uint32_t)(1 - left) * ldb2;
+                uint4 v = ld8<AL>(base, off + kk * ldb2 - back, off1 + kk * ldb2 - back);
+                if (left <= 0) v = make_uint4(0, 0, 0, 0);
+                st[kk] = v;
+            }
+        }
+    }
+    // lds = the A buffer of the stage being filled
+    __device__ __forceinline__ void store(const uint4 *st, half_t *lds) const
+    {
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(st);
+        half_t *dst = lds + lds_extra;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+            uint4 o;
+            o.x = __builtin_amdgcn_perm(w[1 * 4 + (j >> 1)], w[0 * 4 + (j >> 1)], sel);
+            o.y = __builtin_amdgcn_perm(w[3 * 4 + (j >> 1)], w[2 * 4 + (j >> 1)], sel);
+            o.z = __builtin_amdgcn_perm(w[5 * 4 + (j >> 1)], w[4 * 4 + (j >> 1)], sel);
+            o.w = __builtin_amdgcn_perm(w[7 * 4 + (j >> 1)], w[6 * 4 + (j >> 1)], sel);
+            *reinterpret_cast<uint4 *>(dst + lds_off(rc * 8 + j, kq)) = o;
+        }
+    }
+    static constexpr int NREG = 8;
+};
+
+// ---- one k-strided operand, every lane of the block taking part: an item is 4 k x 8 rows
+// (half of LoadKS's), so ROWS * 2 items spread over exactly NT lanes with no idle
+// wavefronts and no branch in the k loop.  Each of the 8 tile rows of an item gets 4 k
+// values (8 bytes of its 16-byte k chunk).
+template <int ROWS, int NT, int AL, bool KTAIL>
+struct LoadKSH {
+    static_assert(ROWS * 2 == NT, "one half item per lane");
+    static constexpr int RC = ROWS / 8;
+    uint32_t off, off1, ldb2;
+    int64_t ld, K;
+    int rc, kq4;                   // row chunk; group of 4 k rows (0..15)
+
+    __device__ __forceinline__ void init(int64_t ld_, int64_t rows_left, int64_t K_)
+    {
+        ld = ld_;
+        K = K_;
+        ldb2 = (uint32_t)(ld_ * 2);
+        rc = threadIdx.x % RC;
+        kq4 = threadIdx.x / RC;
+        int r0 = rc * 8, r1 = rc * 8 + 4;
+        if (AL == 8) {
+            if (r0 > rows_left - 8) r0 = (int)rows_left - 8;
+        } else {
+            if (r0 > rows_left - 4) r0 = (int)rows_left - 4;
+            if (r1 > rows_left - 4) r1 = (int)rows_left - 4;
+        }
+        off = (uint32_t)(((int64_t)kq4 * 4 * ld + r0) * 2);
+        off1 = (uint32_t)(((int64_t)kq4 * 4 * ld + r1) * 2);
+    }
+    __device__ __forceinline__ void load(uint4 *st, const half_t *origin, int64_t k0) const
+    {
+        const half_t *base = origin + k0 * ld;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            if (!KTAIL || k0 + BK <= K) {
+                st[kk] = ld8<AL>(base, off + kk * ldb2, off1 + kk * ldb2);
+            } else {
+                const int left = (int)(K - k0) - (kq4 * 4 + kk);
+                const uint32_t back = left > 0 ? 0 : (uint32_t)(1 - left) * ldb2;
+                uint4 v = ld8<AL>(base, off + kk * ldb2 - back, off1 + kk * ldb2 - back);
+                if (left <= 0) v = make_uint4(0, 0, 0, 0);
+                st[kk] = v;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(const uint4 *st, half_t *lds) const
+    {
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(st);       // [kk][4 words]
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+            uint2 o;
+            o.x = __builtin_amdgcn_perm(w[1 * 4 + (j >> 1)], w[0 * 4 + (j >> 1)], sel);
+            o.y = __builtin_amdgcn_perm(w[3 * 4 + (j >> 1)], w[2 * 4 + (j >> 1)], sel);
+            *reinterpret_cast<uint2 *>(lds + lds_off(rc * 8 + j, kq4 >> 1) + (kq4 & 1) * 4) = o;
+        }
+    }
+    static constexpr int NREG = 4;
+};
+
+// stands in for the B loader when LoadKS2 serves both operands
+struct LoadNone {
+    __device__ __forceinline__ void init(int64_t, int64_t, int64_t) {}
+    __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
+    __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
+    static constexpr int NREG = 1;
+};
+
 template <bool STRIDED, int ROWS, int NT, int T0, int AL, bool KTAIL> struct Loader;
 template <int ROWS, int NT, int T0, int AL, bool KTAIL>
 struct Loader<false, ROWS, NT, T0, AL, KTAIL> : LoadKC<ROWS, NT, AL, KTAIL> {};
@@ -309,12 +452,25 @@ gemm_mfma_kernel(GemmArgs p)
     const int l32 = lane & 31, lh = lane >> 5;
 
     // when both operands are strided they use disjoint halves of the block
-    typedef Loader<TA, BM, NT, 0, AL, KTAIL> LA;
-    typedef Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL, KTAIL> LB;
+    constexpr bool UNI = TA && !TB && BM == BN && BM + BN == NT;  // one combined strided loader
+    // exactly one strided operand and a 128-row tile on 256 lanes: half items on every lane
+    constexpr bool HALF_A = TA && TB && BM * 2 == NT, HALF_B = !TA && !TB && BN * 2 == NT;
+    typedef typename std::conditional<
+        UNI, LoadKS2<BM, NT, AL, KTAIL>,
+        typename std::conditional<HALF_A, LoadKSH<BM, NT, AL, KTAIL>,
+                                  Loader<TA, BM, NT, 0, AL, KTAIL>>::type>::type LA;
+    typedef typename std::conditional<
+        UNI, LoadNone,
+        typename std::conditional<HALF_B, LoadKSH<BN, NT, AL, KTAIL>,
+                                  Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL, KTAIL>>::type>::type LB;
     LA la;
     LB lb;
-    la.init(p.lda, p.M - m0, p.K);
-    lb.init(p.ldb, p.N - n0, p.K);
+    if constexpr (UNI) {
+        la.init(Ao, p.lda, p.M - m0, Bo, p.ldb, p.N - n0, p.K);
+    } else {
+        la.init(p.lda, p.M - m0, p.K);
+        lb.init(p.ldb, p.N - n0, p.K);
+    }
     uint4 ra[STAGES][LA::NREG], rb[STAGES][LB::NREG];
 
     float16_t acc[TM][TN];
@@ -517,11 +673,13 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 template <bool TA, bool TB>
 int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
 {
-    constexpr int S0 = (!TA && TB) ? 2 : 1;       // 128 x 128: two stages only if no operand is strided
+    // 128 x 128 on 256 lanes: every loader is branch-free and small enough for two register
+    // stages
+    constexpr int S0 = 2;
     const bool ktail = (p.K % BK) != 0;
     if (align < 8) {                              // 8-byte aligned operands (the attention blocks)
         return ktail ? launch_cfg<TA, TB, 128, 128, 2, 2, 4, true, 1>(p, nblk, st)
-                     : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, 1>(p, nblk, st);
+                     : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, S0>(p, nblk, st);
     }
     if (ktail) return launch_cfg<TA, TB, 128, 128, 2, 2, 8, true, 1>(p, nblk, st);
     switch (tile) {
