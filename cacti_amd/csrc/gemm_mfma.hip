@@ -485,10 +485,6 @@ gemm_mfma_kernel(GemmArgs p)
     const int ar0 = wm * (BM / WM) + l32, br0 = wn * (BN / WN) + l32;
     const int asw = swz(ar0), bsw = swz(br0);                     // row + 32 i flips bit 2
 
-    // loads past the last tile re-read the last one; their LDS copy is never used
-    auto tile_k = [&](int kt) __attribute__((always_inline)) {
-        return (int64_t)(kt < nk ? kt : nk - 1) * BK;
-    };
     // MFMAs of k step ks run while the operand fragments of step ks + 1 are in flight from
     // LDS (two fragment sets): the wait before a step's MFMAs leaves the next step's reads
     // outstanding
@@ -540,54 +536,51 @@ gemm_mfma_kernel(GemmArgs p)
         }
     };
 
-    if (STAGES == 2) {
-        la.load(ra[0], Ao, tile_k(kt0));
-        lb.load(rb[0], Bo, tile_k(kt0));
-        la.load(ra[STAGES - 1], Ao, tile_k(kt0 + 1));
-        lb.load(rb[STAGES - 1], Bo, tile_k(kt0 + 1));
+    // Software pipeline over k tiles with STAGES register sets and two LDS buffers.  Invariant
+    // at the start of tile t: LDS[t & 1] holds tile t, register set (t + j - kt0) % STAGES
+    // holds tile t + j for j = 1 .. STAGES - 1, and set (t - kt0) % STAGES is free.  A step
+    // loads tile t + STAGES into the free set, runs the MFMAs of tile t, moves tile t + 1 from
+    // its set to the other LDS buffer and ends in the one barrier of the k tile.  The main
+    // loop has no branch (all its loads are inside K); the last 2 STAGES - 1 tiles are
+    // peeled into steps that test what still exists.
+    auto step = [&](auto set_c, auto main_c, int t) __attribute__((always_inline)) {
+        constexpr int U = decltype(set_c)::value, UN = (U + 1) % STAGES;
+        constexpr bool MAIN = decltype(main_c)::value;
+        if (MAIN || t + STAGES < nk) {
+            la.load(ra[U], Ao, (int64_t)(t + STAGES) * BK);
+            lb.load(rb[U], Bo, (int64_t)(t + STAGES) * BK);
+        }
+        compute(t & 1);
+        if (MAIN || t + 1 < nk) {
+            la.store(ra[UN], As + ((t + 1) & 1) * BM * BK);
+            lb.store(rb[UN], Bs + ((t + 1) & 1) * BN * BK);
+        }
+        __syncthreads();
+    };
+    {
+        la.load(ra[0], Ao, (int64_t)kt0 * BK);
+        lb.load(rb[0], Bo, (int64_t)kt0 * BK);
+#pragma unroll
+        for (int u = 1; u < STAGES; u++)
+            if (kt0 + u < nk) {
+                la.load(ra[u], Ao, (int64_t)(kt0 + u) * BK);
+                lb.load(rb[u], Bo, (int64_t)(kt0 + u) * BK);
+            }
         la.store(ra[0], As + (kt0 & 1) * BM * BK);
         lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
         __syncthreads();
         int kt = kt0;
-        for (; kt + 1 < nk; kt += 2) {
-            la.load(ra[0], Ao, tile_k(kt + 2));
-            lb.load(rb[0], Bo, tile_k(kt + 2));
-            compute(kt & 1);
-            la.store(ra[STAGES - 1], As + ((kt + 1) & 1) * BM * BK);
-            lb.store(rb[STAGES - 1], Bs + ((kt + 1) & 1) * BN * BK);
-            __syncthreads();
-            la.load(ra[STAGES - 1], Ao, tile_k(kt + 3));
-            lb.load(rb[STAGES - 1], Bo, tile_k(kt + 3));
-            compute((kt + 1) & 1);
-            la.store(ra[0], As + (kt & 1) * BM * BK);
-            lb.store(rb[0], Bs + (kt & 1) * BN * BK);
-            __syncthreads();
+        for (; kt + 2 * STAGES - 1 < nk; kt += STAGES) {
+            step(std::integral_constant<int, 0>{}, std::true_type{}, kt);
+            if (STAGES > 1) step(std::integral_constant<int, 1 % STAGES>{}, std::true_type{}, kt + 1);
+            if (STAGES > 2) step(std::integral_constant<int, 2 % STAGES>{}, std::true_type{}, kt + 2);
         }
-        if (kt < nk) {                            // odd number of k tiles: the last one is in LDS
-            compute(kt & 1);
-            __syncthreads();
-        }
-    } else {
-        la.load(ra[0], Ao, tile_k(kt0));
-        lb.load(rb[0], Bo, tile_k(kt0));
-        la.store(ra[0], As + (kt0 & 1) * BM * BK);
-        lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
-        __syncthreads();
-        for (int kt = kt0; kt < nk; kt++) {
-            // short-K instantiations skip the load past the last tile (a third of their
-            // traffic when K spans two tiles); the long-K ones keep the loop branch-free
-            const bool more = !KTAIL || kt + 1 < nk;
-            if (more) {
-                la.load(ra[0], Ao, tile_k(kt + 1));
-                lb.load(rb[0], Bo, tile_k(kt + 1));
-            }
-            compute(kt & 1);
-            if (more) {
-                la.store(ra[0], As + ((kt + 1) & 1) * BM * BK);
-                lb.store(rb[0], Bs + ((kt + 1) & 1) * BN * BK);
-            }
-            __syncthreads();
-        }
+        static_assert(STAGES >= 1 && STAGES <= 3, "peeled tail below covers up to 5 tiles");
+        if (kt + 0 < nk) step(std::integral_constant<int, 0 % STAGES>{}, std::false_type{}, kt + 0);
+        if (STAGES > 1 && kt + 1 < nk) step(std::integral_constant<int, 1 % STAGES>{}, std::false_type{}, kt + 1);
+        if (STAGES > 1 && kt + 2 < nk) step(std::integral_constant<int, 2 % STAGES>{}, std::false_type{}, kt + 2);
+        if (STAGES > 2 && kt + 3 < nk) step(std::integral_constant<int, 3 % STAGES>{}, std::false_type{}, kt + 3);
+        if (STAGES > 2 && kt + 4 < nk) step(std::integral_constant<int, 4 % STAGES>{}, std::false_type{}, kt + 4);
     }
 
     // Epilogue through LDS (the operand buffers are free after the last barrier): a lane
