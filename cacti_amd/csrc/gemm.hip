@@ -13,6 +13,8 @@
 //
 // The MFMA is issued with the B fragment as first operand, so a lane ends up with 4
 // consecutive columns of one row of C per accumulator group and stores 8 bytes at a time.
+#include <stdlib.h>
+
 #include "common.h"
 #include "gemm_internal.h"
 
@@ -298,6 +300,8 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nbl
         }
     }
     hipStream_t st = (hipStream_t)stream;
+    if (vec >= 4 && !ta && tb && K <= 128 && beta == 0.f && tri <= 1)
+        return gemm_nt_smallk_launch(p, nblk, st);
     if (vec >= 4) return gemm_mfma_launch(ta, tb, p, nblk, vec, -1, st);
     if (!ta && !tb) return launch_vec<false, false>(vec, p, nblk, st);
     if (!ta && tb) return launch_vec<false, true>(vec, p, nblk, st);

@@ -33,4 +33,8 @@ constexpr int kTriPad = 256;
 int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align, int tile,
                      hipStream_t st);
 
+// C = f16(alpha A B^T) with K <= 128 (attention scores): A [M,K], B [N,K] row-major, rows
+// 8-byte aligned, K % 4 == 0, beta = 0, tri 0 or 1
+int gemm_nt_smallk_launch(const GemmArgs &p, int64_t nblk, hipStream_t st);
+
 }  // namespace cacti

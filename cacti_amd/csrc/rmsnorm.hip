@@ -186,23 +186,28 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
     for (int i = threadIdx.x; i < D; i += blockDim.x) dst[i] = sdw[i];
 }
 
-// dw[d] (+)= f16(sum over block partials); 64 columns x 16 slices per block
-__global__ void __launch_bounds__(1024)
+// dw[d] (+)= f16(sum over block partials): a block owns 32 columns (8 lanes x float4) and
+// splits the partial rows over 32 slices, so D / 32 blocks share the read of the partials
+constexpr int kFinCols = 32, kFinSlices = 32;
+__global__ void __launch_bounds__(kFinCols / 4 * kFinSlices)
 rms_norm_dw_finalize_kernel(int G, int D, const float *__restrict__ part, half_t *dw, int acc)
 {
-    __shared__ float red[16][64];
-    const int col = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int slice = threadIdx.x >> 6;
-    float a = 0.f;
+    __shared__ float red[kFinSlices][kFinCols];
+    const int cg = threadIdx.x & (kFinCols / 4 - 1), slice = threadIdx.x / (kFinCols / 4);
+    const int col = blockIdx.x * kFinCols + cg * 4;            // D % 8 == 0: a float4 is whole
+    float4_t a = {0.f, 0.f, 0.f, 0.f};
     if (col < D)
-        for (int g = slice; g < G; g += 16) a += part[(int64_t)g * D + col];
-    red[slice][threadIdx.x & 63] = a;
+        for (int g = slice; g < G; g += kFinSlices)
+            a += *reinterpret_cast<const float4_t *>(part + (int64_t)g * D + col);
+#pragma unroll
+    for (int i = 0; i < 4; i++) red[slice][cg * 4 + i] = a[i];
     __syncthreads();
-    if (slice == 0 && col < D) {
+    const int c = blockIdx.x * kFinCols + threadIdx.x;
+    if (threadIdx.x < kFinCols && c < D) {
         float s = 0.f;
 #pragma unroll
-        for (int i = 0; i < 16; i++) s += red[i][threadIdx.x];
-        dw[col] = acc ? f2h(h2f(dw[col]) + rnd16(s)) : f2h(s);
+        for (int i = 0; i < kFinSlices; i++) s += red[i][threadIdx.x];
+        dw[c] = acc ? f2h(h2f(dw[c]) + rnd16(s)) : f2h(s);
     }
 }
 
@@ -288,7 +293,8 @@ CACTI_API int cacti_hip_rms_norm_bwd(int64_t N, int64_t D, const void *x, const 
     int rc = launch_status("rms_norm_bwd");
     if (rc) return rc;
     const int G = (int)((N + kWaves - 1) / kWaves);
-    hipLaunchKernelGGL(rms_norm_dw_finalize_kernel, dim3((unsigned)((D + 63) / 64)), dim3(1024), 0,
-                       st, G, (int)D, (const float *)workspace, (half_t *)dw, dw_acc);
+    hipLaunchKernelGGL(rms_norm_dw_finalize_kernel, dim3((unsigned)((D + kFinCols - 1) / kFinCols)),
+                       dim3(kFinCols / 4 * kFinSlices), 0, st, G, (int)D, (const float *)workspace,
+                       (half_t *)dw, dw_acc);
     return launch_status("rms_norm_dw_finalize");
 }

@@ -250,6 +250,7 @@ GEMM_SHAPES = [
     (128, 128, 32), (256, 384, 192), (100, 72, 40), (128, 688, 256), (128, 256, 688),
     (61, 35, 27),            # nothing aligned: scalar path
     (64, 100, 64), (64, 64, 100),   # head_dim 100: 8-byte path
+    (200, 264, 128), (300, 648, 100), (132, 140, 12),   # short K: several column tiles, ragged edges
 ]
 
 
