@@ -64,6 +64,29 @@ def synth_inputs(cfg, seed=1, grad_scale=1024.0):
     return tok, lm_tok, scale
 
 
+# L2-miss traffic per launch of the 128 x 128 GEMM kernel, rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE in KiB per dispatch (profiles/llama3b_step_gemm_hbm_traffic.txt gives the commands);
+# a streaming kernel of known size reads FETCH_SIZE = half its bytes and WRITE_SIZE = its
+# bytes, so bytes = (2.0 * FETCH_SIZE + 1.0 * WRITE_SIZE) * 1024
+GEMM_TRAFFIC_KIB = {
+    ("NT", 2048, 3200, 3200): (53437, 12800), ("NT", 2048, 3200, 8640): (225558, 12800),
+    ("NT", 2048, 8640, 3200): (156643, 34560),
+    ("NN", 2048, 3200, 3200): (61962, 12800), ("NN", 2048, 3200, 8640): (243619, 12800),
+    ("NN", 2048, 8640, 3200): (164838, 34560), ("NN", 2048, 3200, 32000): (1137423, 12800),
+    ("TN", 3200, 3200, 2048): (67231, 20000), ("TN", 8640, 3200, 2048): (164032, 54000),
+    ("TN", 3200, 8640, 2048): (164032, 54000), ("TN", 32000, 3200, 2048): (722906, 200000),
+}
+
+
+def gemm_traffic_bytes(label):
+    m = GEMM_RE.match(label)
+    key = (m.group(2) + m.group(3), int(m.group(5)), int(m.group(6)), int(m.group(7)))
+    if key not in GEMM_TRAFFIC_KIB:
+        return None
+    f, w = GEMM_TRAFFIC_KIB[key]
+    return (2.0 * f + 1.0 * w) * 1024.0
+
+
 GEMM_RE = re.compile(r"^(block_matmul|matmul)\[([NT])([NT]),(\d+)x(\d+)x(\d+)x(\d+)(,acc)?\]$")
 
 
@@ -188,10 +211,14 @@ def run_step(args):
     cnt = sum(c for c, _ in rep.values())
     assert all(kernel_symbol(label) == sym for label in rep), (sym, list(rep))
     achieved = fl / sec / 1e12
+    tr = [(gemm_traffic_bytes(label), c) for label, (c, _) in rep.items()]
+    traffic = None if any(t is None for t, _ in tr) else sum(t * c for t, c in tr) / cnt
     roofline = {"bound": "mfma", "kernel": sym, "timed_launches": cnt,
                 "avg_launch_us": sec / cnt * 1e6, "flops_per_launch": fl / cnt,
                 "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": None}
+                "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": traffic,
+                "traffic_note": "bytes per launch leaving the L2s (MALL or HBM), mean over the timed "
+                                "launches; per-shape counter readings measured offline"}
     out = {
         "metric": "fwd+bwd tokens/sec, 3B-shaped fp16 step, 1 GPU", "value": tokens_s,
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
