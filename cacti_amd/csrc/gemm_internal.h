@@ -25,6 +25,7 @@ struct GemmArgs {
     // of 256 columns; beyond that they are never read.
     int tri;
     int gm, xcd;          // tile walk: rows per group; 1 = XCD-banded numbering
+    int pair;             // 1: a workgroup computes tile rows r and tiles_m - 1 - r (tri 2 / 3)
 };
 constexpr int kTriPad = 256;
 

@@ -420,7 +420,10 @@ gemm_mfma_kernel(GemmArgs p)
         const int xcd = bid & 7, idx = bid >> 3;
         bid = xcd * per + (xcd < rem ? xcd : rem) + idx;
     }
-    const int tiles = p.tiles_m * p.tiles_n;
+    // pair mode (triangular operands): a workgroup takes tile row r and then tile row
+    // tiles_m - 1 - r, whose k ranges add up to the same length for every r
+    const int rows_m = p.pair ? p.tiles_m / 2 : p.tiles_m;
+    const int tiles = rows_m * p.tiles_n;
     const int64_t bz = bid / tiles;
     bid -= (int)bz * tiles;
     // within a block of the batch, tiles are walked in groups of 8 tile rows x all tile
@@ -429,10 +432,12 @@ gemm_mfma_kernel(GemmArgs p)
     const int GM = p.gm;
     const int per_group = GM * p.tiles_n;
     const int first_m = (bid / per_group) * GM;
-    const int gsz = min(GM, p.tiles_m - first_m);
-    int tm = first_m + (bid % per_group) % gsz;
+    const int gsz = min(GM, rows_m - first_m);
+    const int tm_base = first_m + (bid % per_group) % gsz;
     const int tn = (bid % per_group) / gsz;
-    if (p.tri == 2) tm = p.tiles_m - 1 - tm;                      // longest k ranges first
+    for (int rep = 0; rep <= p.pair; rep++) {
+    int tm = rep ? p.tiles_m - 1 - tm_base : tm_base;
+    if (p.tri == 2 && !p.pair) tm = p.tiles_m - 1 - tm;           // longest k ranges first
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
 
     int nk = (int)((p.K + BK - 1) / BK), kt0 = 0;
@@ -638,6 +643,8 @@ gemm_mfma_kernel(GemmArgs p)
             if (p.N - n > 4) *reinterpret_cast<uint2 *>(cp + 4) = make_uint2(v.z, v.w);
         }
     }
+    __syncthreads();                          // the staging buffer is read out before the next tile's operands land
+    }
 }
 
 template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
@@ -653,7 +660,8 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
                                       (int)smem));
         attr_set = true;
     }
-    const int64_t nwg = (int64_t)p.tiles_m * p.tiles_n * nblk;
+    p.pair = (p.tri >= 2 && p.tiles_m % 2 == 0) ? 1 : 0;
+    const int64_t nwg = (int64_t)(p.pair ? p.tiles_m / 2 : p.tiles_m) * p.tiles_n * nblk;
     CACTI_REQUIRE(nwg < (int64_t)1 << 31, CACTI_E_NOTIMPL, "gemm: %lld workgroups exceed the grid limit",
                   (long long)nwg);
     dim3 grid((unsigned)nwg), block(WM * WN * 64);
