@@ -512,6 +512,14 @@ int Ctx::compile()
     std::vector<Entry> out;
     out.reserve(log_.size() * 2);
     for (size_t i = 0; i < log_.size(); i++) {
+        Entry &e = log_[i];
+        // first-write copy (the memcpy adjoint) of a cell that is used nowhere else afterwards:
+        // same bytes under a new name, so the output adopts the source's storage
+        if (e.kind == E_APPLY && thunks_[e.thunk]->is_copy() && e.acc_mask == 0 &&
+            !cells_[e.args[0]].stable && !cells_[e.outs[0]].stable && e.args[0] != e.outs[0] &&
+            cells_[e.args[0]].ty.bytes() == cells_[e.outs[0]].ty.bytes() &&
+            std::find(dies[i].begin(), dies[i].end(), e.args[0]) != dies[i].end())
+            e.move = true;
         out.push_back(std::move(log_[i]));
         std::sort(dies[i].begin(), dies[i].end());
         for (CellPtr c : dies[i]) {
@@ -536,6 +544,21 @@ const char *Ctx::entry_name(size_t i) const
 
 int Ctx::run_entry(const Entry &e)
 {
+    if (e.move) {
+        const CellPtr si = e.args[0], di = e.outs[0];
+        int rc = ensure_vmem(si, true);           // re-uploads a spilled source
+        if (rc) return rc;
+        Cell &src = cells_[si], &dst = cells_[di];
+        CACTI_REQUIRE(dst.alive, CACTI_E_STATE, "move into dead cell %d (%s)", di, dst.name.c_str());
+        if (dst.voff != kNoOffset) pool_.free(dst.voff);
+        dst.voff = src.voff;
+        dst.v_valid = true;
+        dst.h_valid = false;
+        src.voff = kNoOffset;
+        src.v_valid = false;
+        n_moved_++;
+        return 0;
+    }
     const ThunkSpec &sp = *thunks_[e.thunk];
     std::vector<CellType> aty, oty;
     for (CellPtr a : e.args) cells_[a].pin++;

@@ -95,6 +95,9 @@ struct ThunkSpec {
     virtual const char *name() const = 0;
     virtual int arity() const = 0;
     virtual int nout() const { return 1; }
+    // a plain copy of argument 0 into output 0 (lets the runtime hand over the storage of a
+    // source that dies at this entry instead of copying it)
+    virtual bool is_copy() const { return false; }
     virtual int out_ty(const std::vector<CellType> &arg, std::vector<CellType> &out) const = 0;
     virtual size_t workspace(const std::vector<CellType> &) const { return 0; }
     // label under which launches are grouped in the timing report (name + shape for GEMMs)
@@ -113,6 +116,7 @@ struct Entry {
     int thunk = -1;
     std::vector<CellPtr> args, outs;
     uint32_t acc_mask = 0;
+    bool move = false;       // copy whose source dies here: the output takes over its storage
     CellPtr cell = 0;        // E_YIELD_SET / E_UNLIVE
 };
 
@@ -208,6 +212,7 @@ class Ctx {
     // statistics
     uint64_t n_alloc_ = 0, n_evict_ = 0, n_upload_ = 0, bytes_d2h_ = 0, bytes_h2d_ = 0,
              n_soft_oom_ = 0, n_run_ = 0, host_bytes_ = 0;
+    uint64_t n_moved_ = 0;
     int timing_ = 0;
     std::string timing_filter_;
     int timing_every_ = 1;

@@ -14,6 +14,7 @@ inline void *S(Ctx &c) { return (void *)c.stream(); }
 struct CopySpec : ThunkSpec {
     const char *name() const override { return "copy"; }
     int arity() const override { return 1; }
+    bool is_copy() const override { return true; }
     int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
     {
         o = {a[0]};
