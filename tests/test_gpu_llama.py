@@ -147,3 +147,52 @@ def test_pool_too_small_is_a_clean_error(oracle):
         m.step(tok, lm_tok, scale)
     assert e.value.code == -4
     m.close(); ctx.close()
+
+
+def test_full_size_step_properties():
+    """BASELINE's configuration at full shapes (S=2048, D=3200, H=32 x 100, F=8640, V=32000) with
+    4 of the 26 layers (the oracle would need a minute per layer): properties that hold at any
+    size.  (a) the loss is -log softmax(logit)[target] of the logits the step returns, recomputed
+    in fp64; (b) a second cycle is bit-identical; (c) doubling the loss scale (a power of two)
+    doubles the gradients: every product and sum on the adjoint path is homogeneous in the
+    scale, so elements differ only where a value on the way was an f16 subnormal; (d) embedding rows
+    of ids that do not occur get a zero gradient, rows that occur a non-zero one."""
+    import bench
+    from cacti_amd.runtime import Ctx, Llama
+    cfg = dict(bench.LLAMA_3B, L=4)
+    ctx = Ctx(0, 24 << 30, True)
+    m = Llama(ctx, **cfg)
+    bench.synth_params(m)
+    tok, lm_tok, scale = bench.synth_inputs(cfg, grad_scale=8192.0)
+    out = m.step_explicit(tok, lm_tok, scale)
+    lg = out["logit"].astype(np.float64)
+    lse = np.log(np.exp(lg - lg.max(1, keepdims=True)).sum(1)) + lg.max(1)
+    want_loss = lse - lg[np.arange(cfg["S"]), lm_tok]
+    assert np.all(np.isfinite(out["loss"]))
+    assert np.abs(out["loss"] - want_loss).max() < 2e-3 * max(1.0, np.abs(want_loss).max())
+    assert np.mean(out["amax"] == lg.argmax(1)) > 0.999
+
+    idx = {name: i for i, (name, _) in enumerate(m.params)}
+    probe = ["embed", "l0.q", "l0.pre_norm", "l1.down", "l3.gate", "l3.v", "head_norm", "lm_head"]
+    g1 = {n: m.grad(idx[n]) for n in probe}
+    m.step(tok, lm_tok, scale, want_loss=False)
+    for n in probe:
+        assert np.array_equal(m.grad(idx[n]).view(np.uint16), g1[n].view(np.uint16)), n
+
+    present = np.zeros(cfg["V"], bool)
+    present[tok] = True
+    rows = np.abs(g1["embed"].astype(np.float32)).max(1)
+    assert np.all(rows[~present] == 0) and np.mean(rows[present] > 0) > 0.99
+
+    m.step(tok, lm_tok, 2.0 * scale, want_loss=False)
+    tiny = 2.0 ** -14
+    for n in probe:
+        a, b = g1[n].astype(np.float32), m.grad(idx[n]).astype(np.float32)
+        ok = (np.abs(a) >= tiny) & (np.abs(b) < 65504)
+        assert ok.mean() > 0.03, (n, ok.mean())      # embed: only rows of ids that occur
+        same = float(np.mean(b[ok] == 2.0 * a[ok]))
+        err = rel_l2(b, 2.0 * a)
+        print("scale x2: %-12s %.4f of the normal elements doubled exactly, rel_l2 %.2e" % (n, same, err),
+              flush=True)
+        assert err < 5e-3, (n, same, err)
+    m.close(); ctx.close()
