@@ -306,17 +306,18 @@ struct LoadKS2 {
     static constexpr int NREG = 8;
 };
 
-// ---- one k-strided operand, every lane of the block taking part: an item is 4 k x 8 rows
-// (half of LoadKS's), so ROWS * 2 items spread over exactly NT lanes with no idle
-// wavefronts and no branch in the k loop.  Each of the 8 tile rows of an item gets 4 k
-// values (8 bytes of its 16-byte k chunk).
+// ---- one k-strided operand, every lane of the block taking part: an item is KPI k x 8 rows
+// (KPI = 4 or 2, a half or a quarter of LoadKS's), so that the ROWS / 8 x 64 / KPI items spread
+// over exactly NT lanes with no idle wavefronts and no branch in the k loop.  Each of the 8
+// tile rows of an item gets KPI k values (2 KPI bytes of its 16-byte k chunk).
 template <int ROWS, int NT, int AL, bool KTAIL>
 struct LoadKSH {
-    static_assert(ROWS * 2 == NT, "one half item per lane");
     static constexpr int RC = ROWS / 8;
+    static constexpr int KPI = BK * RC / NT;
+    static_assert(KPI == 4 || KPI == 2, "a half or a quarter item per lane");
     uint32_t off, off1, ldb2;
     int64_t ld, K;
-    int rc, kq4;                   // row chunk; group of 4 k rows (0..15)
+    int rc, kq;                    // row chunk; group of KPI k rows
 
     __device__ __forceinline__ void init(int64_t ld_, int64_t rows_left, int64_t K_)
     {
@@ -324,7 +325,7 @@ struct LoadKSH {
         K = K_;
         ldb2 = (uint32_t)(ld_ * 2);
         rc = threadIdx.x % RC;
-        kq4 = threadIdx.x / RC;
+        kq = threadIdx.x / RC;
         int r0 = rc * 8, r1 = rc * 8 + 4;
         if (AL == 8) {
             if (r0 > rows_left - 8) r0 = (int)rows_left - 8;
@@ -332,18 +333,18 @@ struct LoadKSH {
             if (r0 > rows_left - 4) r0 = (int)rows_left - 4;
             if (r1 > rows_left - 4) r1 = (int)rows_left - 4;
         }
-        off = (uint32_t)(((int64_t)kq4 * 4 * ld + r0) * 2);
-        off1 = (uint32_t)(((int64_t)kq4 * 4 * ld + r1) * 2);
+        off = (uint32_t)(((int64_t)kq * KPI * ld + r0) * 2);
+        off1 = (uint32_t)(((int64_t)kq * KPI * ld + r1) * 2);
     }
     __device__ __forceinline__ void load(uint4 *st, const half_t *origin, int64_t k0) const
     {
         const half_t *base = origin + k0 * ld;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
+        for (int kk = 0; kk < KPI; kk++) {
             if (!KTAIL || k0 + BK <= K) {
                 st[kk] = ld8<AL>(base, off + kk * ldb2, off1 + kk * ldb2);
             } else {
-                const int left = (int)(K - k0) - (kq4 * 4 + kk);
+                const int left = (int)(K - k0) - (kq * KPI + kk);
                 const uint32_t back = left > 0 ? 0 : (uint32_t)(1 - left) * ldb2;
                 uint4 v = ld8<AL>(base, off + kk * ldb2 - back, off1 + kk * ldb2 - back);
                 if (left <= 0) v = make_uint4(0, 0, 0, 0);
@@ -354,16 +355,23 @@ struct LoadKSH {
     __device__ __forceinline__ void store(const uint4 *st, half_t *lds) const
     {
         const uint32_t *w = reinterpret_cast<const uint32_t *>(st);       // [kk][4 words]
+        const int k = kq * KPI;                                           // first k of the item
+        half_t *dst = lds + (k & 7);
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-            uint2 o;
-            o.x = __builtin_amdgcn_perm(w[1 * 4 + (j >> 1)], w[0 * 4 + (j >> 1)], sel);
-            o.y = __builtin_amdgcn_perm(w[3 * 4 + (j >> 1)], w[2 * 4 + (j >> 1)], sel);
-            *reinterpret_cast<uint2 *>(lds + lds_off(rc * 8 + j, kq4 >> 1) + (kq4 & 1) * 4) = o;
+            const uint32_t lo = __builtin_amdgcn_perm(w[1 * 4 + (j >> 1)], w[0 * 4 + (j >> 1)], sel);
+            if (KPI == 4) {
+                uint2 o;
+                o.x = lo;
+                o.y = __builtin_amdgcn_perm(w[(KPI - 1) * 4 + (j >> 1)], w[(KPI - 2) * 4 + (j >> 1)], sel);
+                *reinterpret_cast<uint2 *>(dst + lds_off(rc * 8 + j, k >> 3)) = o;
+            } else {
+                *reinterpret_cast<uint32_t *>(dst + lds_off(rc * 8 + j, k >> 3)) = lo;
+            }
         }
     }
-    static constexpr int NREG = 4;
+    static constexpr int NREG = KPI;
 };
 
 // stands in for the B loader when LoadKS2 serves both operands
@@ -458,8 +466,11 @@ gemm_mfma_kernel(GemmArgs p)
 
     // when both operands are strided they use disjoint halves of the block
     constexpr bool UNI = TA && !TB && BM == BN && BM + BN == NT;  // one combined strided loader
-    // exactly one strided operand and a 128-row tile on 256 lanes: half items on every lane
-    constexpr bool HALF_A = TA && TB && BM * 2 == NT, HALF_B = !TA && !TB && BN * 2 == NT;
+    // strided operands whose 8-row x 64-k items divide into 4- or 2-k pieces over all lanes
+    // (128 rows on 256 lanes, 256 or 128 rows on 512 lanes): branch-free on every lane
+    constexpr bool FITS_A = BM * 2 == NT || BM * 4 == NT, FITS_B = BN * 2 == NT || BN * 4 == NT;
+    constexpr bool HALF_A = TA && !UNI && FITS_A && (TB || FITS_B);
+    constexpr bool HALF_B = !TB && !UNI && FITS_B && (!TA || FITS_A);
     typedef typename std::conditional<
         UNI, LoadKS2<BM, NT, AL, KTAIL>,
         typename std::conditional<HALF_A, LoadKSH<BM, NT, AL, KTAIL>,
@@ -685,7 +696,7 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
     if (ktail) return launch_cfg<TA, TB, 128, 128, 2, 2, 8, true, 1>(p, nblk, st);
     switch (tile) {
         case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8, false, S0>(p, nblk, st);
-        case 1: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 1>(p, nblk, st);
+        case 1: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
         case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1>(p, nblk, st);
         default: return launch_cfg<TA, TB, 256, 256, 2, 2, 8, false, 1>(p, nblk, st);
     }
@@ -726,6 +737,12 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             // the chip several times over (the LM-head forward)
             const int64_t big = ((p.M + 255) / 256) * ((p.N + 255) / 256) * nblk;
             tile = (!ta && tb && big >= 768) ? 3 : 0;
+            // A not transposed (forward and dgrad products, M = tokens): one 8-wave 256 x 128
+            // workgroup per CU fetches each B panel half as often as two 128 x 128 ones
+            // (measured +8..14 % on the projection and FFN shapes; the wgrad layout loses 5..17 %
+            // to its coarser tile count and stays on 128 x 128)
+            static const bool wide = !getenv("CACTI_GEMM_NO_NT256");
+            if (wide && !ta && tile == 0 && nblk == 1 && p.M >= 1024 && p.N >= 1024) tile = 1;
         }
     }
     if (!ta && !tb) return launch_tile<false, false>(tile, align, q, nblk, st);
