@@ -100,19 +100,13 @@ def gemm_flops(label):
 
 def kernel_symbol(label):
     """Name of the HIP kernel instantiation a dense GEMM label runs on, as rocprofv3 prints it
-    (the tile choice mirrors gemm_mfma_launch: 256 x 256 / 4 waves for k-contiguous operands
-    when that still gives 768 tiles; else 256 x 128 / 8 waves when A is not transposed and the
-    output is at least 1024 x 1024; else 128 x 128 / 4 waves; two register stages)."""
+    (the tile choice mirrors gemm_mfma_launch: 256 x 128 / 8 waves when A is not transposed and
+    the output is at least 1024 x 1024, else 128 x 128 / 4 waves; two register stages)."""
     m = GEMM_RE.match(label)
     ta, tb = m.group(2) == "T", m.group(3) == "T"
     H, M, N = int(m.group(4)), int(m.group(5)), int(m.group(6))
-    big = ((M + 255) // 256) * ((N + 255) // 256) * H
-    if not ta and tb and big >= 768:
-        tile = "256, 256, 2, 2, 8, false, 1"
-    elif not ta and H == 1 and M >= 1024 and N >= 1024:
-        tile = "256, 128, 4, 2, 8, false, 2"
-    else:
-        tile = "128, 128, 2, 2, 8, false, 2"
+    wide = not ta and H == 1 and M >= 1024 and N >= 1024
+    tile = "256, 128, 4, 2, 8, false, 2" if wide else "128, 128, 2, 2, 8, false, 2"
     return "gemm_mfma_kernel<%s, %s, %s>" % (str(ta).lower(), str(tb).lower(), tile)
 
 

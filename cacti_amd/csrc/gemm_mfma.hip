@@ -3,8 +3,9 @@
 //
 //   C[M,N] = alpha op(A) op(B) + beta C,   f16 in, fp32 MFMA accumulate, f16 out.
 //
-// Block tile BM x BN x 64, WM x WN wavefronts, each owning a (BM/WM) x (BN/WN) patch of
-// 32 x 32 accumulators fed by v_mfma_f32_32x32x16_f16.
+// Block tile BM x BN x 64, WM x WN wavefronts, each owning a 64 x 64 patch of 32 x 32
+// accumulators fed by v_mfma_f32_32x32x16_f16.  Two shapes are instantiated: 128 x 128 on 4
+// waves (two workgroups per CU) and 256 x 128 on 8 waves (one per CU).
 //
 // LDS layout (both operands): [row][64 k] = 128 bytes per row, no padding; the 16-byte
 // k-chunk q of row r sits at chunk position q ^ f(r), f(r) = (r ^ (r >> 3)) & 7.
@@ -14,9 +15,10 @@
 // LDS line, and 16 consecutive rows also spread over both halves of a 256-byte line.
 //
 // An operand whose k index is not contiguous in memory (A^T, or B not transposed) is
-// loaded as 8 k-rows x 8 tile-rows per lane with fully coalesced 16-byte loads, transposed
-// in registers with 32 v_perm_b32, and written as 8 16-byte rows: the MFMA read path is
-// identical for NN / NT / TN / TT.
+// loaded as blocks of k-rows x 8 tile-rows per lane with fully coalesced 16-byte loads,
+// transposed in registers with v_perm_b32, and written as 8 row pieces: the MFMA read path is
+// identical for NN / NT / TN / TT.  The block of a lane is 8, 4 or 2 k-rows deep, whichever
+// spreads the operand tile over every lane of the workgroup.
 //
 // The main loop has no branch: every lane's global offsets (32-bit, relative to the tile
 // origin, clamped into the operand) are computed once, a k step only moves a uniform base
@@ -405,7 +407,7 @@ struct SchedStep<NM, NR, NR> {
 
 // waves per SIMD the register allocation must leave room for: two 128 x 128 blocks (or one
 // 8-wave block) per CU, one 4-wave 256 x 256 block
-constexpr int min_waves(int bm, int bn, int nwaves) { return (bm * bn <= 128 * 128 || nwaves == 8) ? 2 : 1; }
+constexpr int min_waves(int, int, int) { return 2; }              // both tile shapes: 8 waves per CU
 
 template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
 __global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN))
@@ -508,8 +510,8 @@ gemm_mfma_kernel(GemmArgs p)
         const half_t *as = As + cur * BM * BK + ar0 * BK;
         const half_t *bs = Bs + cur * BN * BK + br0 * BK;
         // fragment double-buffering costs (TM + TN) * 4 registers: used where it fits without
-        // spilling (16-byte aligned operands, all but the 8-wave 256 x 256 tile)
-        constexpr bool PIPE = AL == 8 && !(BM * BN == 256 * 256 && WM * WN == 8);
+        // spilling (16-byte aligned operands)
+        constexpr bool PIPE = AL == 8;
         half8_t af[PIPE ? 2 : 1][TM], bf[PIPE ? 2 : 1][TN];
         auto frags = [&](int set, int ks) __attribute__((always_inline)) {
             const int q = ks * 2 + lh;
@@ -696,9 +698,7 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
     if (ktail) return launch_cfg<TA, TB, 128, 128, 2, 2, 8, true, 1>(p, nblk, st);
     switch (tile) {
         case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8, false, S0>(p, nblk, st);
-        case 1: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
-        case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1>(p, nblk, st);
-        default: return launch_cfg<TA, TB, 256, 256, 2, 2, 8, false, 1>(p, nblk, st);
+        default: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
     }
 }
 
@@ -706,8 +706,7 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
 
 namespace cacti {
 
-// tile: 0 = 128x128 (4 waves), 1 = 256x128 (8 waves), 2 = 256x256 (8 waves), 3 = 256x256
-// (4 waves); -1 = pick by shape
+// tile: 0 = 128x128 (4 waves), 1 = 256x128 (8 waves); -1 = pick by shape
 int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align, int tile,
                      hipStream_t st)
 {
@@ -732,15 +731,12 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
         if (forced >= 0) {
             tile = forced;
         } else {
-            // measured on MI355X at the step's shapes: 128 x 128 (two blocks per CU) wins
-            // everywhere except the k-contiguous (NT) case when 256 x 256 tiles still fill
-            // the chip several times over (the LM-head forward)
-            const int64_t big = ((p.M + 255) / 256) * ((p.N + 255) / 256) * nblk;
-            tile = (!ta && tb && big >= 768) ? 3 : 0;
-            // A not transposed (forward and dgrad products, M = tokens): one 8-wave 256 x 128
-            // workgroup per CU fetches each B panel half as often as two 128 x 128 ones
-            // (measured +8..14 % on the projection and FFN shapes; the wgrad layout loses 5..17 %
-            // to its coarser tile count and stays on 128 x 128)
+            // measured on MI355X at the step's shapes.  A not transposed (forward and dgrad
+            // products, M = tokens): one 8-wave 256 x 128 workgroup per CU fetches each B panel
+            // half as often as two 128 x 128 ones (+8..14 % on the projection and FFN shapes, and
+            // the best choice for the LM head too).  The wgrad layout loses 5..17 % to its
+            // coarser tile count and stays on 128 x 128, as do small and batched products.
+            tile = 0;
             static const bool wide = !getenv("CACTI_GEMM_NO_NT256");
             if (wide && !ta && tile == 0 && nblk == 1 && p.M >= 1024 && p.N >= 1024) tile = 1;
         }
