@@ -269,41 +269,62 @@ __global__ void __launch_bounds__(kThreads) fill_zero16_kernel(uint4 *p, int64_t
 
 // Scatter-add, deterministic: the block of position s owns row tok[s] iff s is the
 // first position holding that id; it then sums the dy rows of every position with
-// the same id in position order in fp32 and rounds once.
+// the same id in position order in fp32 and rounds once.  The later positions of the id are
+// collected, in order, by the first wave with ballots (64 positions per step), so a block
+// with duplicates costs a few microseconds instead of a serial scan by every lane.
 __global__ void __launch_bounds__(kThreads)
 embed_bwd_kernel(int64_t V, int64_t D, int64_t S, const uint16_t *__restrict__ tok,
                  const half_t *__restrict__ dy, half_t *dW, int acc)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    uint16_t *ids = reinterpret_cast<uint16_t *>(smem_raw);
+    uint16_t *ids = reinterpret_cast<uint16_t *>(smem_raw);           // [S]
+    uint16_t *dup = ids + S;                                          // [S] later positions of the id
+    __shared__ int ndup;
     const int64_t s = blockIdx.x;
     for (int64_t j = threadIdx.x; j < S; j += blockDim.x) ids[j] = tok[j];
     __syncthreads();
     const uint16_t id = ids[s];
     if ((int64_t)id >= V) return;
-    int earlier = 0, later = 0;
-    for (int64_t j = threadIdx.x; j < S; j += blockDim.x) {
-        if (ids[j] == id) {
-            earlier += (j < s);
-            later += (j > s);
-        }
-    }
+    int earlier = 0;
+    for (int64_t j = threadIdx.x; j < s; j += blockDim.x) earlier += ids[j] == id;
     earlier = __syncthreads_count(earlier);
     if (earlier) return;
-    later = __syncthreads_count(later);
+    if (threadIdx.x < 64) {
+        int n = 0;
+        for (int64_t j0 = s + 1; j0 < S; j0 += 64) {
+            const int64_t j = j0 + threadIdx.x;
+            unsigned long long m = __ballot(j < S && ids[j] == id);
+            while (m) {
+                const int b = __builtin_ctzll(m);
+                if (threadIdx.x == 0) dup[n] = (uint16_t)(j0 + b);
+                n++;
+                m &= m - 1;
+            }
+        }
+        if (threadIdx.x == 0) ndup = n;
+    }
+    __syncthreads();
+    const int n = ndup;
     half_t *dst = dW + (int64_t)id * D;
     for (int c = threadIdx.x; c < D / 8; c += blockDim.x) {
         h8 v = ld8(dy + s * D + c * 8);
         float a[8];
 #pragma unroll
         for (int i = 0; i < 8; i++) a[i] = h2f(v.v[i]);
-        if (later) {
-            for (int64_t j = s + 1; j < S; j++) {
-                if (ids[j] != id) continue;
-                h8 w = ld8(dy + j * D + c * 8);
+        int t = 0;
+        for (; t + 4 <= n; t += 4) {                  // four independent loads in flight
+            h8 w[4];
 #pragma unroll
-                for (int i = 0; i < 8; i++) a[i] += h2f(w.v[i]);
-            }
+            for (int u = 0; u < 4; u++) w[u] = ld8(dy + (int64_t)dup[t + u] * D + c * 8);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) a[i] += h2f(w[u].v[i]);
+        }
+        for (; t < n; t++) {
+            const h8 w = ld8(dy + (int64_t)dup[t] * D + c * 8);
+#pragma unroll
+            for (int i = 0; i < 8; i++) a[i] += h2f(w.v[i]);
         }
         h8 r;
         if (acc) {
@@ -471,8 +492,8 @@ CACTI_API int cacti_hip_embed_bwd(int64_t V, int64_t D, int64_t S, const void *t
 {
     CACTI_REQUIRE(V > 0 && D > 0 && S > 0 && tok && dy && dW, CACTI_E_INVALID,
                   "embed_bwd: null pointer or empty shape");
-    CACTI_REQUIRE(D % 8 == 0 && S <= 32768, CACTI_E_NOTIMPL,
-                  "embed_bwd: need D %% 8 == 0 and S <= 32768 (D=%lld S=%lld)", (long long)D,
+    CACTI_REQUIRE(D % 8 == 0 && S <= 16384, CACTI_E_NOTIMPL,      // 4 S bytes of LDS per block
+                  "embed_bwd: need D %% 8 == 0 and S <= 16384 (D=%lld S=%lld)", (long long)D,
                   (long long)S);
     CACTI_REQUIRE(aligned(dy, 16) && aligned(dW, 16), CACTI_E_INVALID,
                   "embed_bwd: tensors must be 16-byte aligned");
@@ -481,7 +502,7 @@ CACTI_API int cacti_hip_embed_bwd(int64_t V, int64_t D, int64_t S, const void *t
         hipLaunchKernelGGL(fill_zero16_kernel, dim3(grid_for(n16, kThreads, 8192)), dim3(kThreads),
                            0, (hipStream_t)stream, (uint4 *)dW, n16);
     }
-    hipLaunchKernelGGL(embed_bwd_kernel, dim3((unsigned)S), dim3(kThreads), (size_t)S * 2,
+    hipLaunchKernelGGL(embed_bwd_kernel, dim3((unsigned)S), dim3(kThreads), (size_t)S * 4,
                        (hipStream_t)stream, V, D, S, (const uint16_t *)tok, (const half_t *)dy,
                        (half_t *)dW, acc);
     return launch_status("embed_bwd");
