@@ -317,12 +317,25 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
     c.stage_yield_set(m->in_lm_tok);
     c.stage_yield_set(m->in_loss_scale);
 
-    CellPtr stream;
+    // The residual stream enters every norm as the sum of two cells (x1 = stream + o,
+    // x2 = x1 + down, llama.rs:512-532); sum and norm are staged as one fused thunk with both
+    // outputs.  `add_a`, `add_b`: the pending sum's operands (0: `stream` is a plain cell).
+    CellPtr stream, add_a = 0, add_b = 0;
+    auto norm_of_stream = [&](CellPtr w, CellPtr *y) -> int {
+        if (!add_a) return ap(c, make_rms_norm(g.eps), {stream, w}, y);
+        std::vector<CellPtr> outs;
+        int rc = c.stage_apply(c.add_thunk(make_add_rms_norm(g.eps)), {add_a, add_b, w}, &outs);
+        if (rc) return rc;
+        stream = outs[0];
+        *y = outs[1];
+        add_a = add_b = 0;
+        return 0;
+    };
     TRY(ap(c, make_embed(), {m->embed, m->in_tok}, &stream));
     for (size_t l = 0; l < m->layers.size(); l++) {
         const LayerCells &w = m->layers[l];
-        CellPtr pre, q, k, v, qr, kr, s16, p16, attn, o, x1, post, up, gate, h, down, x2;
-        TRY(ap(c, make_rms_norm(g.eps), {stream, w.pre_norm}, &pre));
+        CellPtr pre, q, k, v, qr, kr, s16, p16, attn, o, post, up, gate, h, down;
+        TRY(norm_of_stream(w.pre_norm, &pre));
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.q}, &q));
         TRY(ap(c, make_rope(g.H), {q, m->cos, m->sin}, &qr));
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
@@ -332,17 +345,18 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
         TRY(ap(c, make_causal_softmax(g.H), {s16}, &p16));
         TRY(ap(c, make_causal_pv(g.H), {p16, v}, &attn));
         TRY(ap(c, make_matmul(false, true, 1.f), {attn, w.o}, &o));
-        TRY(ap(c, make_add(), {stream, o}, &x1));
-        TRY(ap(c, make_rms_norm(g.eps), {x1, w.post_norm}, &post));
+        add_a = stream;                                       // x1 = stream + o
+        add_b = o;
+        TRY(norm_of_stream(w.post_norm, &post));
         TRY(ap(c, make_matmul(false, true, 1.f), {post, w.up}, &up));
         TRY(ap(c, make_matmul(false, true, 1.f), {post, w.gate}, &gate));
         TRY(ap(c, make_silu_gate(), {gate, up}, &h));
         TRY(ap(c, make_matmul(false, true, 1.f), {h, w.down}, &down));
-        TRY(ap(c, make_add(), {x1, down}, &x2));
-        stream = x2;
+        add_a = stream;                                       // x2 = x1 + down
+        add_b = down;
     }
     CellPtr hn, logit;
-    TRY(ap(c, make_rms_norm(g.eps), {stream, m->head_norm}, &hn));
+    TRY(norm_of_stream(m->head_norm, &hn));
     TRY(ap(c, make_matmul(false, true, 1.f), {hn, m->lm_head}, &logit));
     std::vector<CellPtr> outs;
     TRY(c.stage_apply(c.add_thunk(make_softmax_ce(want_prob != 0)), {logit, m->in_lm_tok}, &outs));

@@ -16,10 +16,13 @@ namespace {
 constexpr int kWaves = 8;                 // rows per block
 constexpr int kThreads = kWaves * 64;
 
+// x2 != nullptr: the row is first formed as x = f16(x + x2) (the residual add in front of the
+// norm, one thunk boundary) and also written to `sum`
 template <int CH>
 __global__ void __launch_bounds__(kThreads)
-rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t *__restrict__ w,
-                    float eps, half_t *__restrict__ y)
+rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t *__restrict__ x2,
+                    const half_t *__restrict__ w, float eps, half_t *__restrict__ sum,
+                    half_t *__restrict__ y)
 {
     const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
     const int64_t n = (int64_t)blockIdx.x * kWaves + wid;
@@ -33,6 +36,12 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         const int ch = c * 64 + lane;
         if (ch < nchunk) {
             xv[c] = ld8(xr + ch * 8);
+            if (x2) {
+                const h8 bv = ld8(x2 + n * D + ch * 8);
+#pragma unroll
+                for (int i = 0; i < 8; i++) xv[c].v[i] = f2h(h2f(xv[c].v[i]) + h2f(bv.v[i]));
+                st8(sum + n * D + ch * 8, xv[c]);
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 float f = h2f(xv[c].v[i]);
@@ -214,11 +223,11 @@ rms_norm_dw_finalize_kernel(int G, int D, const float *__restrict__ part, half_t
 inline int ch_for(int64_t D) { return (int)((D / 8 + 63) / 64); }
 
 template <int CH>
-void launch_fwd(int64_t N, int D, const half_t *x, const half_t *w, float eps, half_t *y,
-                hipStream_t st)
+void launch_fwd(int64_t N, int D, const half_t *x, const half_t *x2, const half_t *w, float eps,
+                half_t *sum, half_t *y, hipStream_t st)
 {
     hipLaunchKernelGGL(rms_norm_fwd_kernel<CH>, dim3((unsigned)((N + kWaves - 1) / kWaves)),
-                       dim3(kThreads), 0, st, N, D, x, w, eps, y);
+                       dim3(kThreads), 0, st, N, D, x, x2, w, eps, sum, y);
 }
 template <int CH>
 void launch_bwd(int64_t N, int D, const half_t *x, const half_t *w, float eps, const half_t *dy,
@@ -260,9 +269,24 @@ CACTI_API int cacti_hip_rms_norm_fwd(int64_t N, int64_t D, const void *x, const 
                   "rms_norm_fwd: need D %% 8 == 0 and D <= 8192 (D=%lld)", (long long)D);
     CACTI_REQUIRE(aligned(x, 16) && aligned(w, 16) && aligned(y, 16), CACTI_E_INVALID,
                   "rms_norm_fwd: tensors must be 16-byte aligned");
-    CACTI_DISPATCH_CH(ch_for(D), launch_fwd<CH>(N, (int)D, (const half_t *)x, (const half_t *)w,
-                                                eps, (half_t *)y, (hipStream_t)stream));
+    CACTI_DISPATCH_CH(ch_for(D), launch_fwd<CH>(N, (int)D, (const half_t *)x, nullptr, (const half_t *)w,
+                                                eps, nullptr, (half_t *)y, (hipStream_t)stream));
     return launch_status("rms_norm_fwd");
+}
+
+CACTI_API int cacti_hip_add_rms_norm_fwd(int64_t N, int64_t D, const void *a, const void *b, const void *w,
+                                         float eps, void *sum, void *y, void *stream)
+{
+    CACTI_REQUIRE(N > 0 && D > 0 && a && b && w && sum && y, CACTI_E_INVALID,
+                  "add_rms_norm_fwd: null pointer or empty shape");
+    CACTI_REQUIRE(D % 8 == 0 && D <= 8192, CACTI_E_NOTIMPL,
+                  "add_rms_norm_fwd: need D %% 8 == 0 and D <= 8192 (D=%lld)", (long long)D);
+    CACTI_REQUIRE(aligned(a, 16) && aligned(b, 16) && aligned(w, 16) && aligned(sum, 16) && aligned(y, 16),
+                  CACTI_E_INVALID, "add_rms_norm_fwd: tensors must be 16-byte aligned");
+    CACTI_DISPATCH_CH(ch_for(D), launch_fwd<CH>(N, (int)D, (const half_t *)a, (const half_t *)b,
+                                                (const half_t *)w, eps, (half_t *)sum, (half_t *)y,
+                                                (hipStream_t)stream));
+    return launch_status("add_rms_norm_fwd");
 }
 
 CACTI_API size_t cacti_hip_rms_norm_bwd_workspace(int64_t N, int64_t D)

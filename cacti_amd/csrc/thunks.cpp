@@ -158,6 +158,46 @@ struct RmsNormSpec : ThunkSpec {
     }
 };
 
+// x = a + b followed by y = rms_norm(x, w) as one launch with both outputs (the residual add
+// always feeds a norm: llama.rs:512-516 and :532 -> the next layer's :474 / the head's :536).
+// The adjoint is the two thunks' rules in their reverse order: the norm's adjoint accumulates
+// into the adjoint of x, which the add's two memcpy adjoints then hand on.
+struct AddRmsNormSpec : ThunkSpec {
+    float eps;
+    explicit AddRmsNormSpec(float e) : eps(e) {}
+    const char *name() const override { return "add_rms_norm"; }
+    int arity() const override { return 3; }                       // (a, b, w) -> x, y
+    int nout() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[1] && a[0].dtype == F16 && a[2].dtype == F16 && a[0].shape.size() == 2 &&
+                       a[2].numel() == a[0].shape[1],
+                   "add_rms_norm: (a, b f16 [N,D], w f16 [D]) expected");
+        o = {a[0], a[0]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        TY_REQUIRE(acc == 0, "add_rms_norm: accumulate mode not staged on this path");
+        return cacti_hip_add_rms_norm_fwd(aty[0].shape[0], aty[0].shape[1], a[0], a[1], a[2], eps, o[0],
+                                          o[1], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        if (dy[1]) {
+            int rc = c.adj_add({e.outs[0], e.args[2]}, std::unique_ptr<ThunkSpec>(new RmsNormBwdSpec(eps)),
+                               {e.outs[0], e.args[2], dy[1]});
+            if (rc) return rc;
+        }
+        if (!c.adj_written(e.outs[0])) return 0;
+        const CellPtr dx = c.adj_of(e.outs[0]);
+        int rc = c.adj_add({e.args[0]}, make_copy(), {dx});
+        if (rc) return rc;
+        return c.adj_add({e.args[1]}, make_copy(), {dx});
+    }
+};
+
 // ---------------------------------------------------------------------------
 // MatrixMulThunkSpec src/thunk/op.rs:4284-4368 (2-d) and BlockMatrixMulThunkSpec :4719-4918
 // on [R, H*C] tensors (the reference's [B,S,H,C] with B = 1, flattened) whose H per-head
@@ -482,6 +522,10 @@ std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H)
     return std::unique_ptr<ThunkSpec>(new CausalSoftmaxSpec(H));
 }
 std::unique_ptr<ThunkSpec> make_add() { return std::unique_ptr<ThunkSpec>(new AddSpec()); }
+std::unique_ptr<ThunkSpec> make_add_rms_norm(float eps)
+{
+    return std::unique_ptr<ThunkSpec>(new AddRmsNormSpec(eps));
+}
 std::unique_ptr<ThunkSpec> make_copy() { return std::unique_ptr<ThunkSpec>(new CopySpec()); }
 std::unique_ptr<ThunkSpec> make_silu_gate()
 {

@@ -17,6 +17,7 @@ std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H);                    // (p16
 std::unique_ptr<ThunkSpec> make_rope(int64_t H);                      // (x [S,H*Dh], cos, sin) -> y
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H);            // (s16 [S,H*S]) -> p16
 std::unique_ptr<ThunkSpec> make_add();                                // (a, b) -> y
+std::unique_ptr<ThunkSpec> make_add_rms_norm(float eps);              // (a, b, w) -> a + b, norm
 std::unique_ptr<ThunkSpec> make_copy();                               // (x) -> y
 std::unique_ptr<ThunkSpec> make_silu_gate();                          // (g, u) -> h
 std::unique_ptr<ThunkSpec> make_softmax_ce(bool want_prob);           // (logit, tok) -> loss, amax[, prob]

@@ -51,6 +51,7 @@ SIGNATURES = {
     "cacti_hip_accumulate_1d_f16": (ci, [vp, vp, i64, vp]),
     "cacti_hip_accumulate_1d_u16": (ci, [vp, vp, i64, vp]),
     "cacti_hip_rms_norm_fwd": (ci, [i64, i64, vp, vp, f32, vp, vp]),
+    "cacti_hip_add_rms_norm_fwd": (ci, [i64, i64, vp, vp, vp, f32, vp, vp, vp]),
     "cacti_hip_rms_norm_bwd_workspace": (sz, [i64, i64]),
     "cacti_hip_rms_norm_bwd": (ci, [i64, i64, vp, vp, f32, vp, vp, ci, vp, ci, vp, sz, vp]),
     "cacti_hip_rope_tables": (ci, [i64, i64, vp, vp, vp]),

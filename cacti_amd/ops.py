@@ -85,6 +85,16 @@ def rms_norm_fwd(x, w, eps):
     return y
 
 
+def add_rms_norm_fwd(a, b, w, eps):
+    """(f16(a + b), rms_norm of it): the residual add and the norm that follows, one launch."""
+    _chk(a), _chk(b), _chk(w)
+    N, D = a.shape
+    s, y = torch.empty_like(a), torch.empty_like(a)
+    ffi.call("cacti_hip_add_rms_norm_fwd", N, D, a.data_ptr(), b.data_ptr(), w.data_ptr(), eps,
+             s.data_ptr(), y.data_ptr(), _stream())
+    return s, y
+
+
 def rms_norm_bwd(x, w, eps, dy, dx_acc=None, dw_acc=None):
     """Returns (dx, dw).  dx_acc / dw_acc: tensors to accumulate into (updated in place)."""
     _chk(x), _chk(w), _chk(dy)

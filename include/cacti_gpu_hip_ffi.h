@@ -145,6 +145,13 @@ int cacti_hip_accumulate_1d_u16(void *dst, const void *src, int64_t n, void *str
  * x, y: [N,D] f16; w: [D] f16.  D % 8 == 0, D <= 16384. */
 int cacti_hip_rms_norm_fwd(int64_t N, int64_t D, const void *x, const void *w, float eps,
                            void *y, void *stream);
+/* The residual add in front of a norm and the norm in one pass over the rows:
+ * sum = f16(a + b) (AddFutThunkSpec, src/thunk/op.rs:1480-1535; x1 = stream + o and
+ * x2 = x1 + down in src/librarium/llama.rs:512-532), y = rms_norm(sum, w) as above.  Both
+ * outputs are written; the results equal those of cacti_hip_add_f16 followed by
+ * cacti_hip_rms_norm_fwd bit for bit. */
+int cacti_hip_add_rms_norm_fwd(int64_t N, int64_t D, const void *a, const void *b, const void *w,
+                               float eps, void *sum, void *y, void *stream);
 
 /* Adjoint of the chain above (src/spine.rs:447-690 over the same thunks).
  * dx [N,D] f16 receives the two f16 contributions of the reference in order

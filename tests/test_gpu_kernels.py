@@ -64,6 +64,19 @@ def test_rms_norm_fwd(ops, oracle, N, D):
     assert exact_frac(got, want) > 0.999
 
 
+@pytest.mark.parametrize("N,D", [(2048, 3200), (37, 4096), (5, 8)])
+def test_add_rms_norm_fwd_equals_the_two_thunks(ops, oracle, N, D):
+    """One launch for x = a + b and rms_norm(x): bit for bit the add thunk followed by the norm."""
+    say("add_rms_norm_fwd", N, D)
+    r = rng(120 + N)
+    a, b, w = randn16(r, (N, D)), randn16(r, (N, D)), (randn16(r, (D,), 0.1) + np.float16(1))
+    s, y = ops.add_rms_norm_fwd(dev(a), dev(b), dev(w), 1e-6)
+    want_s = oracle.accumulate_f16(a, b)
+    assert_bits(host(s), want_s, "sum")
+    assert_bits(host(y), host(ops.rms_norm_fwd(dev(want_s), dev(w), 1e-6)), "norm vs unfused kernel")
+    assert_parity(host(y), oracle.rmsnorm_fwd(want_s, w, 1e-6)[0], "norm vs oracle")
+
+
 @pytest.mark.parametrize("N,D", [(2048, 3200), (128, 256), (37, 4096), (5, 8), (16, 8192)])
 @pytest.mark.parametrize("acc", [False, True])
 def test_rms_norm_bwd(ops, oracle, N, D, acc):
