@@ -64,17 +64,17 @@ def synth_inputs(cfg, seed=1, grad_scale=1024.0):
     return tok, lm_tok, scale
 
 
-# L2-miss traffic per launch of the 128 x 128 GEMM kernel, rocprofv3 --pmc FETCH_SIZE and
+# L2-miss traffic per launch of the GEMM kernels at the step's shapes, rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE in KiB per dispatch (profiles/llama3b_step_gemm_hbm_traffic.txt gives the commands);
 # a streaming kernel of known size reads FETCH_SIZE = half its bytes and WRITE_SIZE = its
 # bytes, so bytes = (2.0 * FETCH_SIZE + 1.0 * WRITE_SIZE) * 1024
 GEMM_TRAFFIC_KIB = {
-    ("NT", 2048, 3200, 3200): (53437, 12800), ("NT", 2048, 3200, 8640): (225558, 12800),
-    ("NT", 2048, 8640, 3200): (156643, 34560),
-    ("NN", 2048, 3200, 3200): (61962, 12800), ("NN", 2048, 3200, 8640): (243619, 12800),
-    ("NN", 2048, 8640, 3200): (164838, 34560), ("NN", 2048, 3200, 32000): (1137423, 12800),
-    ("TN", 3200, 3200, 2048): (67231, 20000), ("TN", 8640, 3200, 2048): (164032, 54000),
-    ("TN", 3200, 8640, 2048): (164032, 54000), ("TN", 32000, 3200, 2048): (722906, 200000),
+    ("NT", 2048, 3200, 3200): (64068, 12800), ("NT", 2048, 3200, 8640): (172868, 12800),
+    ("NT", 2048, 8640, 3200): (159799, 34560), ("NT", 2048, 32000, 3200): (640965, 128000),
+    ("NN", 2048, 3200, 3200): (67274, 12800), ("NN", 2048, 3200, 8640): (176074, 12800),
+    ("NN", 2048, 8640, 3200): (159691, 34560), ("NN", 2048, 3200, 32000): (640147, 12800),
+    ("TN", 3200, 3200, 2048): (67640, 20000), ("TN", 8640, 3200, 2048): (165781, 54000),
+    ("TN", 3200, 8640, 2048): (165781, 54000), ("TN", 32000, 3200, 2048): (739452, 200000),
 }
 
 
