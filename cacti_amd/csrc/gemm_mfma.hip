@@ -3,9 +3,11 @@
 //
 //   C[M,N] = alpha op(A) op(B) + beta C,   f16 in, fp32 MFMA accumulate, f16 out.
 //
-// Block tile BM x BN x 64, WM x WN wavefronts, each owning a 64 x 64 patch of 32 x 32
-// accumulators fed by v_mfma_f32_32x32x16_f16.  Two shapes are instantiated: 128 x 128 on 4
-// waves (two workgroups per CU) and 256 x 128 on 8 waves (one per CU).
+// Block tile BM x BN x 64, WM x WN wavefronts, each owning BM / WM x BN / WN outputs as
+// 32 x 32 accumulators fed by v_mfma_f32_32x32x16_f16 (the 32 x 32 tiles of a wave are
+// interleaved with those of the other waves, 32 WM rows / 32 WN columns apart).  Shapes
+// instantiated: 128 x 128 on 4 waves (two workgroups per CU), 256 x 128 and 256 x 256 on 8
+// waves (one per CU), 64 x 64 on 4 waves (remainder columns).
 //
 // LDS layout (both operands): [row][64 k] = 128 bytes per row, no padding; the 16-byte
 // k-chunk q of row r sits at chunk position q ^ f(r), f(r) = (r ^ (r >> 3)) & 7.
@@ -142,6 +144,53 @@ struct LoadKC {
         }
     }
     static constexpr int NREG = NL;
+    static constexpr int NVMEM = NL * (AL == 8 ? 1 : 2);          // load instructions per tile
+    static constexpr int NDMA = 0;
+    __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
+};
+
+// ---- k-contiguous operand fetched straight into LDS (global_load_lds_dwordx4: the 16 bytes
+// of lane l land at LDS address M0 + 16 l, no register staging and no LDS store instruction).
+// A wave fills 1 KB = 8 consecutive tile rows per instruction; the chunk swizzle of the LDS
+// layout is applied on the global side: the lane at chunk position p of row r fetches k chunk
+// p ^ f(r), which stays inside the row's 128-byte segment.  The loads are issued from inline
+// assembly, so the compiler neither counts them nor knows that they write LDS: the kernel
+// waits for them itself (vmcnt) before the barrier that publishes the tile.
+template <int ROWS, int NT>
+struct LoadKCD {
+    static_assert(ROWS * 8 % NT == 0, "whole instructions per wave");
+    static constexpr int NL = ROWS * 8 / NT;
+    uint32_t off[NL];              // byte offset of the lane's chunk from (row0, k = 0)
+
+    __device__ __forceinline__ void init(int64_t ld, int64_t rows_left, int64_t)
+    {
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            const int c = threadIdx.x + it * NT;
+            const int r = c >> 3, q = (c & 7) ^ swz(r);
+            const int64_t row = r < rows_left ? r : rows_left - 1;
+            off[it] = (uint32_t)((row * ld + q * 8) * 2);
+        }
+    }
+    // lds = byte address in LDS of the tile buffer to fill; origin = &op[row0][0]
+    __device__ __forceinline__ void dma(uint32_t lds, const half_t *origin, int64_t k0) const
+    {
+        const half_t *base = origin + k0;
+        const uint32_t wave = lds + (threadIdx.x & ~63u) * 16;
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            const uint32_t m0 = __builtin_amdgcn_readfirstlane(wave + it * NT * 16);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :
+                         : "s"(m0), "v"(off[it]), "s"(base)
+                         : "memory");
+        }
+    }
+    __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
+    __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
+    static constexpr int NREG = 1;
+    static constexpr int NVMEM = 0;
+    static constexpr int NDMA = NL;
 };
 
 // ---- k-strided operand (memory [k][row]): item c -> row chunk c % (ROWS/8), k group
@@ -233,6 +282,9 @@ struct LoadKS {
         }
     }
     static constexpr int NREG = NL * 8;
+    static constexpr int NVMEM = 0;                               // depends on the wave: not counted
+    static constexpr int NDMA = 0;
+    __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
 
 // ---- both operands k-strided (A^T and B), square block tile with exactly one 8 k x 8 rows
@@ -306,6 +358,9 @@ struct LoadKS2 {
         }
     }
     static constexpr int NREG = 8;
+    static constexpr int NVMEM = 8 * (AL == 8 ? 1 : 2);
+    static constexpr int NDMA = 0;
+    __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
 
 // ---- one k-strided operand, every lane of the block taking part: an item is KPI k x 8 rows
@@ -374,6 +429,9 @@ struct LoadKSH {
         }
     }
     static constexpr int NREG = KPI;
+    static constexpr int NVMEM = KPI * (AL == 8 ? 1 : 2);
+    static constexpr int NDMA = 0;
+    __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
 
 // stands in for the B loader when LoadKS2 serves both operands
@@ -381,7 +439,10 @@ struct LoadNone {
     __device__ __forceinline__ void init(int64_t, int64_t, int64_t) {}
     __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
     __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
+    __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
     static constexpr int NREG = 1;
+    static constexpr int NVMEM = 0;
+    static constexpr int NDMA = 0;
 };
 
 template <bool STRIDED, int ROWS, int NT, int T0, int AL, bool KTAIL> struct Loader;
@@ -407,17 +468,38 @@ struct SchedStep<NM, NR, NR> {
 
 // waves per SIMD the register allocation must leave room for: two 128 x 128 blocks (or one
 // 8-wave block) per CU, one 4-wave 256 x 256 block
-constexpr int min_waves(int, int, int) { return 2; }              // both tile shapes: 8 waves per CU
+constexpr int min_waves(int bm, int bn, int waves, int nbuf)
+{
+    const int blocks = 160 * 1024 / (nbuf * (bm + bn) * BK * 2);  // workgroups per CU by LDS
+    const int w = blocks * waves / 4;
+    return w >= 2 ? 2 : 1;
+}
 
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
-__global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN))
+// wait until at most n vector memory loads are outstanding (s_waitcnt vmcnt only)
+template <int N>
+__device__ __forceinline__ void wait_vmem()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// NBUF = 3: the k-contiguous operands are fetched straight into LDS two tiles ahead (three
+// LDS buffers); strided operands keep their register stages.  NBUF = 2: everything through
+// registers.
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES, int NBUF>
+__global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN, NBUF))
 gemm_mfma_kernel(GemmArgs p)
 {
+    static_assert(NBUF == 2 || (NBUF == 3 && STAGES == 2 && AL == 8 && !KTAIL && (!TA || TB)),
+                  "direct loads: 16-byte aligned whole k tiles, at least one k-contiguous operand");
+    constexpr bool DMA_A = NBUF == 3 && !TA, DMA_B = NBUF == 3 && TB;
+    static_assert((WM % 2 == 0 || BM / WM == 32) && (WN % 2 == 0 || BN / WN == 32),
+                  "tiles of a wave lie 32 WM rows apart: a multiple of 64 keeps their swizzle equal");
     constexpr int NT = WM * WN * 64;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;          // 32x32 tiles per wave
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    half_t *As = reinterpret_cast<half_t *>(smem_raw);            // [2][BM*BK]
-    half_t *Bs = As + 2 * BM * BK;                                // [2][BN*BK]
+    half_t *As = reinterpret_cast<half_t *>(smem_raw);            // [NBUF][BM*BK]
+    half_t *Bs = As + NBUF * BM * BK;                             // [NBUF][BN*BK]
 
     // XCD-aware numbering over the flattened (block of the batch, tile) sequence: dispatch
     // order i lands on XCD i % 8; give each XCD a contiguous band.  With a batch that is a
@@ -476,11 +558,13 @@ gemm_mfma_kernel(GemmArgs p)
     typedef typename std::conditional<
         UNI, LoadKS2<BM, NT, AL, KTAIL>,
         typename std::conditional<HALF_A, LoadKSH<BM, NT, AL, KTAIL>,
-                                  Loader<TA, BM, NT, 0, AL, KTAIL>>::type>::type LA;
+                                  Loader<TA, BM, NT, 0, AL, KTAIL>>::type>::type LA_REG;
     typedef typename std::conditional<
         UNI, LoadNone,
         typename std::conditional<HALF_B, LoadKSH<BN, NT, AL, KTAIL>,
-                                  Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL, KTAIL>>::type>::type LB;
+                                  Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL, KTAIL>>::type>::type LB_REG;
+    typedef typename std::conditional<DMA_A, LoadKCD<BM, NT>, LA_REG>::type LA;
+    typedef typename std::conditional<DMA_B, LoadKCD<BN, NT>, LB_REG>::type LB;
     LA la;
     LB lb;
     if constexpr (UNI) {
@@ -499,9 +583,12 @@ gemm_mfma_kernel(GemmArgs p)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // per-lane row offsets and swizzles of the operand fragments
-    const int ar0 = wm * (BM / WM) + l32, br0 = wn * (BN / WN) + l32;
-    const int asw = swz(ar0), bsw = swz(br0);                     // row + 32 i flips bit 2
+    // per-lane row offsets and swizzles of the operand fragments.  The 32 x 32 tiles of a wave
+    // lie 32 WM rows (32 WN columns) apart, a multiple of 64 rows, so every tile of a lane has
+    // the same swizzle and differs from the first only by a constant LDS offset.
+    const int ar0 = wm * 32 + l32, br0 = wn * 32 + l32;
+    const int asw = swz(ar0), bsw = swz(br0);
+    constexpr int ASTEP = (TM > 1 ? 32 * WM : 0) * BK, BSTEP = (TN > 1 ? 32 * WN : 0) * BK;
 
     // MFMAs of k step ks run while the operand fragments of step ks + 1 are in flight from
     // LDS (two fragment sets): the wait before a step's MFMAs leaves the next step's reads
@@ -517,12 +604,10 @@ gemm_mfma_kernel(GemmArgs p)
             const int q = ks * 2 + lh;
 #pragma unroll
             for (int i = 0; i < TM; i++)
-                af[set][i] = *reinterpret_cast<const half8_t *>(
-                    as + i * 32 * BK + ((q ^ asw ^ ((i & 1) << 2)) << 3));
+                af[set][i] = *reinterpret_cast<const half8_t *>(as + i * ASTEP + ((q ^ asw) << 3));
 #pragma unroll
             for (int j = 0; j < TN; j++)
-                bf[set][j] = *reinterpret_cast<const half8_t *>(
-                    bs + j * 32 * BK + ((q ^ bsw ^ ((j & 1) << 2)) << 3));
+                bf[set][j] = *reinterpret_cast<const half8_t *>(bs + j * BSTEP + ((q ^ bsw) << 3));
         };
         if (PIPE) frags(0, 0);
 #pragma unroll
@@ -554,28 +639,54 @@ gemm_mfma_kernel(GemmArgs p)
         }
     };
 
-    // Software pipeline over k tiles with STAGES register sets and two LDS buffers.  Invariant
-    // at the start of tile t: LDS[t & 1] holds tile t, register set (t + j - kt0) % STAGES
-    // holds tile t + j for j = 1 .. STAGES - 1, and set (t - kt0) % STAGES is free.  A step
-    // loads tile t + STAGES into the free set, runs the MFMAs of tile t, moves tile t + 1 from
-    // its set to the other LDS buffer and ends in the one barrier of the k tile.  The main
-    // loop has no branch (all its loads are inside K); the last 2 STAGES - 1 tiles are
-    // peeled into steps that test what still exists.
-    auto step = [&](auto set_c, auto main_c, int t) __attribute__((always_inline)) {
+    // Software pipeline over k tiles with STAGES register sets and NBUF LDS buffers.  Invariant
+    // at the start of tile t (cb = its LDS buffer): LDS[cb] holds tile t behind a barrier,
+    // register set (t + j - kt0) % STAGES holds tile t + j of the operands staged in registers
+    // for j = 1 .. STAGES - 1, set (t - kt0) % STAGES is free, and the direct loads of tile
+    // t + 1 are in flight to the next buffer.  A step issues the direct loads of tile t + 2 into
+    // the buffer tile t - 1 has left, loads tile t + STAGES into the free register set, runs the
+    // MFMAs of tile t, moves tile t + 1 from its set to the next LDS buffer, waits for the
+    // direct loads of tile t + 1 (everything but what this step issued) and ends in the one
+    // barrier of the k tile.  The main loop has no branch (all its loads are inside K); the
+    // last 2 STAGES - 1 tiles are peeled into steps that test what still exists.
+    auto next_buf = [](int b) __attribute__((always_inline)) { return b + 1 == NBUF ? 0 : b + 1; };
+    auto lds_addr = [](const half_t *q) __attribute__((always_inline)) {
+        return (uint32_t)(uintptr_t)q;                            // LDS byte address of a shared pointer
+    };
+    auto step = [&](auto set_c, auto main_c, int t, int cbv) __attribute__((always_inline)) {
         constexpr int U = decltype(set_c)::value, UN = (U + 1) % STAGES;
         constexpr bool MAIN = decltype(main_c)::value;
+        const int cb = NBUF == 2 ? (t & 1) : cbv, nb1 = next_buf(cb);
+        if (NBUF == 3 && (MAIN || t + 2 < nk)) {
+            const int nb2 = next_buf(nb1);
+            la.dma(lds_addr(As + nb2 * BM * BK), Ao, (int64_t)(t + 2) * BK);
+            lb.dma(lds_addr(Bs + nb2 * BN * BK), Bo, (int64_t)(t + 2) * BK);
+        }
         if (MAIN || t + STAGES < nk) {
             la.load(ra[U], Ao, (int64_t)(t + STAGES) * BK);
             lb.load(rb[U], Bo, (int64_t)(t + STAGES) * BK);
         }
-        compute(t & 1);
+        compute(cb);
         if (MAIN || t + 1 < nk) {
-            la.store(ra[UN], As + ((t + 1) & 1) * BM * BK);
-            lb.store(rb[UN], Bs + ((t + 1) & 1) * BN * BK);
+            la.store(ra[UN], As + nb1 * BM * BK);
+            lb.store(rb[UN], Bs + nb1 * BN * BK);
+        }
+        if (NBUF == 3) {
+            // everything older than this step's own loads has landed: tile t + 1 is in LDS
+            if (MAIN) wait_vmem<LA::NDMA + LB::NDMA + LA::NVMEM + LB::NVMEM>();
+            else wait_vmem<0>();
         }
         __syncthreads();
     };
     {
+        if (NBUF == 3) {
+            la.dma(lds_addr(As), Ao, (int64_t)kt0 * BK);
+            lb.dma(lds_addr(Bs), Bo, (int64_t)kt0 * BK);
+            if (kt0 + 1 < nk) {
+                la.dma(lds_addr(As + BM * BK), Ao, (int64_t)(kt0 + 1) * BK);
+                lb.dma(lds_addr(Bs + BN * BK), Bo, (int64_t)(kt0 + 1) * BK);
+            }
+        }
         la.load(ra[0], Ao, (int64_t)kt0 * BK);
         lb.load(rb[0], Bo, (int64_t)kt0 * BK);
 #pragma unroll
@@ -584,21 +695,30 @@ gemm_mfma_kernel(GemmArgs p)
                 la.load(ra[u], Ao, (int64_t)(kt0 + u) * BK);
                 lb.load(rb[u], Bo, (int64_t)(kt0 + u) * BK);
             }
-        la.store(ra[0], As + (kt0 & 1) * BM * BK);
-        lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
+        const int b0 = NBUF == 2 ? (kt0 & 1) : 0;
+        la.store(ra[0], As + b0 * BM * BK);
+        lb.store(rb[0], Bs + b0 * BN * BK);
+        if (NBUF == 3) wait_vmem<0>();
         __syncthreads();
-        int kt = kt0;
+        int kt = kt0, cb = 0;
         for (; kt + 2 * STAGES - 1 < nk; kt += STAGES) {
-            step(std::integral_constant<int, 0>{}, std::true_type{}, kt);
-            if (STAGES > 1) step(std::integral_constant<int, 1 % STAGES>{}, std::true_type{}, kt + 1);
-            if (STAGES > 2) step(std::integral_constant<int, 2 % STAGES>{}, std::true_type{}, kt + 2);
+            step(std::integral_constant<int, 0>{}, std::true_type{}, kt, cb);
+            cb = next_buf(cb);
+            if (STAGES > 1) {
+                step(std::integral_constant<int, 1 % STAGES>{}, std::true_type{}, kt + 1, cb);
+                cb = next_buf(cb);
+            }
+            if (STAGES > 2) {
+                step(std::integral_constant<int, 2 % STAGES>{}, std::true_type{}, kt + 2, cb);
+                cb = next_buf(cb);
+            }
         }
         static_assert(STAGES >= 1 && STAGES <= 3, "peeled tail below covers up to 5 tiles");
-        if (kt + 0 < nk) step(std::integral_constant<int, 0 % STAGES>{}, std::false_type{}, kt + 0);
-        if (STAGES > 1 && kt + 1 < nk) step(std::integral_constant<int, 1 % STAGES>{}, std::false_type{}, kt + 1);
-        if (STAGES > 1 && kt + 2 < nk) step(std::integral_constant<int, 2 % STAGES>{}, std::false_type{}, kt + 2);
-        if (STAGES > 2 && kt + 3 < nk) step(std::integral_constant<int, 3 % STAGES>{}, std::false_type{}, kt + 3);
-        if (STAGES > 2 && kt + 4 < nk) step(std::integral_constant<int, 4 % STAGES>{}, std::false_type{}, kt + 4);
+        if (kt + 0 < nk) { step(std::integral_constant<int, 0 % STAGES>{}, std::false_type{}, kt + 0, cb); cb = next_buf(cb); }
+        if (STAGES > 1 && kt + 1 < nk) { step(std::integral_constant<int, 1 % STAGES>{}, std::false_type{}, kt + 1, cb); cb = next_buf(cb); }
+        if (STAGES > 1 && kt + 2 < nk) { step(std::integral_constant<int, 2 % STAGES>{}, std::false_type{}, kt + 2, cb); cb = next_buf(cb); }
+        if (STAGES > 2 && kt + 3 < nk) { step(std::integral_constant<int, 3 % STAGES>{}, std::false_type{}, kt + 3, cb); cb = next_buf(cb); }
+        if (STAGES > 2 && kt + 4 < nk) { step(std::integral_constant<int, 4 % STAGES>{}, std::false_type{}, kt + 4, cb); cb = next_buf(cb); }
     }
 
     // Epilogue through LDS (the operand buffers are free after the last barrier): a lane
@@ -609,25 +729,27 @@ gemm_mfma_kernel(GemmArgs p)
     // alpha acc + beta C is still rounded to f16 exactly once.
     half_t *Cs = reinterpret_cast<half_t *>(smem_raw);
     constexpr int CPRC = BN / 8;                                  // 16-byte chunks per row
+    constexpr int CSW = CPRC - 1;                                 // chunk swizzle mask
+    static_assert((CPRC & CSW) == 0, "the chunk swizzle must stay inside the row");
     const bool has_beta = p.beta != 0.f;
     if (has_beta) {
         for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
             const int row = c / CPRC, cc = c % CPRC;
             const int64_t m = m0 + row, n = n0 + cc * 8;
             const uint4 v = load8_guarded<AL>(C + m * p.ldc + n, m < p.M ? p.N - n : 0);
-            *reinterpret_cast<uint4 *>(Cs + row * BN + ((cc ^ (row & (CPRC - 1))) << 3)) = v;
+            *reinterpret_cast<uint4 *>(Cs + row * BN + ((cc ^ (row & CSW)) << 3)) = v;
         }
         __syncthreads();
     }
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-        const int row = wm * (BM / WM) + i * 32 + l32;
+        const int row = i * (32 * WM) + wm * 32 + l32;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const int col = wn * (BN / WN) + j * 32 + q * 8 + lh * 4;
-                half_t *sp = Cs + row * BN + ((((col >> 3) ^ (row & (CPRC - 1))) << 3) | (col & 4));
+                const int col = j * (32 * WN) + wn * 32 + q * 8 + lh * 4;
+                half_t *sp = Cs + row * BN + ((((col >> 3) ^ (row & CSW)) << 3) | (col & 4));
                 half4_t o;
                 if (has_beta) {
                     const half4_t old = *reinterpret_cast<const half4_t *>(sp);
@@ -647,7 +769,7 @@ gemm_mfma_kernel(GemmArgs p)
         const int row = c / CPRC, cc = c % CPRC;
         const int64_t m = m0 + row, n = n0 + cc * 8;
         if (m >= p.M || n >= p.N) continue;
-        const uint4 v = *reinterpret_cast<const uint4 *>(Cs + row * BN + ((cc ^ (row & (CPRC - 1))) << 3));
+        const uint4 v = *reinterpret_cast<const uint4 *>(Cs + row * BN + ((cc ^ (row & CSW)) << 3));
         half_t *cp = C + m * p.ldc + n;
         if (AL == 8) {
             *reinterpret_cast<uint4 *>(cp) = v;
@@ -660,13 +782,13 @@ gemm_mfma_kernel(GemmArgs p)
     }
 }
 
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES>
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES, int NBUF = 2>
 int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 {
     p.tiles_m = (int)((p.M + BM - 1) / BM);
     p.tiles_n = (int)((p.N + BN - 1) / BN);
-    const size_t smem = (size_t)2 * (BM + BN) * BK * sizeof(half_t);
-    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES>;
+    const size_t smem = (size_t)NBUF * (BM + BN) * BK * sizeof(half_t);
+    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES, NBUF>;
     static bool attr_set = false;                 // one flag per instantiation
     if (!attr_set) {
         CACTI_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -682,31 +804,70 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
     return launch_status("gemm_mfma");
 }
 
-// register stages per layout: a strided operand stages 8 x 16 bytes per lane, so two
-// stages only pay where the accumulators leave room
+// tile: 0 = 128 x 128 on 4 waves, two register stages (every loader is branch-free on 256
+// lanes); 1 = 256 x 128 on 8 waves; 2 = 256 x 256 on 8 waves (128 x 64 per wave; one register
+// stage, what the 128 accumulator registers leave room for); 3 = 64 x 64 on 4 waves;
+// 4 = 256 x 128 on 8 waves with the k-contiguous operands loaded straight into LDS
 template <bool TA, bool TB>
 int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
 {
-    // 128 x 128 on 256 lanes: every loader is branch-free and small enough for two register
-    // stages
-    constexpr int S0 = 2;
     const bool ktail = (p.K % BK) != 0;
     if (align < 8) {                              // 8-byte aligned operands (the attention blocks)
         return ktail ? launch_cfg<TA, TB, 128, 128, 2, 2, 4, true, 1>(p, nblk, st)
-                     : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, S0>(p, nblk, st);
+                     : launch_cfg<TA, TB, 128, 128, 2, 2, 4, false, 2>(p, nblk, st);
     }
     if (ktail) return launch_cfg<TA, TB, 128, 128, 2, 2, 8, true, 1>(p, nblk, st);
     switch (tile) {
-        case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8, false, S0>(p, nblk, st);
+        case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8, false, 2>(p, nblk, st);
+        case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1>(p, nblk, st);
+        case 3: return launch_cfg<TA, TB, 64, 64, 2, 2, 8, false, 2>(p, nblk, st);
+        case 4:
+            if constexpr (!TA || TB) return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2, 3>(p, nblk, st);
+            else return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
         default: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
     }
+}
+
+template <bool TA, bool TB>
+int launch_auto(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
+{
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        CACTI_HIP(hipGetDevice(&dev));
+        CACTI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    }
+    static const bool no_split = getenv("CACTI_GEMM_NO_SPLIT") != nullptr;
+    // One 256 x 128 workgroup per CU runs in rounds of `cus` tiles.  When the last round would
+    // hold only a few tiles (N = 8640 at 2048 tokens: 2 full rounds + 32 tiles, a third of
+    // the launch time for 6 % of the work), the columns of the full rounds go to one launch
+    // and the remaining ones to a second launch of 64 x 64 tiles, which spreads them over
+    // every CU: -12..19 % at that shape.  (The dgrad layout would gain 8 %; it is left whole so
+    // that each of its launches stays one kernel.)
+    if ((tile == 1 || tile == 4) && !TA && TB && nblk == 1 && align >= 8 && p.K % BK == 0 && p.tri == 0 &&
+        !no_split) {
+        const int64_t tiles_m = (p.M + 255) / 256, tiles_n = (p.N + 127) / 128;
+        const int64_t rounds = tiles_m * tiles_n / cus;
+        const int64_t cols_main = rounds * cus / tiles_m;
+        const int64_t rest = tiles_m * (tiles_n - cols_main);
+        if (rounds >= 1 && cols_main < tiles_n && rest * 4 <= cus) {
+            GemmArgs a = p, b = p;
+            a.N = cols_main * 128;
+            b.N = p.N - a.N;
+            b.B = p.B + (TB ? a.N * p.ldb : a.N);
+            b.C = p.C + a.N;
+            const int rc = launch_tile<TA, TB>(tile, align, a, nblk, st);
+            return rc ? rc : launch_tile<TA, TB>(3, align, b, nblk, st);
+        }
+    }
+    return launch_tile<TA, TB>(tile, align, p, nblk, st);
 }
 
 }  // namespace
 
 namespace cacti {
 
-// tile: 0 = 128x128 (4 waves), 1 = 256x128 (8 waves); -1 = pick by shape
+// tile: as launch_tile; -1 = pick by shape
 int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align, int tile,
                      hipStream_t st)
 {
@@ -734,17 +895,25 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             // measured on MI355X at the step's shapes.  A not transposed (forward and dgrad
             // products, M = tokens): one 8-wave 256 x 128 workgroup per CU fetches each B panel
             // half as often as two 128 x 128 ones (+8..14 % on the projection and FFN shapes, and
-            // the best choice for the LM head too).  The wgrad layout loses 5..17 % to its
-            // coarser tile count and stays on 128 x 128, as do small and batched products.
+            // the best choice for the LM head too); with both operands k-contiguous (forward)
+            // they go straight into LDS (+8..12 % on the FFN and LM-head shapes, +2 % on the
+            // projections; with only A direct the dgrad layout loses 10 %, so it keeps its
+            // register stages).  The wgrad layout loses 5..17 % to 256 x 128's coarser tile
+            // count but gains 3..15 % from 256 x 256 with 128 x 64 per wave on the weight-sized
+            // outputs; small and batched products stay on 128 x 128.
             tile = 0;
-            static const bool wide = !getenv("CACTI_GEMM_NO_NT256");
-            if (wide && !ta && tile == 0 && nblk == 1 && p.M >= 1024 && p.N >= 1024) tile = 1;
+            if (nblk == 1 && p.M >= 1024 && p.N >= 1024) {
+                static const bool no_direct = getenv("CACTI_GEMM_NO_DIRECT") != nullptr;
+                static const bool no_wide_tn = getenv("CACTI_GEMM_NO_WIDE_TN") != nullptr;
+                if (!ta) tile = tb && !no_direct ? 4 : 1;
+                else if (!tb && p.M >= 2048 && p.N >= 2048 && !no_wide_tn) tile = 2;
+            }
         }
     }
-    if (!ta && !tb) return launch_tile<false, false>(tile, align, q, nblk, st);
-    if (!ta && tb) return launch_tile<false, true>(tile, align, q, nblk, st);
-    if (ta && !tb) return launch_tile<true, false>(tile, align, q, nblk, st);
-    return launch_tile<true, true>(tile, align, q, nblk, st);
+    if (!ta && !tb) return launch_auto<false, false>(tile, align, q, nblk, st);
+    if (!ta && tb) return launch_auto<false, true>(tile, align, q, nblk, st);
+    if (ta && !tb) return launch_auto<true, false>(tile, align, q, nblk, st);
+    return launch_auto<true, true>(tile, align, q, nblk, st);
 }
 
 }  // namespace cacti

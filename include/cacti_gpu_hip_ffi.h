@@ -147,7 +147,7 @@ int cacti_hip_rms_norm_fwd(int64_t N, int64_t D, const void *x, const void *w, f
                            void *y, void *stream);
 /* The residual add in front of a norm and the norm in one pass over the rows:
  * sum = f16(a + b) (AddFutThunkSpec, src/thunk/op.rs:1480-1535; x1 = stream + o and
- * x2 = x1 + down in src/librarium/llama.rs:512-532), y = rms_norm(sum, w) as above.  Both
+ * x2 = x1 + down in src/librarium/llama.rs:514-533), y = rms_norm(sum, w) as above.  Both
  * outputs are written; the results equal those of cacti_hip_add_f16 followed by
  * cacti_hip_rms_norm_fwd bit for bit. */
 int cacti_hip_add_rms_norm_fwd(int64_t N, int64_t D, const void *a, const void *b, const void *w,
