@@ -109,16 +109,18 @@ def gemm_dims(label):
 def kernel_symbol(label):
     """Name of the HIP kernel instantiation a dense GEMM label runs on, as rocprofv3 prints it.
     The tile choice mirrors gemm_mfma_launch for 16-byte aligned operands and K % 64 == 0: with an
-    output of at least 1024 x 1024 and one block, NT runs 256 x 128 / 8 waves with direct-to-LDS
-    loads (3 LDS buffers), NN 256 x 128 / 8 waves through registers, TN 256 x 256 / 8 waves from
-    2048 x 2048 outputs on; everything else 128 x 128 / 4 waves."""
+    output of at least 1024 x 1024 and one block, A not transposed runs 256 x 128 / 8 waves (from
+    768 tiles of 256 x 256 on: that tile) and A transposed 256 x 256 / 8 waves from 2048 x 2048
+    outputs on, all with direct-to-LDS loads; everything else 128 x 128 / 4 waves through
+    registers."""
     ta, tb, H, M, N, K = gemm_dims(label)
-    tile = "128, 128, 2, 2, 8, false, 2, 2"
+    tile = "128, 128, 2, 2, 8, false, 2, 2, false"
     if H == 1 and M >= 1024 and N >= 1024:
+        tiles256 = ((M + 255) // 256) * ((N + 255) // 256)
         if not ta:
-            tile = "256, 128, 4, 2, 8, false, 2, 3" if tb else "256, 128, 4, 2, 8, false, 2, 2"
-        elif not tb and M >= 2048 and N >= 2048:
-            tile = "256, 256, 2, 4, 8, false, 1, 2"
+            tile = "256, 256, 2, 4, 8, false, 1, 2, true" if tiles256 >= 768 else "256, 128, 4, 2, 8, false, 1, 3, true"
+        elif M >= 2048 and N >= 2048:
+            tile = "256, 256, 2, 4, 8, false, 1, 2, true"
     return "gemm_mfma_kernel<%s, %s, %s>" % (str(ta).lower(), str(tb).lower(), tile)
 
 
@@ -128,6 +130,8 @@ def is_split(label):
     pair then brackets both, so it is left out of a single kernel's roofline sample."""
     ta, tb, H, M, N, K = gemm_dims(label)
     if ta or not tb or H != 1 or M < 1024 or N < 1024 or K % 64:
+        return False
+    if ((M + 255) // 256) * ((N + 255) // 256) >= 768:
         return False
     tiles_m, tiles_n = (M + 255) // 256, (N + 127) // 128
     rounds = tiles_m * tiles_n // N_CUS

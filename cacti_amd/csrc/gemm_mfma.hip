@@ -9,6 +9,14 @@
 // instantiated: 128 x 128 on 4 waves (two workgroups per CU), 256 x 128 and 256 x 256 on 8
 // waves (one per CU), 64 x 64 on 4 waves (remainder columns).
 //
+// Two ways from global memory to LDS.  Through registers (any alignment >= 8 bytes, k tails):
+// described below.  Direct (16-byte aligned operands, K a multiple of 64; the large dense
+// products): global_load_lds_dwordx4 writes each wave's 1 KB straight into LDS, NBUF - 1 k
+// tiles ahead, with no staging registers, no LDS store instructions and no transposes in
+// registers; a k-contiguous operand lands in the swizzled [row][k] layout below (the swizzle
+// is applied to the global address), a k-strided one in its own [k][row] layout and is
+// transposed on the way out of LDS by ds_read_b64_tr_b16.
+//
 // LDS layout (both operands): [row][64 k] = 128 bytes per row, no padding; the 16-byte
 // k-chunk q of row r sits at chunk position q ^ f(r), f(r) = (r ^ (r >> 3)) & 7.
 // With this swizzle (a) the 16-byte MFMA operand reads of 8 consecutive rows, (b) the
@@ -176,6 +184,52 @@ struct LoadKCD {
     __device__ __forceinline__ void dma(uint32_t lds, const half_t *origin, int64_t k0) const
     {
         const half_t *base = origin + k0;
+        const uint32_t wave = lds + (threadIdx.x & ~63u) * 16;
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            const uint32_t m0 = __builtin_amdgcn_readfirstlane(wave + it * NT * 16);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :
+                         : "s"(m0), "v"(off[it]), "s"(base)
+                         : "memory");
+        }
+    }
+    __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
+    __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
+    static constexpr int NREG = 1;
+    static constexpr int NVMEM = 0;
+    static constexpr int NDMA = NL;
+};
+
+// ---- k-strided operand (memory [k][row]) fetched straight into LDS in its own layout,
+// [64 k][ROWS] with the 16-byte chunks of k row k swizzled by 2 (k & 3); the MFMA fragments
+// come out of it through ds_read_b64_tr_b16, which hands each lane of a 16-lane group 4
+// consecutive k of one row from a 4 k x 16 rows block (the swizzle spreads the 4 k rows of such
+// a block over all banks).  A wave fills 1 KB = 1024 / (2 ROWS) whole k rows per instruction.
+template <int ROWS, int NT>
+struct LoadKSD {
+    static constexpr int CPR = ROWS / 8;           // 16-byte chunks per k row
+    static_assert(BK * CPR % NT == 0 && CPR >= 8, "whole instructions per wave");
+    static constexpr int NL = BK * CPR / NT;
+    uint32_t off[NL];              // byte offset of the lane's chunk from (k = 0, row0)
+    int64_t ld;
+
+    __device__ __forceinline__ void init(int64_t ld_, int64_t rows_left, int64_t)
+    {
+        ld = ld_;
+#pragma unroll
+        for (int it = 0; it < NL; it++) {
+            const int c = threadIdx.x + it * NT;
+            const int k = c / CPR, q = (c % CPR) ^ (2 * (k & 3));
+            int64_t col = q * 8;
+            if (col > rows_left - 8) col = rows_left - 8;          // rows_left is a multiple of 8
+            off[it] = (uint32_t)((k * ld_ + col) * 2);
+        }
+    }
+    // lds = byte address in LDS of the tile buffer to fill; origin = &op[0][row0]
+    __device__ __forceinline__ void dma(uint32_t lds, const half_t *origin, int64_t k0) const
+    {
+        const half_t *base = origin + k0 * ld;
         const uint32_t wave = lds + (threadIdx.x & ~63u) * 16;
 #pragma unroll
         for (int it = 0; it < NL; it++) {
@@ -483,16 +537,27 @@ __device__ __forceinline__ void wait_vmem()
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
 
-// NBUF = 3: the k-contiguous operands are fetched straight into LDS two tiles ahead (three
-// LDS buffers); strided operands keep their register stages.  NBUF = 2: everything through
-// registers.
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES, int NBUF>
+typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+
+// 4 consecutive k of this lane's row out of a [k][row] tile (ds_read_b64_tr_b16)
+__device__ __forceinline__ uint2 lds_read_tr(const unsigned char *q)
+{
+    typedef __attribute__((address_space(3))) fp16x4_t *lds_ptr;
+    const fp16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4f16((lds_ptr)q);
+    uint2 r;
+    __builtin_memcpy(&r, &v, 8);
+    return r;
+}
+
+// DMA = true: both operands are fetched straight into LDS, NBUF - 1 tiles ahead, no register
+// stages (STAGES is 1); DMA = false: through registers, two LDS buffers.
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES, int NBUF, bool DMA>
 __global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN, NBUF))
 gemm_mfma_kernel(GemmArgs p)
 {
-    static_assert(NBUF == 2 || (NBUF == 3 && STAGES == 2 && AL == 8 && !KTAIL && (!TA || TB)),
-                  "direct loads: 16-byte aligned whole k tiles, at least one k-contiguous operand");
-    constexpr bool DMA_A = NBUF == 3 && !TA, DMA_B = NBUF == 3 && TB;
+    static_assert(DMA ? (STAGES == 1 && AL == 8 && !KTAIL) : NBUF == 2,
+                  "direct loads: 16-byte aligned operands, whole k tiles");
+    constexpr bool TR_A = DMA && TA, TR_B = DMA && !TB;           // fragments by transposing reads
     static_assert((WM % 2 == 0 || BM / WM == 32) && (WN % 2 == 0 || BN / WN == 32),
                   "tiles of a wave lie 32 WM rows apart: a multiple of 64 keeps their swizzle equal");
     constexpr int NT = WM * WN * 64;
@@ -549,7 +614,7 @@ gemm_mfma_kernel(GemmArgs p)
     const int l32 = lane & 31, lh = lane >> 5;
 
     // when both operands are strided they use disjoint halves of the block
-    constexpr bool UNI = TA && !TB && BM == BN && BM + BN == NT;  // one combined strided loader
+    constexpr bool UNI = !DMA && TA && !TB && BM == BN && BM + BN == NT;  // one combined strided loader
     // strided operands whose 8-row x 64-k items divide into 4- or 2-k pieces over all lanes
     // (128 rows on 256 lanes, 256 or 128 rows on 512 lanes): branch-free on every lane
     constexpr bool FITS_A = BM * 2 == NT || BM * 4 == NT, FITS_B = BN * 2 == NT || BN * 4 == NT;
@@ -563,8 +628,10 @@ gemm_mfma_kernel(GemmArgs p)
         UNI, LoadNone,
         typename std::conditional<HALF_B, LoadKSH<BN, NT, AL, KTAIL>,
                                   Loader<!TB, BN, NT, (TA && !TB) ? NT / 2 : 0, AL, KTAIL>>::type>::type LB_REG;
-    typedef typename std::conditional<DMA_A, LoadKCD<BM, NT>, LA_REG>::type LA;
-    typedef typename std::conditional<DMA_B, LoadKCD<BN, NT>, LB_REG>::type LB;
+    typedef typename std::conditional<
+        DMA, typename std::conditional<TA, LoadKSD<BM, NT>, LoadKCD<BM, NT>>::type, LA_REG>::type LA;
+    typedef typename std::conditional<
+        DMA, typename std::conditional<TB, LoadKCD<BN, NT>, LoadKSD<BN, NT>>::type, LB_REG>::type LB;
     LA la;
     LB lb;
     if constexpr (UNI) {
@@ -589,6 +656,15 @@ gemm_mfma_kernel(GemmArgs p)
     const int ar0 = wm * 32 + l32, br0 = wn * 32 + l32;
     const int asw = swz(ar0), bsw = swz(br0);
     constexpr int ASTEP = (TM > 1 ? 32 * WM : 0) * BK, BSTEP = (TN > 1 ? 32 * WN : 0) * BK;
+    // [k][row] tiles: byte offset of the lane's first transposing read (k step 0, first 32 x 32
+    // tile).  In its 16-lane group the lane addresses k row a4 (of 4), rows 4 b4 .. 4 b4 + 3
+    // (of 16); k steps, the second half of a fragment and further tiles add constants.
+    const int a4 = (lane >> 2) & 3, b4 = lane & 3, n16 = (lane >> 4) & 1;
+    auto tr_base = [&](int w32, int pitch) __attribute__((always_inline)) {
+        const int chunk = (w32 + 16 * n16) / 8 + (b4 >> 1);
+        return (8 * lh + a4) * pitch + ((chunk ^ (2 * a4)) << 4) + ((b4 & 1) << 3);
+    };
+    const int atr = tr_base(wm * 32, BM * 2), btr = tr_base(wn * 32, BN * 2);
 
     // MFMAs of k step ks run while the operand fragments of step ks + 1 are in flight from
     // LDS (two fragment sets): the wait before a step's MFMAs leaves the next step's reads
@@ -600,14 +676,33 @@ gemm_mfma_kernel(GemmArgs p)
         // spilling (16-byte aligned operands)
         constexpr bool PIPE = AL == 8;
         half8_t af[PIPE ? 2 : 1][TM], bf[PIPE ? 2 : 1][TN];
+        auto frag_tr = [&](const unsigned char *q, int pitch) __attribute__((always_inline)) {
+            const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * pitch);
+            const uint4 v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            half8_t f;
+            __builtin_memcpy(&f, &v, 16);
+            return f;
+        };
         auto frags = [&](int set, int ks) __attribute__((always_inline)) {
             const int q = ks * 2 + lh;
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-                af[set][i] = *reinterpret_cast<const half8_t *>(as + i * ASTEP + ((q ^ asw) << 3));
+            for (int i = 0; i < TM; i++) {
+                if (TR_A)
+                    af[set][i] = frag_tr(reinterpret_cast<const unsigned char *>(As + cur * BM * BK) + atr +
+                                             ks * 16 * (BM * 2) + i * (32 * WM * 2),
+                                         BM * 2);
+                else
+                    af[set][i] = *reinterpret_cast<const half8_t *>(as + i * ASTEP + ((q ^ asw) << 3));
+            }
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-                bf[set][j] = *reinterpret_cast<const half8_t *>(bs + j * BSTEP + ((q ^ bsw) << 3));
+            for (int j = 0; j < TN; j++) {
+                if (TR_B)
+                    bf[set][j] = frag_tr(reinterpret_cast<const unsigned char *>(Bs + cur * BN * BK) + btr +
+                                             ks * 16 * (BN * 2) + j * (32 * WN * 2),
+                                         BN * 2);
+                else
+                    bf[set][j] = *reinterpret_cast<const half8_t *>(bs + j * BSTEP + ((q ^ bsw) << 3));
+            }
         };
         if (PIPE) frags(0, 0);
 #pragma unroll
@@ -626,12 +721,12 @@ gemm_mfma_kernel(GemmArgs p)
             // pin that order for the instruction scheduler (it would otherwise sink each read
             // to just before its use): the first fragment set, then per k step its MFMAs
             // with the next step's LDS reads spread between them
-            constexpr int NM = TM * TN, NR = TM + TN;
+            constexpr int NM = TM * TN, NR = (TR_A ? 2 : 1) * TM + (TR_B ? 2 : 1) * TN;
             // with one register stage the global loads of the next tile (same scheduling region
             // when no operand is strided) must go first, so that their latency overlaps the
             // whole k tile; with two stages they are a tile ahead anyway and are left to the
             // scheduler (measured: pinning them first costs 5 %)
-            if (STAGES == 1) __builtin_amdgcn_sched_group_barrier(0x020, LA::NREG + LB::NREG, 0);
+            if (STAGES == 1 && !DMA) __builtin_amdgcn_sched_group_barrier(0x020, LA::NREG + LB::NREG, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
 #pragma unroll
             for (int ks = 0; ks + 1 < BK / 16; ks++) SchedStep<NM, NR, 0>::run();
@@ -639,16 +734,18 @@ gemm_mfma_kernel(GemmArgs p)
         }
     };
 
-    // Software pipeline over k tiles with STAGES register sets and NBUF LDS buffers.  Invariant
-    // at the start of tile t (cb = its LDS buffer): LDS[cb] holds tile t behind a barrier,
-    // register set (t + j - kt0) % STAGES holds tile t + j of the operands staged in registers
-    // for j = 1 .. STAGES - 1, set (t - kt0) % STAGES is free, and the direct loads of tile
-    // t + 1 are in flight to the next buffer.  A step issues the direct loads of tile t + 2 into
-    // the buffer tile t - 1 has left, loads tile t + STAGES into the free register set, runs the
-    // MFMAs of tile t, moves tile t + 1 from its set to the next LDS buffer, waits for the
-    // direct loads of tile t + 1 (everything but what this step issued) and ends in the one
-    // barrier of the k tile.  The main loop has no branch (all its loads are inside K); the
-    // last 2 STAGES - 1 tiles are peeled into steps that test what still exists.
+    // Software pipeline over k tiles.  Through registers (STAGES register sets, two LDS
+    // buffers): at the start of tile t, LDS[t & 1] holds tile t, register set
+    // (t + j - kt0) % STAGES holds tile t + j for j = 1 .. STAGES - 1 and set (t - kt0) % STAGES
+    // is free; a step loads tile t + STAGES into the free set, runs the MFMAs of tile t, moves
+    // tile t + 1 from its set to the other LDS buffer and ends in the one barrier of the k tile.
+    // Direct (NBUF LDS buffers): at the start of tile t its buffer is complete behind a barrier
+    // and the loads of tiles t + 1 .. t + NBUF - 2 are in flight; a step issues the loads of tile
+    // t + NBUF - 1 into the buffer tile t - 1 has left, runs the MFMAs of tile t, waits until
+    // only the loads issued after those of tile t + 1 are outstanding, and ends in the barrier.
+    // The main loop has no branch (all its loads are inside K); the last tiles are peeled
+    // into steps that test what still exists.
+    constexpr int LOOK = DMA ? NBUF - 1 : STAGES;                 // tiles between load and use
     auto next_buf = [](int b) __attribute__((always_inline)) { return b + 1 == NBUF ? 0 : b + 1; };
     auto lds_addr = [](const half_t *q) __attribute__((always_inline)) {
         return (uint32_t)(uintptr_t)q;                            // LDS byte address of a shared pointer
@@ -656,52 +753,53 @@ gemm_mfma_kernel(GemmArgs p)
     auto step = [&](auto set_c, auto main_c, int t, int cbv) __attribute__((always_inline)) {
         constexpr int U = decltype(set_c)::value, UN = (U + 1) % STAGES;
         constexpr bool MAIN = decltype(main_c)::value;
-        const int cb = NBUF == 2 ? (t & 1) : cbv, nb1 = next_buf(cb);
-        if (NBUF == 3 && (MAIN || t + 2 < nk)) {
-            const int nb2 = next_buf(nb1);
-            la.dma(lds_addr(As + nb2 * BM * BK), Ao, (int64_t)(t + 2) * BK);
-            lb.dma(lds_addr(Bs + nb2 * BN * BK), Bo, (int64_t)(t + 2) * BK);
-        }
-        if (MAIN || t + STAGES < nk) {
-            la.load(ra[U], Ao, (int64_t)(t + STAGES) * BK);
-            lb.load(rb[U], Bo, (int64_t)(t + STAGES) * BK);
+        const int cb = DMA ? cbv : (t & 1), nb1 = next_buf(cb);
+        if (MAIN || t + LOOK < nk) {
+            if (DMA) {
+                const int dst = NBUF == 2 ? nb1 : next_buf(nb1);
+                static_assert(!DMA || NBUF == 2 || NBUF == 3, "destination buffer above");
+                la.dma(lds_addr(As + dst * BM * BK), Ao, (int64_t)(t + LOOK) * BK);
+                lb.dma(lds_addr(Bs + dst * BN * BK), Bo, (int64_t)(t + LOOK) * BK);
+            } else {
+                la.load(ra[U], Ao, (int64_t)(t + LOOK) * BK);
+                lb.load(rb[U], Bo, (int64_t)(t + LOOK) * BK);
+            }
         }
         compute(cb);
-        if (MAIN || t + 1 < nk) {
+        if (!DMA && (MAIN || t + 1 < nk)) {
             la.store(ra[UN], As + nb1 * BM * BK);
             lb.store(rb[UN], Bs + nb1 * BN * BK);
         }
-        if (NBUF == 3) {
-            // everything older than this step's own loads has landed: tile t + 1 is in LDS
-            if (MAIN) wait_vmem<LA::NDMA + LB::NDMA + LA::NVMEM + LB::NVMEM>();
+        if (DMA) {
+            if (MAIN) wait_vmem<(LOOK - 1) * (LA::NDMA + LB::NDMA)>();
             else wait_vmem<0>();
         }
         __syncthreads();
     };
     {
-        if (NBUF == 3) {
-            la.dma(lds_addr(As), Ao, (int64_t)kt0 * BK);
-            lb.dma(lds_addr(Bs), Bo, (int64_t)kt0 * BK);
-            if (kt0 + 1 < nk) {
-                la.dma(lds_addr(As + BM * BK), Ao, (int64_t)(kt0 + 1) * BK);
-                lb.dma(lds_addr(Bs + BN * BK), Bo, (int64_t)(kt0 + 1) * BK);
-            }
-        }
-        la.load(ra[0], Ao, (int64_t)kt0 * BK);
-        lb.load(rb[0], Bo, (int64_t)kt0 * BK);
+        if (DMA) {
 #pragma unroll
-        for (int u = 1; u < STAGES; u++)
-            if (kt0 + u < nk) {
-                la.load(ra[u], Ao, (int64_t)(kt0 + u) * BK);
-                lb.load(rb[u], Bo, (int64_t)(kt0 + u) * BK);
-            }
-        const int b0 = NBUF == 2 ? (kt0 & 1) : 0;
-        la.store(ra[0], As + b0 * BM * BK);
-        lb.store(rb[0], Bs + b0 * BN * BK);
-        if (NBUF == 3) wait_vmem<0>();
+            for (int u = 0; u < LOOK; u++)
+                if (kt0 + u < nk) {
+                    la.dma(lds_addr(As + u * BM * BK), Ao, (int64_t)(kt0 + u) * BK);
+                    lb.dma(lds_addr(Bs + u * BN * BK), Bo, (int64_t)(kt0 + u) * BK);
+                }
+            wait_vmem<0>();
+        } else {
+            la.load(ra[0], Ao, (int64_t)kt0 * BK);
+            lb.load(rb[0], Bo, (int64_t)kt0 * BK);
+#pragma unroll
+            for (int u = 1; u < STAGES; u++)
+                if (kt0 + u < nk) {
+                    la.load(ra[u], Ao, (int64_t)(kt0 + u) * BK);
+                    lb.load(rb[u], Bo, (int64_t)(kt0 + u) * BK);
+                }
+            la.store(ra[0], As + (kt0 & 1) * BM * BK);
+            lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
+        }
         __syncthreads();
         int kt = kt0, cb = 0;
-        for (; kt + 2 * STAGES - 1 < nk; kt += STAGES) {
+        for (; kt + STAGES - 1 + LOOK < nk; kt += STAGES) {
             step(std::integral_constant<int, 0>{}, std::true_type{}, kt, cb);
             cb = next_buf(cb);
             if (STAGES > 1) {
@@ -713,12 +811,13 @@ gemm_mfma_kernel(GemmArgs p)
                 cb = next_buf(cb);
             }
         }
-        static_assert(STAGES >= 1 && STAGES <= 3, "peeled tail below covers up to 5 tiles");
-        if (kt + 0 < nk) { step(std::integral_constant<int, 0 % STAGES>{}, std::false_type{}, kt + 0, cb); cb = next_buf(cb); }
-        if (STAGES > 1 && kt + 1 < nk) { step(std::integral_constant<int, 1 % STAGES>{}, std::false_type{}, kt + 1, cb); cb = next_buf(cb); }
-        if (STAGES > 1 && kt + 2 < nk) { step(std::integral_constant<int, 2 % STAGES>{}, std::false_type{}, kt + 2, cb); cb = next_buf(cb); }
-        if (STAGES > 2 && kt + 3 < nk) { step(std::integral_constant<int, 3 % STAGES>{}, std::false_type{}, kt + 3, cb); cb = next_buf(cb); }
-        if (STAGES > 2 && kt + 4 < nk) { step(std::integral_constant<int, 4 % STAGES>{}, std::false_type{}, kt + 4, cb); cb = next_buf(cb); }
+        constexpr int TAIL = STAGES - 1 + LOOK;                   // tiles left at most
+        static_assert(STAGES >= 1 && STAGES <= 3 && TAIL <= 5, "peeled tail below covers up to 5 tiles");
+        if (TAIL > 0 && kt + 0 < nk) { step(std::integral_constant<int, 0 % STAGES>{}, std::false_type{}, kt + 0, cb); cb = next_buf(cb); }
+        if (TAIL > 1 && kt + 1 < nk) { step(std::integral_constant<int, 1 % STAGES>{}, std::false_type{}, kt + 1, cb); cb = next_buf(cb); }
+        if (TAIL > 2 && kt + 2 < nk) { step(std::integral_constant<int, 2 % STAGES>{}, std::false_type{}, kt + 2, cb); cb = next_buf(cb); }
+        if (TAIL > 3 && kt + 3 < nk) { step(std::integral_constant<int, 3 % STAGES>{}, std::false_type{}, kt + 3, cb); cb = next_buf(cb); }
+        if (TAIL > 4 && kt + 4 < nk) { step(std::integral_constant<int, 4 % STAGES>{}, std::false_type{}, kt + 4, cb); cb = next_buf(cb); }
     }
 
     // Epilogue through LDS (the operand buffers are free after the last barrier): a lane
@@ -782,13 +881,13 @@ gemm_mfma_kernel(GemmArgs p)
     }
 }
 
-template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES, int NBUF = 2>
+template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, int STAGES, int NBUF = 2, bool DMA = false>
 int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 {
     p.tiles_m = (int)((p.M + BM - 1) / BM);
     p.tiles_n = (int)((p.N + BN - 1) / BN);
     const size_t smem = (size_t)NBUF * (BM + BN) * BK * sizeof(half_t);
-    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES, NBUF>;
+    auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES, NBUF, DMA>;
     static bool attr_set = false;                 // one flag per instantiation
     if (!attr_set) {
         CACTI_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -805,9 +904,8 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 }
 
 // tile: 0 = 128 x 128 on 4 waves, two register stages (every loader is branch-free on 256
-// lanes); 1 = 256 x 128 on 8 waves; 2 = 256 x 256 on 8 waves (128 x 64 per wave; one register
-// stage, what the 128 accumulator registers leave room for); 3 = 64 x 64 on 4 waves;
-// 4 = 256 x 128 on 8 waves with the k-contiguous operands loaded straight into LDS
+// lanes); 1 = 256 x 128 on 8 waves, two register stages; 3 = 64 x 64 on 4 waves; 4 = 256 x 128
+// and 5 = 256 x 256 (128 x 64 per wave) on 8 waves with both operands loaded straight into LDS
 template <bool TA, bool TB>
 int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
 {
@@ -819,11 +917,9 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
     if (ktail) return launch_cfg<TA, TB, 128, 128, 2, 2, 8, true, 1>(p, nblk, st);
     switch (tile) {
         case 0: return launch_cfg<TA, TB, 128, 128, 2, 2, 8, false, 2>(p, nblk, st);
-        case 2: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1>(p, nblk, st);
         case 3: return launch_cfg<TA, TB, 64, 64, 2, 2, 8, false, 2>(p, nblk, st);
-        case 4:
-            if constexpr (!TA || TB) return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2, 3>(p, nblk, st);
-            else return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
+        case 4: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 1, 3, true>(p, nblk, st);
+        case 5: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1, 2, true>(p, nblk, st);
         default: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
     }
 }
@@ -892,21 +988,19 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
         if (forced >= 0) {
             tile = forced;
         } else {
-            // measured on MI355X at the step's shapes.  A not transposed (forward and dgrad
-            // products, M = tokens): one 8-wave 256 x 128 workgroup per CU fetches each B panel
-            // half as often as two 128 x 128 ones (+8..14 % on the projection and FFN shapes, and
-            // the best choice for the LM head too); with both operands k-contiguous (forward)
-            // they go straight into LDS (+8..12 % on the FFN and LM-head shapes, +2 % on the
-            // projections; with only A direct the dgrad layout loses 10 %, so it keeps its
-            // register stages).  The wgrad layout loses 5..17 % to 256 x 128's coarser tile
-            // count but gains 3..15 % from 256 x 256 with 128 x 64 per wave on the weight-sized
-            // outputs; small and batched products stay on 128 x 128.
+            // measured on MI355X at the step's shapes (TFLOP/s on cold operands, register
+            // path 128 x 128 or 256 x 128 -> direct loads).  A not transposed (forward and dgrad,
+            // M = tokens): 256 x 128, one workgroup per CU; NT 661..821 -> 707..881, NN 702..787
+            // -> 773..864; the LM head's 1000 tiles of 256 x 256 run at 1074 against 977.  Wgrad
+            // (both operands strided, weight-sized outputs): 256 x 256, 558..715 -> 755..932.
+            // Small and batched products stay on 128 x 128 through registers.
             tile = 0;
+            static const bool no_direct = getenv("CACTI_GEMM_NO_DIRECT") != nullptr;
             if (nblk == 1 && p.M >= 1024 && p.N >= 1024) {
-                static const bool no_direct = getenv("CACTI_GEMM_NO_DIRECT") != nullptr;
-                static const bool no_wide_tn = getenv("CACTI_GEMM_NO_WIDE_TN") != nullptr;
-                if (!ta) tile = tb && !no_direct ? 4 : 1;
-                else if (!tb && p.M >= 2048 && p.N >= 2048 && !no_wide_tn) tile = 2;
+                const int64_t tiles256 = ((p.M + 255) / 256) * ((p.N + 255) / 256);
+                if (no_direct) tile = ta ? 0 : 1;
+                else if (!ta) tile = tiles256 >= 768 ? 5 : 4;
+                else if (p.M >= 2048 && p.N >= 2048) tile = 5;
             }
         }
     }
