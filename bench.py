@@ -111,7 +111,7 @@ def kernel_symbol(label):
     The tile choice mirrors gemm_mfma_launch for 16-byte aligned operands and K % 64 == 0: with an
     output of at least 1024 x 1024 and one block, A not transposed runs 256 x 128 / 8 waves (from
     768 tiles of 256 x 256 on: that tile) and A transposed 256 x 256 / 8 waves from 2048 x 2048
-    outputs on, all with direct-to-LDS loads; everything else 128 x 128 / 4 waves through
+    outputs on (256 x 192 where that fills the CUs markedly better), all with direct-to-LDS loads; everything else 128 x 128 / 4 waves through
     registers."""
     ta, tb, H, M, N, K = gemm_dims(label)
     tile = "128, 128, 2, 2, 8, false, 2, 2, false"
@@ -120,7 +120,10 @@ def kernel_symbol(label):
         if not ta:
             tile = "256, 256, 2, 4, 8, false, 1, 2, true" if tiles256 >= 768 else "256, 128, 4, 2, 8, false, 1, 3, true"
         elif M >= 2048 and N >= 2048:
-            tile = "256, 256, 2, 4, 8, false, 1, 2, true"
+            fill = lambda t: t / (-(-t // N_CUS) * N_CUS)
+            tiles192 = ((M + 255) // 256) * ((N + 191) // 192)
+            tile = "256, 192, 4, 2, 8, false, 1, 2, true" if fill(tiles192) > 1.2 * fill(tiles256) \
+                else "256, 256, 2, 4, 8, false, 1, 2, true"
     return "gemm_mfma_kernel<%s, %s, %s>" % (str(ta).lower(), str(tb).lower(), tile)
 
 

@@ -334,7 +334,27 @@ def test_gemm_colmajor_entry(ops, oracle):
 
 
 # ---------------------------------------------------------------- attention block
-@pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100), (1024, 2, 100)])
+@pytest.mark.parametrize("ta", [0, 1])
+def test_head_slab_products_accumulate_in_place(ops, oracle, ta):
+    """C[:, h, :] += op(A_h) B[:, h, :] on [S, H, 100] slabs (every other head starts 8 bytes off a
+    16-byte boundary): each head's 100 columns get exactly its own product, nothing else moves."""
+    say("head slabs accumulate", ta)
+    S, H, Dh = 256, 4, 100
+    r = rng(1100 + ta)
+    a = randn16(r, (S, H, S), 0.1)
+    b, c0 = randn16(r, (S, H, Dh)), randn16(r, (S, H, Dh))
+    want = np.empty_like(c0)
+    for h in range(H):
+        want[:, h, :] = oracle.matmul(ta, 0, np.ascontiguousarray(a[:, h, :]),
+                                      np.ascontiguousarray(b[:, h, :]), 0.5, 1.0,
+                                      np.ascontiguousarray(c0[:, h, :]))
+    c = dev(c0)
+    ops.gemm_strided_batched(bool(ta), False, H, S, Dh, S, 0.5, dev(a), H * S, S, dev(b), H * Dh, Dh,
+                             1.0, c, H * Dh, Dh)
+    assert_parity(host(c), want, "slab accumulate")
+
+
+@pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100), (1024, 2, 100), (512, 4, 100), (384, 6, 100)])
 @pytest.mark.parametrize("tri", [False, True])
 def test_attention_block_via_thunks(ops, oracle, S, H, Dh, tri):
     """Q K^T -> causal softmax -> P V and the adjoint, composed as the reference stages them;
