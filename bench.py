@@ -69,18 +69,22 @@ def synth_inputs(cfg, seed=1, grad_scale=1024.0):
 # a streaming kernel of known size reads FETCH_SIZE = half its bytes and WRITE_SIZE = its
 # bytes, so bytes = (2.0 * FETCH_SIZE + 1.0 * WRITE_SIZE) * 1024
 GEMM_TRAFFIC_KIB = {
-    ("NT", 2048, 3200, 3200): (64068, 12800), ("NT", 2048, 3200, 8640): (172868, 12800),
-    ("NT", 2048, 8640, 3200): (159799, 34560), ("NT", 2048, 32000, 3200): (640965, 128000),
-    ("NN", 2048, 3200, 3200): (67274, 12800), ("NN", 2048, 3200, 8640): (176074, 12800),
-    ("NN", 2048, 8640, 3200): (159691, 34560), ("NN", 2048, 3200, 32000): (640147, 12800),
-    ("TN", 3200, 3200, 2048): (67640, 20000), ("TN", 8640, 3200, 2048): (165781, 54000),
-    ("TN", 3200, 8640, 2048): (165781, 54000), ("TN", 32000, 3200, 2048): (739452, 200000),
+    ("NT", 2048, 3200, 3200): (64224, 12800), ("NT", 2048, 3200, 8640): (172856, 12800),
+    ("NT", 2048, 8640, 3200): (128057 + 19248, 32768 + 1792),      # two launches: 8192 + 448 columns
+    ("NT", 2048, 32000, 3200): (383065, 128000),
+    ("NN", 2048, 3200, 3200): (64064, 12800), ("NN", 2048, 3200, 3200, "acc"): (70465, 12800),
+    ("NN", 2048, 3200, 8640): (172864, 12800), ("NN", 2048, 3200, 8640, "acc"): (179265, 12800),
+    ("NN", 2048, 8640, 3200): (159697, 34560), ("NN", 2048, 3200, 32000): (640083, 12800),
+    ("TN", 3200, 3200, 2048): (44234, 20000), ("TN", 8640, 3200, 2048): (109951, 54000),
+    ("TN", 3200, 8640, 2048): (96772, 54000), ("TN", 32000, 3200, 2048): (534651, 200000),
 }
 
 
 def gemm_traffic_bytes(label):
     m = GEMM_RE.match(label)
     key = (m.group(2) + m.group(3), int(m.group(5)), int(m.group(6)), int(m.group(7)))
+    if m.group(8) and key + ("acc",) in GEMM_TRAFFIC_KIB:
+        key = key + ("acc",)
     if key not in GEMM_TRAFFIC_KIB:
         return None
     f, w = GEMM_TRAFFIC_KIB[key]
