@@ -283,6 +283,32 @@ def test_gemm_small(ops, oracle, ta, tb, M, N, K):
         assert exact_frac(got, want) > 0.98
 
 
+# shapes that reach the direct-to-LDS kernels (outputs of at least 1024 x 1024, 16-byte aligned,
+# K % 64 == 0) with ragged last tiles in both directions, the 256 x 256 and 256 x 192 wgrad tiles,
+# and the forward product whose last columns go to a second launch of small tiles
+DIRECT_SHAPES = [
+    (0, 1, 1096, 1032, 192), (0, 0, 1096, 1032, 192), (1, 0, 1096, 1032, 128), (1, 1, 1032, 1096, 64),
+    (1, 0, 2056, 2304, 64),      # 256 x 256 tiles
+    (1, 0, 3200, 3200, 64),      # 256 x 192 tiles
+    (0, 1, 1024, 8640, 64),      # 64 full-round column tiles + 448 columns on 64 x 64 tiles
+    (0, 1, 2048, 24584, 64),     # forward product with at least 768 tiles of 256 x 256
+]
+
+
+@pytest.mark.parametrize("ta,tb,M,N,K", DIRECT_SHAPES)
+def test_gemm_direct_load_kernels(ops, oracle, ta, tb, M, N, K):
+    say("gemm direct", ta, tb, M, N, K)
+    r = rng(970 + M + N + K + 2 * ta + tb)
+    A = randn16(r, (K, M) if ta else (M, K))
+    B = randn16(r, (N, K) if tb else (K, N), 0.1)
+    C0 = randn16(r, (M, N))
+    for alpha, beta in [(1.0, 0.0), (0.5, 1.0)]:
+        want = oracle.matmul(ta, tb, A, B, alpha, beta, C0)
+        got = host(ops.gemm(dev(A), dev(B), bool(ta), bool(tb), alpha, beta, dev(C0)))
+        assert_parity(got, want, "gemm direct")
+        assert exact_frac(got, want) > 0.98
+
+
 @pytest.mark.parametrize("case", ["fwd", "dgrad", "wgrad"])
 def test_gemm_projection_shapes(ops, oracle, case):
     """The three GEMMs of one projection at a reduced token count (oracle finishes in seconds)."""
