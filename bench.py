@@ -110,40 +110,56 @@ def gemm_dims(label):
     return (m.group(2) == "T", m.group(3) == "T") + tuple(int(m.group(i)) for i in (4, 5, 6, 7))
 
 
+def plan_tokens_product(M, N):
+    """Mirror of plan_tokens_product in csrc/gemm_mfma.hip: (tile, columns of the first launch)."""
+    best, best_cost = (4, N), None
+    for tile, bn, round_cost in ((4, 128, 32768), (5, 256, 54613)):
+        tiles_m, tiles_n = (M + 255) // 256, (N + bn - 1) // bn
+        total = tiles_m * tiles_n
+        full = total // N_CUS
+        cols_main = full * N_CUS // tiles_m
+        rest = tiles_m * (tiles_n - cols_main)
+        if full >= 1 and cols_main < tiles_n and rest * bn * 4 <= N_CUS * 128:
+            cost, main_cols = full * round_cost + 12288, cols_main * bn
+        else:
+            cost, main_cols = -(-total // N_CUS) * round_cost, N
+        if best_cost is None or cost < best_cost:
+            best, best_cost = (tile, main_cols), cost
+    return best
+
+
+TILE_ARGS = {0: "128, 128, 2, 2, 8, false, 2, 2, false", 4: "256, 128, 4, 2, 8, false, 1, 3, true",
+             5: "256, 256, 2, 4, 8, false, 1, 2, true", 6: "256, 192, 4, 2, 8, false, 1, 2, true"}
+
+
 def kernel_symbol(label):
-    """Name of the HIP kernel instantiation a dense GEMM label runs on, as rocprofv3 prints it.
-    The tile choice mirrors gemm_mfma_launch for 16-byte aligned operands and K % 64 == 0: with an
-    output of at least 1024 x 1024 and one block, A not transposed runs 256 x 128 / 8 waves (from
-    768 tiles of 256 x 256 on: that tile) and A transposed 256 x 256 / 8 waves from 2048 x 2048
-    outputs on (256 x 192 where that fills the CUs markedly better), all with direct-to-LDS loads; everything else 128 x 128 / 4 waves through
-    registers."""
+    """Name of the HIP kernel instantiation a dense GEMM label runs on (its first launch), as
+    rocprofv3 prints it.  The tile choice mirrors gemm_mfma_launch for 16-byte aligned operands
+    and K % 64 == 0: with an output of at least 1024 x 1024 and one block, A not transposed runs
+    256 x 128 or 256 x 256 / 8 waves by plan_tokens_product, A transposed 256 x 256 / 8 waves from
+    2048 x 2048 outputs on (256 x 192 where that fills the CUs markedly better), all with
+    direct-to-LDS loads; everything else 128 x 128 / 4 waves through registers."""
     ta, tb, H, M, N, K = gemm_dims(label)
-    tile = "128, 128, 2, 2, 8, false, 2, 2, false"
+    tile = 0
     if H == 1 and M >= 1024 and N >= 1024:
-        tiles256 = ((M + 255) // 256) * ((N + 255) // 256)
         if not ta:
-            tile = "256, 256, 2, 4, 8, false, 1, 2, true" if tiles256 >= 768 else "256, 128, 4, 2, 8, false, 1, 3, true"
+            tile = plan_tokens_product(M, N)[0]
         elif M >= 2048 and N >= 2048:
             fill = lambda t: t / (-(-t // N_CUS) * N_CUS)
+            tiles256 = ((M + 255) // 256) * ((N + 255) // 256)
             tiles192 = ((M + 255) // 256) * ((N + 191) // 192)
-            tile = "256, 192, 4, 2, 8, false, 1, 2, true" if fill(tiles192) > 1.2 * fill(tiles256) \
-                else "256, 256, 2, 4, 8, false, 1, 2, true"
-    return "gemm_mfma_kernel<%s, %s, %s>" % (str(ta).lower(), str(tb).lower(), tile)
+            tile = 6 if fill(tiles192) > 1.2 * fill(tiles256) else 5
+    return "gemm_mfma_kernel<%s, %s, %s>" % (str(ta).lower(), str(tb).lower(), TILE_ARGS[tile])
 
 
 def is_split(label):
-    """True if the thunk issues two kernels (gemm_mfma_launch: the columns of an NT product
-    beyond its full rounds of 256 x 128 tiles go to a second launch of 64 x 64 tiles): its event
-    pair then brackets both, so it is left out of a single kernel's roofline sample."""
+    """True if the thunk issues two kernels (the columns beyond the full rounds of its tiles go to
+    a second launch of 64 x 64 tiles): its event pair then brackets both, so it is left out of a
+    single kernel's roofline sample."""
     ta, tb, H, M, N, K = gemm_dims(label)
-    if ta or not tb or H != 1 or M < 1024 or N < 1024 or K % 64:
+    if ta or H != 1 or M < 1024 or N < 1024 or K % 64:
         return False
-    if ((M + 255) // 256) * ((N + 255) // 256) >= 768:
-        return False
-    tiles_m, tiles_n = (M + 255) // 256, (N + 127) // 128
-    rounds = tiles_m * tiles_n // N_CUS
-    cols_main = rounds * N_CUS // tiles_m
-    return rounds >= 1 and cols_main < tiles_n and tiles_m * (tiles_n - cols_main) * 4 <= N_CUS
+    return plan_tokens_product(M, N)[1] < N
 
 
 def label_prefix(label):

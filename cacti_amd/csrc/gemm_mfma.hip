@@ -929,37 +929,69 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
     }
 }
 
-template <bool TA, bool TB>
-int launch_auto(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
+int cu_count()
 {
     static int cus = 0;
     if (!cus) {
         int dev = 0;
-        CACTI_HIP(hipGetDevice(&dev));
-        CACTI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
     }
-    static const bool no_split = getenv("CACTI_GEMM_NO_SPLIT") != nullptr;
-    // One 256 x 128 workgroup per CU runs in rounds of `cus` tiles.  When the last round would
-    // hold only a few tiles (N = 8640 at 2048 tokens: 2 full rounds + 32 tiles, a third of
-    // the launch time for 6 % of the work), the columns of the full rounds go to one launch
-    // and the remaining ones to a second launch of 64 x 64 tiles, which spreads them over
-    // every CU: -12..19 % at that shape.  (The dgrad layout would gain 8 %; it is left whole so
-    // that each of its launches stays one kernel.)
-    if ((tile == 1 || tile == 4) && !TA && TB && nblk == 1 && align >= 8 && p.K % BK == 0 && p.tri == 0 &&
-        !no_split) {
-        const int64_t tiles_m = (p.M + 255) / 256, tiles_n = (p.N + 127) / 128;
-        const int64_t rounds = tiles_m * tiles_n / cus;
-        const int64_t cols_main = rounds * cus / tiles_m;
-        const int64_t rest = tiles_m * (tiles_n - cols_main);
-        if (rounds >= 1 && cols_main < tiles_n && rest * 4 <= cus) {
-            GemmArgs a = p, b = p;
-            a.N = cols_main * 128;
-            b.N = p.N - a.N;
-            b.B = p.B + (TB ? a.N * p.ldb : a.N);
-            b.C = p.C + a.N;
-            const int rc = launch_tile<TA, TB>(tile, align, a, nblk, st);
-            return rc ? rc : launch_tile<TA, TB>(3, align, b, nblk, st);
+    return cus;
+}
+
+// How a large product with A not transposed (M = tokens) is cut into workgroups.  One workgroup
+// per CU runs in rounds of `cus` tiles, and a last round that holds only a few tiles costs as
+// much as a full one (N = 8640 at 2048 tokens: 544 tiles of 256 x 128 = 2 rounds + 32 tiles).
+// The columns of the full rounds can instead go to one launch and the few remaining ones to a
+// second launch of 64 x 64 tiles, which spreads them over every CU.  The plan compares
+// 256 x 128 tiles with 256 x 256 tiles (measured 1.2 x the rate per tile area: 883 -> 1075
+// TFLOP/s on 2048 x 8192 x 3200) by rounds x tile area / rate, the second launch costing 3/8 of
+// a 256 x 128 round.  At 2048 tokens: N = 3200 -> 200 tiles of 256 x 128 (one round); N = 8640
+// -> 256 tiles of 256 x 256 + 448 columns (135 -> 122 us); N = 32000 -> 1000 tiles of 256 x 256.
+struct Plan {
+    int tile;               // 4 or 5
+    int64_t cols_main;      // columns of the first launch (N: a single launch)
+};
+Plan plan_tokens_product(int64_t M, int64_t N, bool may_split)
+{
+    const int64_t cus = cu_count();
+    Plan best{4, N};
+    int64_t best_cost = -1;
+    const int tiles[2] = {4, 5};
+    const int64_t widths[2] = {128, 256}, round_cost[2] = {32768, 54613};   // 256 bn / rate
+    for (int c = 0; c < 2; c++) {
+        const int64_t bn = widths[c], tiles_m = (M + 255) / 256, tiles_n = (N + bn - 1) / bn;
+        const int64_t total = tiles_m * tiles_n, full = total / cus;
+        const int64_t cols_main = full * cus / tiles_m, rest = tiles_m * (tiles_n - cols_main);
+        int64_t cost, main_cols;
+        if (may_split && full >= 1 && cols_main < tiles_n && rest * bn * 4 <= cus * 128) {
+            cost = full * round_cost[c] + 12288;
+            main_cols = cols_main * bn;
+        } else {
+            cost = (total + cus - 1) / cus * round_cost[c];
+            main_cols = N;
         }
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = Plan{tiles[c], main_cols};
+        }
+    }
+    return best;
+}
+
+template <bool TA, bool TB>
+int launch_auto(int tile, int64_t cols_main, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
+{
+    if (cols_main > 0 && cols_main < p.N) {
+        GemmArgs a = p, b = p;
+        a.N = cols_main;
+        b.N = p.N - a.N;
+        b.B = p.B + (TB ? a.N * p.ldb : a.N);
+        b.C = p.C + a.N;
+        const int rc = launch_tile<TA, TB>(tile, align, a, nblk, st);
+        return rc ? rc : launch_tile<TA, TB>(3, align, b, nblk, st);
     }
     return launch_tile<TA, TB>(tile, align, p, nblk, st);
 }
@@ -984,6 +1016,7 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
         q.gm = gm;
         q.xcd = xcd;
     }
+    int64_t cols_main = 0;                        // > 0: a second launch takes the columns from here on
     if (tile < 0) {
         static int forced = -2;
         if (forced == -2) {
@@ -995,25 +1028,26 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
         } else {
             // measured on MI355X at the step's shapes (TFLOP/s on cold operands, register
             // path 128 x 128 or 256 x 128 -> direct loads).  A not transposed (forward and dgrad,
-            // M = tokens): 256 x 128, one workgroup per CU; NT 661..821 -> 707..881, NN 702..787
-            // -> 773..864; the LM head's 1000 tiles of 256 x 256 run at 1074 against 977.  Wgrad
-            // (both operands strided, weight-sized outputs): 256 x 256, 558..715 -> 755..932.
+            // M = tokens): NT 661..821 -> 707..881, NN 702..787 -> 773..864 on 256 x 128, one
+            // workgroup per CU; 256 x 256 where its rounds fit (plan_tokens_product).  Wgrad (both
+            // operands strided, weight-sized outputs): 256 x 256, 558..715 -> 755..932.
             // Small and batched products stay on 128 x 128 through registers.
             tile = 0;
             static const bool no_direct = getenv("CACTI_GEMM_NO_DIRECT") != nullptr;
+            static const bool no_split = getenv("CACTI_GEMM_NO_SPLIT") != nullptr;
             if (nblk == 1 && p.M >= 1024 && p.N >= 1024) {
-                const int64_t tiles256 = ((p.M + 255) / 256) * ((p.N + 255) / 256);
-                if (no_direct) tile = ta ? 0 : 1;
-                else if (!ta) tile = tiles256 >= 768 ? 5 : 4;
-                else if (p.M >= 2048 && p.N >= 2048) {
+                if (no_direct) {
+                    tile = ta ? 0 : 1;
+                } else if (!ta) {
+                    const bool direct_ok = align >= 8 && p.K % BK == 0;     // else launch_tile ignores the tile
+                    const Plan plan = plan_tokens_product(p.M, p.N, direct_ok && p.tri == 0 && !no_split);
+                    tile = plan.tile;
+                    cols_main = plan.cols_main;
+                } else if (p.M >= 2048 && p.N >= 2048) {
                     // 256 x 192 where its tile count fills the CUs markedly better (3200 x 3200:
                     // 221 tiles in one round against 169; +5 %)
-                    static int cus = 0;
-                    if (!cus) {
-                        int dev = 0;
-                        CACTI_HIP(hipGetDevice(&dev));
-                        CACTI_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-                    }
+                    const int64_t cus = cu_count();
+                    const int64_t tiles256 = ((p.M + 255) / 256) * ((p.N + 255) / 256);
                     const int64_t tiles192 = ((p.M + 255) / 256) * ((p.N + 191) / 192);
                     auto fill = [&](int64_t tiles) { return (double)tiles / (double)((tiles + cus - 1) / cus * cus); };
                     tile = fill(tiles192) > 1.2 * fill(tiles256) ? 6 : 5;
@@ -1021,10 +1055,10 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             }
         }
     }
-    if (!ta && !tb) return launch_auto<false, false>(tile, align, q, nblk, st);
-    if (!ta && tb) return launch_auto<false, true>(tile, align, q, nblk, st);
-    if (ta && !tb) return launch_auto<true, false>(tile, align, q, nblk, st);
-    return launch_auto<true, true>(tile, align, q, nblk, st);
+    if (!ta && !tb) return launch_auto<false, false>(tile, cols_main, align, q, nblk, st);
+    if (!ta && tb) return launch_auto<false, true>(tile, cols_main, align, q, nblk, st);
+    if (ta && !tb) return launch_auto<true, false>(tile, cols_main, align, q, nblk, st);
+    return launch_auto<true, true>(tile, cols_main, align, q, nblk, st);
 }
 
 }  // namespace cacti
