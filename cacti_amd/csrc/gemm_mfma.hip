@@ -42,6 +42,7 @@
 #include "common.h"
 #include "gemm_internal.h"
 
+#include <cmath>
 #include <type_traits>
 
 using namespace cacti;
@@ -894,6 +895,19 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
                                       (int)smem));
         attr_set = true;
     }
+    if (p.gm <= 0) {
+        // tile rows per group of the walk.  An XCD works on a band of tiles / 8 consecutive tiles,
+        // i.e. on gm tile rows x band / gm tile columns at a time, and fetches gm A panels and
+        // band / gm B panels per k tile into its L2: least for gm = sqrt(band BN / BM).  (Run
+        // time hardly reacts, the re-reads being served by the MALL; the L2-miss traffic does:
+        // -25 % at 2048 x 3200 x 8640.)
+        p.gm = 8;
+        if (nblk == 1) {
+            const double band = (double)p.tiles_m * p.tiles_n / 8.0;
+            const int g = (int)(sqrt(band * BN / BM) + 0.5);
+            p.gm = g < 1 ? 1 : (g > 8 ? 8 : g);
+        }
+    }
     p.pair = (p.tri >= 2 && p.tiles_m % 2 == 0) ? 1 : 0;
     const int64_t nwg = (int64_t)(p.pair ? p.tiles_m / 2 : p.tiles_m) * p.tiles_n * nblk;
     CACTI_REQUIRE(nwg < (int64_t)1 << 31, CACTI_E_NOTIMPL, "gemm: %lld workgroups exceed the grid limit",
@@ -1007,9 +1021,9 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
     GemmArgs q = p;
     {
         static int gm = 0, xcd = -1;
-        if (!gm) {
+        if (gm == 0) {
             const char *e = getenv("CACTI_GEMM_GM");
-            gm = e ? atoi(e) : 8;
+            gm = e ? atoi(e) : -1;                  // -1: chosen per launch
             e = getenv("CACTI_GEMM_XCD");
             xcd = e ? atoi(e) : 1;
         }
