@@ -69,15 +69,15 @@ def synth_inputs(cfg, seed=1, grad_scale=1024.0):
 # a streaming kernel of known size reads FETCH_SIZE = half its bytes and WRITE_SIZE = its
 # bytes, so bytes = (2.0 * FETCH_SIZE + 1.0 * WRITE_SIZE) * 1024
 GEMM_TRAFFIC_KIB = {
-    ("NT", 2048, 3200, 3200): (64070, 12800), ("NT", 2048, 3200, 8640): (172864, 12800),
-    ("NT", 2048, 8640, 3200): (76884 + 19248, 32768 + 1792),       # two launches: 8192 + 448 columns
-    ("NT", 2048, 32000, 3200): (384416, 128000),
-    ("NN", 2048, 3200, 3200): (64064, 12800), ("NN", 2048, 3200, 3200, "acc"): (70465, 12800),
-    ("NN", 2048, 3200, 8640): (172864, 12800), ("NN", 2048, 3200, 8640, "acc"): (179266, 12800),
-    ("NN", 2048, 8640, 3200): (76886 + 19250, 32768 + 1792),       # two launches
-    ("NN", 2048, 3200, 32000): (640118, 12800),
-    ("TN", 3200, 3200, 2048): (44234, 20000), ("TN", 8640, 3200, 2048): (109942, 54000),
-    ("TN", 3200, 8640, 2048): (96498, 54000), ("TN", 32000, 3200, 2048): (549026, 200000),
+    ("NT", 2048, 3200, 3200): (48063, 12800), ("NT", 2048, 3200, 8640): (129663, 12800),
+    ("NT", 2048, 8640, 3200): (76884 + 17648, 32768 + 1792),       # two launches: 8192 + 448 columns
+    ("NT", 2048, 32000, 3200): (382107, 128000),
+    ("NN", 2048, 3200, 3200): (48064, 12800), ("NN", 2048, 3200, 3200, "acc"): (54465, 12800),
+    ("NN", 2048, 3200, 8640): (129664, 12800), ("NN", 2048, 3200, 8640, "acc"): (136065, 12800),
+    ("NN", 2048, 8640, 3200): (76886 + 17650, 32768 + 1792),       # two launches
+    ("NN", 2048, 3200, 32000): (480064, 12800),
+    ("TN", 3200, 3200, 2048): (46154, 20000), ("TN", 8640, 3200, 2048): (109965, 54000),
+    ("TN", 3200, 8640, 2048): (95674, 54000), ("TN", 32000, 3200, 2048): (516334, 200000),
 }
 
 

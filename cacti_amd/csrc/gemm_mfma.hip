@@ -42,7 +42,6 @@
 #include "common.h"
 #include "gemm_internal.h"
 
-#include <cmath>
 #include <type_traits>
 
 using namespace cacti;
@@ -898,14 +897,20 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
     if (p.gm <= 0) {
         // tile rows per group of the walk.  An XCD works on a band of tiles / 8 consecutive tiles,
         // i.e. on gm tile rows x band / gm tile columns at a time, and fetches gm A panels and
-        // band / gm B panels per k tile into its L2: least for gm = sqrt(band BN / BM).  (Run
+        // band / gm B panels per k tile into its L2: the power of two with the fewest rows fetched.  (Run
         // time hardly reacts, the re-reads being served by the MALL; the L2-miss traffic does:
         // -25 % at 2048 x 3200 x 8640.)
         p.gm = 8;
         if (nblk == 1) {
             const double band = (double)p.tiles_m * p.tiles_n / 8.0;
-            const int g = (int)(sqrt(band * BN / BM) + 0.5);
-            p.gm = g < 1 ? 1 : (g > 8 ? 8 : g);
+            double best = 0;
+            for (int g = 8; g >= 2; g /= 2) {             // ties: the larger group
+                const double fetched = g * (double)BM + band / g * (double)BN;
+                if (best == 0 || fetched < best) {
+                    best = fetched;
+                    p.gm = g;
+                }
+            }
         }
     }
     p.pair = (p.tri >= 2 && p.tiles_m % 2 == 0) ? 1 : 0;
