@@ -168,25 +168,29 @@ def label_prefix(label):
     return label.split(",")[0]
 
 
+CPU_SAMPLE_LAYERS = 3
+
+
 def cpu_baseline(cfg):
-    """The CPU port (the oracle) on a bounded sample of the same workload: one decoder layer
-    and the LM head + loss at full shapes, forward + backward, extrapolated to 26 layers."""
+    """The CPU port (the oracle) on a bounded sample of the same workload (about 10 s of CPU
+    work): the LM head + loss alone and with 3 decoder layers at full shapes, forward + backward,
+    extrapolated to 26 layers."""
     from oracle import oracle as o
     from tests.llama_ref import make_inputs
     times = {}
-    for L in (0, 1):
+    for L in (0, CPU_SAMPLE_LAYERS):
         c = dict(cfg, L=L)
         ocfg, flat, tok, lm_tok, scale = make_inputs(c, seed=0, norm_mean=1.0, grad_scale=1024.0)
         t0 = time.time()
         o.llama_step(ocfg, flat, tok, lm_tok, scale)
         times[L] = time.time() - t0
         log("cpu_baseline: oracle L=%d fwd+bwd %.2f s" % (L, times[L]))
-    layer = max(times[1] - times[0], 1e-9)
+    layer = max(times[CPU_SAMPLE_LAYERS] - times[0], 1e-9) / CPU_SAMPLE_LAYERS
     full = times[0] + cfg["L"] * layer
     return {"value": cfg["S"] / full, "unit": "tokens/s", "cores": o.num_threads(), "kind": "port",
-            "sample": "oracle fwd+bwd of 1 of %d layers (%.2f s) and of embedding+LM head+loss "
+            "sample": "oracle fwd+bwd of %d of %d layers (%.2f s each) and of embedding+LM head+loss "
                       "(%.2f s) at full shapes, S=%d; step time extrapolated as head + %d x layer"
-                      % (cfg["L"], layer, times[0], cfg["S"], cfg["L"])}
+                      % (CPU_SAMPLE_LAYERS, cfg["L"], layer, times[0], cfg["S"], cfg["L"])}
 
 
 def run_step(args):
