@@ -300,8 +300,29 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nbl
         }
     }
     hipStream_t st = (hipStream_t)stream;
+    p.win = 0;
     if (vec >= 4 && !ta && tb && K <= 128 && beta == 0.f && tri <= 1)
         return gemm_nt_smallk_launch(p, nblk, st);
+    // The attention products with a [sequence, heads, head_dim] operand: A (probabilities or
+    // their adjoint) is 16-byte aligned, B and C are per-head slabs whose offset (head_dim 100)
+    // is only a multiple of 8 bytes.  Addressed from the 16-byte boundary below each slab they
+    // take the direct-load path; the extra columns read stay inside the columns the blocks
+    // cover in one row of B (checked here).
+    if (vec == 4 && !tb && nblk > 1 && mult(K, 64) && mult(ta ? M : K, 8) && mult(lda, 8) &&
+        mult(stride_a, 8) && aligned(A, 16) && mult(ldb, 8) && mult(ldc, 8) && aligned(B, 16) &&
+        aligned(C, 16) && (stride_b & 7) == (stride_c & 7) && !getenv("CACTI_GEMM_NO_WINDOW")) {
+        const int64_t row_end = (nblk - 1) * stride_b + N;
+        bool inside = stride_b >= 0 && row_end <= ldb;
+        for (int64_t bz = 0; bz < nblk && inside; bz++) {
+            const int64_t shift = (bz * stride_b) & 7;
+            const int64_t first = bz * stride_b - shift;          // >= 0: bz * stride_b >= shift
+            inside = first + (shift + N + 7) / 8 * 8 <= row_end;
+        }
+        if (inside) {
+            p.win = 1;
+            return gemm_mfma_launch(ta, tb, p, nblk, 8, -1, st);
+        }
+    }
     if (vec >= 4) return gemm_mfma_launch(ta, tb, p, nblk, vec, -1, st);
     if (!ta && !tb) return launch_vec<false, false>(vec, p, nblk, st);
     if (!ta && tb) return launch_vec<false, true>(vec, p, nblk, st);

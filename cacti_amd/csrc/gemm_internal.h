@@ -26,6 +26,10 @@ struct GemmArgs {
     int tri;
     int gm, xcd;          // tile walk: rows per group; 1 = XCD-banded numbering
     int pair;             // 1: a workgroup computes tile rows r and tiles_m - 1 - r (tri 2 / 3)
+    // 1: B ([K][N] row-major) and C are addressed per block from the 16-byte boundary at or
+    // below their first column (column window); set by the entry point when A is 16-byte
+    // aligned and B, C are only 8-byte aligned because of their batch stride
+    int win;
 };
 constexpr int kTriPad = 256;
 

@@ -71,28 +71,6 @@ __device__ __forceinline__ uint4 ld8(const half_t *base, uint32_t off0, uint32_t
     return make_uint4(lo.x, lo.y, hi.x, hi.y);
 }
 
-// old C tile for the beta path: zero outside the matrix
-template <int AL>
-__device__ __forceinline__ uint4 load8_guarded(const half_t *p, int64_t n)
-{
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (AL == 8) {
-        if (n > 0) v = *reinterpret_cast<const uint4 *>(p);
-    } else {
-        if (n > 0) {
-            const uint2 lo = *reinterpret_cast<const uint2 *>(p);
-            v.x = lo.x;
-            v.y = lo.y;
-        }
-        if (n > 4) {
-            const uint2 hi = *reinterpret_cast<const uint2 *>(p + 4);
-            v.z = hi.x;
-            v.w = hi.y;
-        }
-    }
-    return v;
-}
-
 // ---- k-contiguous operand (memory [row][k]): chunk c -> row c / 8, k-chunk c % 8 ----------
 template <int ROWS, int NT, int AL, bool KTAIL>
 struct LoadKC {
@@ -603,8 +581,15 @@ gemm_mfma_kernel(GemmArgs p)
     if (p.tri == 3) kt0 = (int)(m0 / BK);
 
     const half_t *A = p.A + bz * p.sa;
-    const half_t *B = p.B + bz * p.sb;
-    half_t *C = p.C + bz * p.sc;
+    // column window (p.win): the [k][n] operand B and C of block bz start 8 bytes off a 16-byte
+    // boundary when bz * sb is an odd multiple of 4 (head_dim 100).  Both are then addressed
+    // from the boundary before: column `shift` of this view is the block's column 0, columns
+    // below it and from nw on hold the neighbouring blocks' data, are multiplied like the rest
+    // and never stored.
+    const int shift = p.win ? (int)((bz * p.sb) & 7) : 0;
+    const int64_t nw = p.N + shift;                               // end of the window
+    const half_t *B = p.B + bz * p.sb - shift;
+    half_t *C = p.C + bz * p.sc - shift;
     // tile origins: &op[row0][0] for a k-contiguous operand, &op[0][row0] for a strided one
     const half_t *Ao = TA ? A + m0 : A + m0 * p.lda;
     const half_t *Bo = TB ? B + n0 * p.ldb : B + n0;
@@ -635,10 +620,10 @@ gemm_mfma_kernel(GemmArgs p)
     LA la;
     LB lb;
     if constexpr (UNI) {
-        la.init(Ao, p.lda, p.M - m0, Bo, p.ldb, p.N - n0, p.K);
+        la.init(Ao, p.lda, p.M - m0, Bo, p.ldb, nw - n0, p.K);
     } else {
         la.init(p.lda, p.M - m0, p.K);
-        lb.init(p.ldb, p.N - n0, p.K);
+        lb.init(p.ldb, (p.win ? (nw + 7) / 8 * 8 : nw) - n0, p.K);
     }
     uint4 ra[STAGES][LA::NREG], rb[STAGES][LB::NREG];
 
@@ -835,7 +820,23 @@ gemm_mfma_kernel(GemmArgs p)
         for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
             const int row = c / CPRC, cc = c % CPRC;
             const int64_t m = m0 + row, n = n0 + cc * 8;
-            const uint4 v = load8_guarded<AL>(C + m * p.ldc + n, m < p.M ? p.N - n : 0);
+            const bool lo = m < p.M && n >= shift && n < nw, hi = m < p.M && n + 4 >= shift && n + 4 < nw;
+            const half_t *cp = C + m * p.ldc + n;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (AL == 8 && lo && hi) {
+                v = *reinterpret_cast<const uint4 *>(cp);
+            } else {
+                if (lo) {
+                    const uint2 t = *reinterpret_cast<const uint2 *>(cp);
+                    v.x = t.x;
+                    v.y = t.y;
+                }
+                if (hi) {
+                    const uint2 t = *reinterpret_cast<const uint2 *>(cp + 4);
+                    v.z = t.x;
+                    v.w = t.y;
+                }
+            }
             *reinterpret_cast<uint4 *>(Cs + row * BN + ((cc ^ (row & CSW)) << 3)) = v;
         }
         __syncthreads();
@@ -867,14 +868,15 @@ gemm_mfma_kernel(GemmArgs p)
     for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
         const int row = c / CPRC, cc = c % CPRC;
         const int64_t m = m0 + row, n = n0 + cc * 8;
-        if (m >= p.M || n >= p.N) continue;
+        if (m >= p.M) continue;
+        const bool lo = n >= shift && n < nw, hi = n + 4 >= shift && n + 4 < nw;   // 4-column halves
         const uint4 v = *reinterpret_cast<const uint4 *>(Cs + row * BN + ((cc ^ (row & CSW)) << 3));
         half_t *cp = C + m * p.ldc + n;
-        if (AL == 8) {
+        if (AL == 8 && lo && hi) {
             *reinterpret_cast<uint4 *>(cp) = v;
         } else {
-            *reinterpret_cast<uint2 *>(cp) = make_uint2(v.x, v.y);
-            if (p.N - n > 4) *reinterpret_cast<uint2 *>(cp + 4) = make_uint2(v.z, v.w);
+            if (lo) *reinterpret_cast<uint2 *>(cp) = make_uint2(v.x, v.y);
+            if (hi) *reinterpret_cast<uint2 *>(cp + 4) = make_uint2(v.z, v.w);
         }
     }
     __syncthreads();                          // the staging buffer is read out before the next tile's operands land
@@ -885,7 +887,7 @@ template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, 
 int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 {
     p.tiles_m = (int)((p.M + BM - 1) / BM);
-    p.tiles_n = (int)((p.N + BN - 1) / BN);
+    p.tiles_n = (int)((p.N + (p.win ? 4 : 0) + BN - 1) / BN);
     const size_t smem = (size_t)NBUF * (BM + BN) * BK * sizeof(half_t);
     auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES, NBUF, DMA>;
     static bool attr_set = false;                 // one flag per instantiation
@@ -924,8 +926,8 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 
 // tile: 0 = 128 x 128 on 4 waves, two register stages (every loader is branch-free on 256
 // lanes); 1 = 256 x 128 on 8 waves, two register stages; 3 = 64 x 64 on 4 waves; 4 = 256 x 128,
-// 5 = 256 x 256 (128 x 64 per wave) and 6 = 256 x 192 (64 x 96 per wave) on 8 waves with both
-// operands loaded straight into LDS
+// 5 = 256 x 256 (128 x 64 per wave), 6 = 256 x 192 (64 x 96 per wave) and 7 = 128 x 128 (64 x 32
+// per wave) on 8 waves with both operands loaded straight into LDS
 template <bool TA, bool TB>
 int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
 {
@@ -944,6 +946,7 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
         case 4: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 1, 3, true>(p, nblk, st);
         case 5: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1, 2, true>(p, nblk, st);
         case 6: return launch_cfg<TA, TB, 256, 192, 4, 2, 8, false, 1, 2, true>(p, nblk, st);
+        case 7: return launch_cfg<TA, TB, 128, 128, 2, 4, 8, false, 1, 3, true>(p, nblk, st);
         default: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
     }
 }
@@ -1053,6 +1056,9 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             // Small and batched products stay on 128 x 128 through registers.
             tile = 0;
             static const bool no_direct = getenv("CACTI_GEMM_NO_DIRECT") != nullptr;
+            // the attention products on per-head slabs: 128 x 128, 8 waves of 64 x 32, three
+            // LDS buffers (-5 us per launch against the register path with 8 waves)
+            if (p.win) tile = 7;
             static const bool no_split = getenv("CACTI_GEMM_NO_SPLIT") != nullptr;
             if (nblk == 1 && p.M >= 1024 && p.N >= 1024) {
                 if (no_direct) {
