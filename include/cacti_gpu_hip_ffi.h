@@ -95,7 +95,10 @@ int cacti_hip_gemm_f16(int ta, int tb, int64_t M, int64_t N, int64_t K, float al
  * BlockMatrixMulF16F32GpuThunkImpl::_enter, src/thunk/op.rs:5027-5471
  * (cublasGemmBatchedEx, cacti_gpu_cu_ffi/src/lib.rs:793-885).  No padding of
  * the inner dimension is needed (the reference pads Dh 100 -> 104,
- * src/op.rs:1454-1482). */
+ * src/op.rs:1454-1482).  When the blocks of a not transposed B lie side by side in
+ * its rows (stride_b < ldb), a block's product may read columns of the neighbouring
+ * blocks in the same row, never anything outside the columns
+ * [0, (nblk - 1) * stride_b + N) of B's rows; C is written only inside each block. */
 int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N,
                                        int64_t K, float alpha, const void *A, int64_t lda,
                                        int64_t stride_a, const void *B, int64_t ldb,
