@@ -230,7 +230,7 @@ def run_step(args):
                "total_ms_per_step": tot_ms / n_survey}
         if fl is not None:
             ent["tflops"] = fl / (tot_ms / cnt * 1e-3) / 1e12
-            if label.startswith("matmul"):
+            if label.startswith("matmul") and not is_split(label):     # one thunk = one launch
                 s_ = by_sym.setdefault(kernel_symbol(label), [0.0, set()])
                 s_[0] += tot_ms
                 s_[1].add(label_prefix(label))
@@ -238,7 +238,7 @@ def run_step(args):
     dev_ms = sum(v[1] for v in rep.values()) / n_survey
     sym, (_, prefixes) = max(by_sym.items(), key=lambda kv: kv[1][0])
     assert len(prefixes) == 1, prefixes
-    prefix = prefixes.pop()
+    prefix = next(iter(prefixes))
 
     # timed region: exactly K steps, events around every EVENT_STRIDE-th launch of the dominant
     # kernel (the stride is coprime to the 7 such launches per layer, so all shapes are sampled)
@@ -262,11 +262,13 @@ def run_step(args):
     ms = dt / args.steps * 1e3
     tokens_s = cfg["S"] * args.steps / dt
 
-    rep = {label: v for label, v in rep.items() if not is_split(label)}
+    # the filter matches by label prefix: keep the launches that are exactly one launch of the
+    # dominant kernel
+    rep = {label: v for label, v in rep.items() if not is_split(label) and kernel_symbol(label) == sym}
+    assert rep, "no sampled launch of %s" % sym
     fl = sum(gemm_flops(label) * cnt for label, (cnt, _) in rep.items())
     sec = sum(tot_ms for _, tot_ms in rep.values()) * 1e-3
     cnt = sum(c for c, _ in rep.values())
-    assert all(kernel_symbol(label) == sym for label in rep), (sym, list(rep))
     achieved = fl / sec / 1e12
     tr = [(gemm_traffic_bytes(label), c) for label, (c, _) in rep.items()]
     traffic = None if any(t is None for t, _ in tr) else sum(t * c for t, c in tr) / cnt
