@@ -5,6 +5,7 @@ on one MI355X, with the roofline of the dominant kernel and the CPU port timed b
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--pool-gb G] [--no-cpu-baseline]
     python bench.py --workload adjoints      # HBM-bound adjoint kernels at 3B shapes
     python bench.py --workload gemm          # every GEMM shape of the step, standalone
+    python bench.py --workload digests       # NaN counts + abs-log2 histograms of all parameters and gradients
 
 Prints ONE JSON line on stdout.  A step = reset + stage + vadd_vjp + compile + resume of
 the 26-layer cycle (the reference's per-cycle control flow), inputs resident on the device
@@ -419,6 +420,57 @@ def run_gemm(args):
             "kernels": res}
 
 
+def run_digests(args):
+    """The numerical-health digests the reference's example takes every cycle: nan_count and
+    abs_log2_hist8 of each of the 237 parameters and 237 gradients (2 x 6.85 GB of f16), after one
+    step; value = bytes digested per second, the CPU port timed on the embedding alone."""
+    import torch
+    from cacti_amd.runtime import Ctx, Llama
+    cfg = dict(LLAMA_3B)
+    if args.layers is not None:
+        cfg["L"] = args.layers
+    ctx = Ctx(0, 0, True)
+    model = Llama(ctx, **cfg)
+    synth_params(model)
+    tok, lm_tok, scale = synth_inputs(cfg)
+    model.step(tok, lm_tok, scale, want_loss=False)
+    for g in (True, False):
+        model.digests(of_grads=g)
+    ctx.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        gh, gn = model.digests(of_grads=True)
+        ph, pn = model.digests(of_grads=False)
+    dt = (time.perf_counter() - t0) / args.steps
+    nbytes = 2 * 2 * int(ph.sum())                       # every element is counted once per histogram
+    assert int(gh.sum()) == int(ph.sum()) and int(gn.sum()) == 0 and int(pn.sum()) == 0
+    out = {"metric": "numerical-health digests (nan_count + abs_log2_hist8) of all parameters and gradients",
+           "value": nbytes / dt / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": 1,
+           "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "u16", "data": "synthetic (the benchmark step's parameters and gradients)",
+           "config": {"workload": "2 x %d f16 tensors, %.2f GB each set, both digests of a set in one launch"
+                                  % (len(model.params), int(ph.sum()) * 2 / 1e9)},
+           "roofline": {"bound": "hbm", "achieved": nbytes / dt / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": nbytes / dt / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "note": "every tensor is read once; wall time of the two model-level calls "
+                                "including their stream synchronisations and result copies"}}
+    model.close()
+    ctx.close()
+    if not args.no_cpu_baseline:
+        from oracle import oracle as o
+        x = (np.random.default_rng(0).standard_normal((cfg["V"], cfg["D"])) * 0.02).astype(np.float16)
+        t0 = time.time()
+        o.abs_log2_hist8(x)
+        o.nan_count(x)
+        t = time.time() - t0
+        out["cpu_baseline"] = {"value": x.nbytes / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "oracle digests of one [32000, 3200] f16 tensor (%.2f s)" % t}
+    else:
+        out["cpu_baseline"] = None
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -428,7 +480,7 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -438,6 +490,8 @@ def main():
         out = run_step(args)
     elif args.workload == "adjoints":
         out = run_adjoints(args)
+    elif args.workload == "digests":
+        out = run_digests(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)

@@ -130,7 +130,6 @@ struct LoadKC {
         }
     }
     static constexpr int NREG = NL;
-    static constexpr int NVMEM = NL * (AL == 8 ? 1 : 2);          // load instructions per tile
     static constexpr int NDMA = 0;
     __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
@@ -175,7 +174,6 @@ struct LoadKCD {
     __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
     __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
     static constexpr int NREG = 1;
-    static constexpr int NVMEM = 0;
     static constexpr int NDMA = NL;
 };
 
@@ -221,7 +219,6 @@ struct LoadKSD {
     __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
     __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
     static constexpr int NREG = 1;
-    static constexpr int NVMEM = 0;
     static constexpr int NDMA = NL;
 };
 
@@ -314,7 +311,6 @@ struct LoadKS {
         }
     }
     static constexpr int NREG = NL * 8;
-    static constexpr int NVMEM = 0;                               // depends on the wave: not counted
     static constexpr int NDMA = 0;
     __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
@@ -390,7 +386,6 @@ struct LoadKS2 {
         }
     }
     static constexpr int NREG = 8;
-    static constexpr int NVMEM = 8 * (AL == 8 ? 1 : 2);
     static constexpr int NDMA = 0;
     __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
@@ -461,7 +456,6 @@ struct LoadKSH {
         }
     }
     static constexpr int NREG = KPI;
-    static constexpr int NVMEM = KPI * (AL == 8 ? 1 : 2);
     static constexpr int NDMA = 0;
     __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
 };
@@ -473,7 +467,6 @@ struct LoadNone {
     __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
     __device__ __forceinline__ void dma(uint32_t, const half_t *, int64_t) const {}
     static constexpr int NREG = 1;
-    static constexpr int NVMEM = 0;
     static constexpr int NDMA = 0;
 };
 

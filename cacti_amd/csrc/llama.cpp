@@ -294,6 +294,13 @@ CACTI_API int cacti_llama_grad_get(cacti_llama *m, int i, void *host, size_t byt
     return m->ctx->c.cell_get(m->grads[i], host, bytes);
 }
 
+CACTI_API int cacti_llama_digests(cacti_llama *m, int of_grads, int64_t *hist, int64_t *nan)
+{
+    CACTI_REQUIRE(m && hist && nan, CACTI_E_INVALID, "digests: null argument");
+    const std::vector<CellPtr> &cells = of_grads ? m->grads : m->params;
+    return m->ctx->c.cells_digest(cells.data(), (int)cells.size(), hist, nan);
+}
+
 CACTI_API int cacti_llama_io_cells(cacti_llama *m, int *tok, int *lm_tok, int *loss_scale,
                                    int *logit, int *loss, int *amax, int *prob)
 {

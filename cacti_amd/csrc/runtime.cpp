@@ -247,6 +247,70 @@ int Ctx::cell_get(CellPtr ci, void *host, size_t bytes)
     return 0;
 }
 
+// csrc/digest.hip
+size_t digest_batch_scratch_bytes(int count);
+int digest_batch_f16(int count, const void *const *xs, const int64_t *ns, void *out, void *segs_dev,
+                     hipStream_t st);
+
+// One launch digests every cell: all of them are made resident first (a cell that cannot be
+// held beside the others fails the call with the pool's error).
+int Ctx::cells_digest(const CellPtr *cells, int n, int64_t *hist, int64_t *nan)
+{
+    CACTI_REQUIRE(n >= 0 && (n == 0 || (cells && hist && nan)), CACTI_E_INVALID, "cells_digest: null argument");
+    if (n == 0) return 0;
+    // device scratch: per cell 256 histogram bins + the NaN count, then the launch's descriptors
+    const size_t out_bytes = (size_t)n * 257 * sizeof(int64_t);
+    size_t off;
+    int rc = pool_alloc(out_bytes + digest_batch_scratch_bytes(n), &off);
+    if (rc) return rc;
+    char *scratch = static_cast<char *>(dev_ptr(off));
+    std::vector<const void *> xs((size_t)n);
+    std::vector<int64_t> ns((size_t)n);
+    std::vector<int64_t> host((size_t)n * 257);
+    int done = 0;
+    while (done < n && rc == 0) {
+        // as many cells as stay resident together
+        int m = 0;
+        for (int i = done; i < n; i++) {
+            const CellPtr ci = cells[i];
+            if (ci <= 0 || (size_t)ci >= cells_.size() || !cells_[ci].alive || cells_[ci].ty.dtype != F16) {
+                set_error("cells_digest: cell %d is not a live f16 cell", ci);
+                rc = CACTI_E_INVALID;
+                break;
+            }
+            cells_[ci].pin++;
+            rc = ensure_vmem(ci, true);
+            if (rc) {
+                cells_[ci].pin--;
+                if (m > 0 && rc == CACTI_E_OOM) rc = 0;   // digest what fits, then go on
+                break;
+            }
+            xs[(size_t)m] = dev_ptr(cells_[ci].voff);
+            ns[(size_t)m] = (int64_t)(cells_[ci].ty.bytes() / 2);
+            m++;
+        }
+        if (rc == 0 && m > 0)
+            rc = digest_batch_f16(m, xs.data(), ns.data(), scratch + (size_t)done * 257 * sizeof(int64_t),
+                                  scratch + out_bytes, stream_);
+        for (int i = done; i < done + m; i++) cells_[cells[i]].pin--;
+        if (rc == 0 && m == 0) rc = CACTI_E_OOM;
+        done += m;
+    }
+    if (rc == 0) {
+        rc = hip_status(hipMemcpyAsync(host.data(), scratch, out_bytes, hipMemcpyDeviceToHost, stream_), "digest d2h");
+        bytes_d2h_ += out_bytes;
+    }
+    const int rs = hip_status(hipStreamSynchronize(stream_), "digest sync");
+    pool_.free(off);
+    if (rc) return rc;
+    if (rs) return rs;
+    for (int i = 0; i < n; i++) {
+        memcpy(hist + (size_t)i * 256, host.data() + (size_t)i * 257, 256 * sizeof(int64_t));
+        nan[i] = host[(size_t)i * 257 + 256];
+    }
+    return 0;
+}
+
 // VMem -> Mem: keep (or make) a host copy of the current version, then drop the device
 // replica.  PCell::read_loc(.., Locus::Mem) + yeet, src/pctx/nvgpu.rs:2198-2251.
 int Ctx::evict(CellPtr ci)

@@ -134,6 +134,9 @@ class Ctx {
     void set_const(CellPtr c) { cells_[c].konst = true; }
     int cell_put(CellPtr c, const void *host, size_t bytes);     // host -> cell (Mem, then VMem)
     int cell_get(CellPtr c, void *host, size_t bytes);           // cell -> host (syncs)
+    // NaN count and abs-log2 histogram (int64 [256]) of n f16 cells, one stream sync for all;
+    // x.nan_count(), x.abs_log2_hist8() of the reference's example (open_llama_3b_train.rs:409-424)
+    int cells_digest(const CellPtr *cells, int n, int64_t *hist, int64_t *nan);
     int cell_free_all(CellPtr c);
     void *dev_ptr(size_t off) { return base_ + off; }
     // make the VMem replica exist (evicting others if needed) and, if `need_value`, hold

@@ -67,6 +67,10 @@ SIGNATURES = {
     "cacti_hip_embed_bwd": (ci, [i64, i64, i64, vp, vp, vp, ci, vp]),
     "cacti_hip_add_f16": (ci, [i64, vp, vp, vp, vp]),
     "cacti_hip_selftest_wave_reduce": (ci, [vp, vp]),
+    "cacti_hip_nan_count_f16": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_abs_log2_hist8_f16": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_digests_scratch_bytes": (sz, [ci]),
+    "cacti_hip_digests_f16_batch": (ci, [ci, vp, vp, vp, vp, vp]),
     # ---- runtime (include/cacti_hip_runtime.h)
     "cacti_ctx_create": (ci, [pvp, ci, sz, ci]),
     "cacti_ctx_destroy": (ci, [vp]),
@@ -96,6 +100,7 @@ SIGNATURES = {
                                     C.POINTER(ci), C.POINTER(ci)]),
     "cacti_llama_param_put": (ci, [vp, ci, vp, sz]),
     "cacti_llama_grad_get": (ci, [vp, ci, vp, sz]),
+    "cacti_llama_digests": (ci, [vp, ci, vp, vp]),
     "cacti_llama_io_cells": (ci, [vp] + [C.POINTER(ci)] * 7),
     "cacti_llama_stage": (ci, [vp, ci, ci]),
     "cacti_llama_step": (ci, [vp, vp, vp, vp, ci, ci, vp]),

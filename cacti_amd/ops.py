@@ -233,3 +233,39 @@ def accumulate_1d(dst, src):
     ffi.call("cacti_hip_accumulate_1d_" + name, dst.data_ptr(), src.data_ptr(), dst.numel(),
              _stream())
     return dst
+
+
+# ---------------------------------------------------------------- numerical-health digests
+def nan_count(x):
+    """Number of NaNs of an f16 tensor as a 0-d int64 device tensor (src/thunk/op.rs:273-349)."""
+    _chk(x)
+    out = torch.empty((), dtype=torch.int64, device=x.device)
+    ffi.call("cacti_hip_nan_count_f16", x.numel(), x.data_ptr(), out.data_ptr(), _stream())
+    return out
+
+
+def abs_log2_hist8(x):
+    """int64[256] histogram of the floor(log2 |x|) classes of an f16 tensor (src/thunk/op.rs:351-441)."""
+    _chk(x)
+    out = torch.empty(256, dtype=torch.int64, device=x.device)
+    ffi.call("cacti_hip_abs_log2_hist8_f16", x.numel(), x.data_ptr(), out.data_ptr(), _stream())
+    return out
+
+
+def digests(xs):
+    """Both digests of a list of f16 tensors in one launch: (hist int64[n,256], nan int64[n])
+    (the per-cycle loop of examples/open_llama_3b_train.rs:409-424)."""
+    import ctypes as C
+    n = len(xs)
+    for x in xs:
+        _chk(x)
+    dev = xs[0].device if n else torch.device("cuda")
+    out = torch.empty((n, 257), dtype=torch.int64, device=dev)
+    if n == 0:
+        return out[:, :256], out[:, 256]
+    scratch = torch.empty(ffi.lib().cacti_hip_digests_scratch_bytes(n), dtype=torch.uint8, device=dev)
+    ptrs = (C.c_void_p * n)(*[x.data_ptr() for x in xs])
+    ns = (C.c_int64 * n)(*[x.numel() for x in xs])
+    ffi.call("cacti_hip_digests_f16_batch", n, C.cast(ptrs, C.c_void_p), C.cast(ns, C.c_void_p),
+             out.data_ptr(), scratch.data_ptr(), _stream())
+    return out[:, :256], out[:, 256]

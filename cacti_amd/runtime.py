@@ -153,6 +153,15 @@ class Llama:
     def grads(self):
         return {name: self.grad(i) for i, (name, _) in enumerate(self.params)}
 
+    def digests(self, of_grads=False):
+        """(hist int64 [num_params, 256], nan int64 [num_params]) of every parameter or gradient:
+        abs_log2_hist8 and nan_count as the reference's example takes them each cycle
+        (examples/open_llama_3b_train.rs:409-424)."""
+        n = len(self.params)
+        hist, nan = np.zeros((n, 256), np.int64), np.zeros(n, np.int64)
+        ffi.call("cacti_llama_digests", self._m, int(of_grads), hist.ctypes.data, nan.ctypes.data)
+        return hist, nan
+
     def io_cells(self):
         v = [C.c_int(0) for _ in range(7)]
         ffi.call("cacti_llama_io_cells", self._m, *[C.byref(x) for x in v])

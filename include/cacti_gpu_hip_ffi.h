@@ -233,6 +233,30 @@ int cacti_hip_add_f16(int64_t n, const void *a, const void *b, void *y, void *st
  * LDS path).  Returns the kernel launch status only; the caller compares. */
 int cacti_hip_selftest_wave_reduce(void *out4, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Numerical-health digests of an f16 tensor of n elements (any shape, contiguous), integer-exact.
+ * The reference's training example takes both of every parameter and gradient each cycle
+ * (examples/open_llama_3b_train.rs:409-424).
+ *
+ * nan_count: *count_i64 = number of NaNs (exponent field all ones, mantissa not zero);
+ * NanCountFutThunkSpec, src/thunk/op.rs:273-349 (output: i64 scalar).
+ * abs_log2_hist8: hist_i64_256[b] = number of elements of class b, where b = 255 for inf and nan,
+ * 0 for +-0 and floor(log2 |x|) + 127 otherwise (103..112 subnormal, 113..142 normal);
+ * AbsLog2Hist8FutThunkSpec, src/thunk/op.rs:351-441 (output: i64[256]).
+ * The outputs are device memory, overwritten; x must be 16-byte aligned. */
+int cacti_hip_nan_count_f16(int64_t n, const void *x, void *count_i64, void *stream);
+int cacti_hip_abs_log2_hist8_f16(int64_t n, const void *x, void *hist_i64_256, void *stream);
+
+/* Both digests of `count` tensors in one launch and one read of each tensor (the example's loop
+ * over all parameters and gradients, examples/open_llama_3b_train.rs:409-424, as one call):
+ * out_i64[257 * i + b] = abs_log2_hist8 class b of tensor i, out_i64[257 * i + 256] = its NaN
+ * count.  xs[i] (device, 16-byte aligned) holds ns[i] >= 0 f16 elements; xs and ns are host
+ * arrays read before the call returns.  out_i64 (count * 257 values) and scratch
+ * (cacti_hip_digests_scratch_bytes(count) bytes) are device memory, 8-byte aligned. */
+size_t cacti_hip_digests_scratch_bytes(int count);
+int cacti_hip_digests_f16_batch(int count, const void *const *xs, const int64_t *ns, void *out_i64,
+                                void *scratch, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -100,6 +100,12 @@ int cacti_llama_param_info(cacti_llama *model, int i, char *name, size_t name_ca
                            int64_t *rows, int64_t *cols, int *param_cell, int *grad_cell);
 int cacti_llama_param_put(cacti_llama *model, int i, const void *host, size_t bytes);
 int cacti_llama_grad_get(cacti_llama *model, int i, void *host, size_t bytes);
+/* Numerical-health digests of every parameter (of_grads = 0) or gradient (1), in parameter
+ * order: hist [num_params][256] and nan [num_params], int64, host memory.  What the reference's
+ * example computes each cycle with p.abs_log2_hist8(), p.nan_count(), g.abs_log2_hist8(),
+ * g.nan_count() (examples/open_llama_3b_train.rs:409-424, read at :587-650); bins as in
+ * cacti_hip_abs_log2_hist8_f16.  One stream synchronisation for the whole call. */
+int cacti_llama_digests(cacti_llama *model, int of_grads, int64_t *hist, int64_t *nan);
 /* cells of the inputs (tok u16 [S], lm_tok u16 [S], loss_scale f32 [S]) and of the kept
  * outputs of the last staged cycle (logit f16 [S,V], loss f32 [S], amax u16 [S],
  * prob f32 [S,V] or 0) */

@@ -976,6 +976,52 @@ ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const ui
     return 0;
 }
 
+/* ---------------------------------------------------------------------------
+ * Numerical-health digests over f16 tensors (integer-exact).
+ * NanCountFutThunkSpec, src/thunk/op.rs:273-349: elements whose exponent field is all ones and
+ * whose mantissa is not zero.
+ * AbsLog2Hist8FutThunkSpec, src/thunk/op.rs:351-441: histogram over 256 bins of
+ * bin = u8(i8(v) + 0x7f), v = -0x80 for inf / nan, -0x7f for +-0, floor(log2 |x|) otherwise
+ * (exponent field - 15 for normal numbers, -24 + u16_nz_log2(mantissa) for subnormal ones);
+ * u16_nz_log2 is the reference's multiply-and-look-up form in 16-bit arithmetic (:398-405). */
+static int th_u16_nz_log2(uint16_t x)
+{
+    static const int8_t v_tab[16] = {0, 7, 1, 13, 8, 10, 2, 14, 6, 12, 9, 5, 11, 4, 3, 15};
+    const uint16_t c = 0xf2d;
+    x |= (uint16_t)(x >> 1);
+    x |= (uint16_t)(x >> 2);
+    x |= (uint16_t)(x >> 4);
+    x |= (uint16_t)(x >> 8);
+    return v_tab[(uint16_t)(c * x) >> 12];
+}
+
+ORACLE_API int oracle_abs_log2_bin(uint16_t u)
+{
+    const uint16_t b = (u >> 10) & 0x1f, m = u & 0x3ff;
+    const int8_t e = (int8_t)((int8_t)b - 0xf);
+    int8_t v;
+    if (b == 0x1f) v = -0x80;
+    else if (b == 0) v = m == 0 ? -0x7f : (int8_t)(-14 - 10 + th_u16_nz_log2(m));
+    else v = e;
+    return (uint8_t)(int8_t)(v + 0x7f);
+}
+
+ORACLE_API i64 oracle_nan_count_f16(i64 n, const h16 *x)
+{
+    i64 cnt = 0;
+    for (i64 i = 0; i < n; i++) {
+        const uint16_t u = x[i], b = (u >> 10) & 0x1f, m = u & 0x3ff;
+        cnt += (b == 0x1f && m != 0) ? 1 : 0;
+    }
+    return cnt;
+}
+
+ORACLE_API void oracle_abs_log2_hist8_f16(i64 n, const h16 *x, i64 *hist /* [256] */)
+{
+    for (int i = 0; i < 256; i++) hist[i] = 0;
+    for (i64 i = 0; i < n; i++) hist[oracle_abs_log2_bin(x[i])] += 1;
+}
+
 ORACLE_API int oracle_num_threads(void)
 {
 #ifdef _OPENMP

@@ -56,6 +56,9 @@ def lib():
         _LIB.th_softmax_nll_f32.restype = i64
         _LIB.th_outer_select_f16.restype = i64
         _LIB.oracle_layer_elems.restype = i64
+        _LIB.oracle_nan_count_f16.restype = i64
+        _LIB.oracle_abs_log2_bin.restype = C.c_int
+        _LIB.oracle_abs_log2_bin.argtypes = [C.c_uint16]
         _LIB.oracle_param_elems.restype = i64
         _LIB.oracle_num_threads.restype = C.c_int
     return _LIB
@@ -285,3 +288,23 @@ def llama_step(cfg, param, tok, lm_tok, loss_scale, want_grad=True):
     if rc:
         raise IndexError("oracle_llama_step failed rc=%d" % rc)
     return dict(loss=loss, logit=logit, amax=amax, grad=grad)
+
+
+# ---------------------------------------------------------------- numerical-health digests
+def nan_count(x):
+    """Number of NaNs in an f16 tensor (src/thunk/op.rs:273-349)."""
+    x = np.ascontiguousarray(x)
+    return int(lib().oracle_nan_count_f16(i64(x.size), P(x)))
+
+
+def abs_log2_hist8(x):
+    """int64[256] histogram of floor(log2 |x|) classes of an f16 tensor (src/thunk/op.rs:351-441)."""
+    x = np.ascontiguousarray(x)
+    h = np.zeros(256, np.int64)
+    lib().oracle_abs_log2_hist8_f16(i64(x.size), P(x), P(h))
+    return h
+
+
+def abs_log2_bin(bits):
+    """Histogram bin of one f16 bit pattern."""
+    return int(lib().oracle_abs_log2_bin(int(bits)))

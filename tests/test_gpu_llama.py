@@ -138,6 +138,33 @@ def test_capped_pool_spills_and_matches(oracle, pagelocked):
     m.close(); ctx.close()
 
 
+@pytest.mark.parametrize("capped", [False, True])
+def test_digests_of_parameters_and_gradients(oracle, capped):
+    """abs_log2_hist8 and nan_count of every parameter and gradient after a cycle, as the
+    reference's example takes them (examples/open_llama_3b_train.rs:409-424): bit-exact against
+    the oracle's digests of the same tensors; also with cells spilled to the host in between."""
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=4, norm_mean=1.0, grad_scale=1024.0)
+    ctx, m = _model(cfg)
+    m.put_params_flat(flat)
+    m.step(tok, lm_tok, scale)
+    if capped:
+        peak = ctx.stats()["pool_peak"]
+        m.close(); ctx.close()
+        ctx, m = _model(cfg, pool_bytes=int(peak * 0.45))
+        m.put_params_flat(flat)
+        m.step(tok, lm_tok, scale)
+    grads = m.grads()
+    gh, gn = m.digests(of_grads=True)
+    ph, pn = m.digests(of_grads=False)
+    want_p = oracle.split_params(cfg, flat)
+    for i, (name, shape) in enumerate(m.params):
+        assert np.array_equal(gh[i], oracle.abs_log2_hist8(grads[name])), name
+        assert gn[i] == oracle.nan_count(grads[name]) == 0, name
+        assert np.array_equal(ph[i], oracle.abs_log2_hist8(want_p[name])), name
+        assert pn[i] == 0 and ph[i].sum() == int(np.prod(shape)), name
+    m.close(); ctx.close()
+
+
 def test_pool_too_small_is_a_clean_error(oracle):
     from cacti_amd.ffi import CactiError
     cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=3)
