@@ -471,6 +471,70 @@ def run_digests(args):
     return out
 
 
+def run_adamw(args):
+    """One AdamW32 step of every parameter of the 3B model (the minibatch boundary of the reference's
+    example, examples/open_llama_3b_train.rs:252-268, which it runs on the CPU): moment averages,
+    master-weight update and the cast back to f16, one launch.  value = parameters updated per second;
+    algorithmic bytes = 28 per parameter (read f16 grad + 3 f32 states, write 3 f32 states + f16 param)."""
+    import torch
+    from cacti_amd.runtime import Ctx, Llama
+    cfg = dict(LLAMA_3B)
+    if args.layers is not None:
+        cfg["L"] = args.layers
+    opt = dict(grad_scale=1024.0, lr=2.0e-5, wd=0.1, a1=0.1, a2=0.05, eps=1.0e-5)   # the example's AdamW32
+    ctx = Ctx(0, 0, True)
+    model = Llama(ctx, **cfg)
+    synth_params(model)
+    tok, lm_tok, scale = synth_inputs(cfg)
+    model.step(tok, lm_tok, scale, want_loss=False)
+    model.adamw_init()
+    nparam = sum(int(np.prod(shp)) for _, shp in model.params)
+    for it in range(1, args.warmup + 1):
+        model.adamw_step(it, **opt)
+    ctx.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for it in range(args.warmup + 1, args.warmup + args.steps + 1):
+        model.adamw_step(it, **opt)
+    ctx.sync()
+    dt = (time.perf_counter() - t0) / args.steps
+    # property that holds at any size: the parameters are the f16 rounding of the master weights
+    for i in (1, len(model.params) - 1):
+        assert np.array_equal(model.param(i).view(np.uint16),
+                              model.adamw_state(i, "master").astype(np.float16).view(np.uint16))
+    out = {"metric": "AdamW32 step (moment averages, master update, cast to f16) over all parameters",
+           "value": nparam / dt, "unit": "parameters/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32", "data": "synthetic (the benchmark step's parameters and gradients)",
+           "config": {"workload": "%d tensors, %.3f G parameters, one launch per step" % (len(model.params), nparam / 1e9)},
+           "roofline": {"bound": "hbm", "achieved": 28.0 * nparam / dt / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": 28.0 * nparam / dt / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "note": "28 bytes per parameter; wall time of the calls, synchronised once at the end"}}
+    model.close()
+    ctx.close()
+    if not args.no_cpu_baseline:
+        from oracle import oracle as o
+        r = np.random.default_rng(0)
+        n = cfg["V"] * cfg["D"]
+        g = (r.standard_normal(n, dtype=np.float32) * 0.3).astype(np.float16)
+        a = np.zeros(n, np.float32); b = np.zeros(n, np.float32)
+        w = r.standard_normal(n, dtype=np.float32) * 0.02
+        sc = o.adamw32_scalars(2, **opt)
+        p16 = np.empty(n, np.float16)
+        o.lib().oracle_adamw32_step(o.i64(n), o.P(g), o.P(a), o.P(b), o.P(w), o.P(p16), o.P(sc))   # touch the pages
+        t0 = time.time()
+        reps = 3
+        for _ in range(reps):
+            o.lib().oracle_adamw32_step(o.i64(n), o.P(g), o.P(a), o.P(b), o.P(w), o.P(p16), o.P(sc))
+        t = (time.time() - t0) / reps
+        out["cpu_baseline"] = {"value": n / t, "unit": "parameters/s", "cores": o.num_threads(), "kind": "port",
+                               "sample": "oracle AdamW32 step (four thunks) of one [32000, 3200] tensor, in place, "
+                                         "%d repetitions of %.2f s" % (reps, t)}
+    else:
+        out["cpu_baseline"] = None
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -480,7 +544,7 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -492,6 +556,8 @@ def main():
         out = run_adjoints(args)
     elif args.workload == "digests":
         out = run_digests(args)
+    elif args.workload == "adamw":
+        out = run_adamw(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)

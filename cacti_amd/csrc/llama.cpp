@@ -24,6 +24,7 @@ struct cacti_llama {
     cacti_ctx *ctx;
     cacti_llama_cfg cfg;
     std::vector<CellPtr> params, grads;
+    std::vector<CellPtr> master, grad_avg, grad2_avg;           // f32 optimiser state (adamw_init)
     std::vector<std::string> names;
     CellPtr embed, head_norm, lm_head;
     std::vector<LayerCells> layers;
@@ -299,6 +300,52 @@ CACTI_API int cacti_llama_digests(cacti_llama *m, int of_grads, int64_t *hist, i
     CACTI_REQUIRE(m && hist && nan, CACTI_E_INVALID, "digests: null argument");
     const std::vector<CellPtr> &cells = of_grads ? m->grads : m->params;
     return m->ctx->c.cells_digest(cells.data(), (int)cells.size(), hist, nan);
+}
+
+CACTI_API int cacti_llama_adamw_init(cacti_llama *m)
+{
+    CACTI_REQUIRE(m, CACTI_E_INVALID, "adamw_init: null model");
+    Ctx &c = m->ctx->c;
+    if (m->master.empty()) {
+        for (size_t i = 0; i < m->params.size(); i++) {
+            const CellType ty(c.cell(m->params[i]).ty.shape, F32);
+            m->master.push_back(c.cell_new(ty, true, ("master:" + m->names[i]).c_str()));
+            m->grad_avg.push_back(c.cell_new(ty, true, ("grad_avg:" + m->names[i]).c_str()));
+            m->grad2_avg.push_back(c.cell_new(ty, true, ("grad2_avg:" + m->names[i]).c_str()));
+        }
+        for (CellPtr x : m->master) c.set_const(x);
+        for (CellPtr x : m->grad_avg) c.set_const(x);
+        for (CellPtr x : m->grad2_avg) c.set_const(x);
+    }
+    for (size_t i = 0; i < m->params.size(); i++) {
+        int rc = c.cell_cast_f16_f32(m->params[i], m->master[i]);
+        if (!rc) rc = c.cell_zero(m->grad_avg[i]);
+        if (!rc) rc = c.cell_zero(m->grad2_avg[i]);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+CACTI_API int cacti_llama_adamw_step(cacti_llama *m, int iter_nr, const cacti_adamw32 *opt, int skip_embed)
+{
+    CACTI_REQUIRE(m && opt, CACTI_E_INVALID, "adamw_step: null argument");
+    CACTI_REQUIRE(!m->master.empty(), CACTI_E_STATE, "adamw_step before adamw_init");
+    float sc[7];
+    int rc = cacti_adamw32_scalars(iter_nr, opt->grad_scale, opt->lr, opt->wd, opt->a1, opt->a2, opt->eps, sc);
+    if (rc) return rc;
+    const size_t first = skip_embed ? 1 : 0;                     // the embedding is parameter 0
+    return m->ctx->c.cells_adamw32((int)(m->params.size() - first), m->grads.data() + first,
+                                   m->grad_avg.data() + first, m->grad2_avg.data() + first,
+                                   m->master.data() + first, m->params.data() + first, sc);
+}
+
+CACTI_API int cacti_llama_adamw_state_get(cacti_llama *m, int i, int which, void *host, size_t bytes)
+{
+    CACTI_REQUIRE(m && i >= 0 && (size_t)i < m->params.size() && which >= 0 && which <= 2, CACTI_E_INVALID,
+                  "adamw_state_get: index out of range");
+    CACTI_REQUIRE(!m->master.empty(), CACTI_E_STATE, "adamw_state_get before adamw_init");
+    const std::vector<CellPtr> &v = which == 0 ? m->master : which == 1 ? m->grad_avg : m->grad2_avg;
+    return m->ctx->c.cell_get(v[(size_t)i], host, bytes);
 }
 
 CACTI_API int cacti_llama_io_cells(cacti_llama *m, int *tok, int *lm_tok, int *loss_scale,

@@ -311,6 +311,108 @@ int Ctx::cells_digest(const CellPtr *cells, int n, int64_t *hist, int64_t *nan)
     return 0;
 }
 
+int Ctx::cell_cast_f16_f32(CellPtr src, CellPtr dst)
+{
+    CACTI_REQUIRE(src > 0 && dst > 0 && (size_t)src < cells_.size() && (size_t)dst < cells_.size() &&
+                      cells_[src].alive && cells_[dst].alive && cells_[src].ty.dtype == F16 &&
+                      cells_[dst].ty.dtype == F32 && cells_[src].ty.bytes() * 2 == cells_[dst].ty.bytes(),
+                  CACTI_E_INVALID, "cell_cast: wants a live f16 source and an f32 destination of the same shape");
+    cells_[src].pin++;
+    cells_[dst].pin++;
+    int rc = ensure_vmem(src, true);
+    if (!rc) rc = ensure_vmem(dst, false);
+    if (!rc)
+        rc = cacti_hip_cast_f16_f32((int64_t)(cells_[src].ty.bytes() / 2), dev_ptr(cells_[src].voff),
+                                    dev_ptr(cells_[dst].voff), stream_);
+    cells_[src].pin--;
+    cells_[dst].pin--;
+    if (!rc) {
+        cells_[dst].v_valid = true;
+        cells_[dst].h_valid = false;
+    }
+    return rc;
+}
+
+int Ctx::cell_zero(CellPtr c)
+{
+    CACTI_REQUIRE(c > 0 && (size_t)c < cells_.size() && cells_[c].alive, CACTI_E_INVALID, "cell_zero: dead cell");
+    int rc = ensure_vmem(c, false);
+    if (rc) return rc;
+    CACTI_HIP(hipMemsetAsync(dev_ptr(cells_[c].voff), 0, cells_[c].ty.bytes(), stream_));
+    cells_[c].v_valid = true;
+    cells_[c].h_valid = false;
+    return 0;
+}
+
+// The five cells of a tensor must be resident together; with a capped pool the list is cut into
+// as many launches as needed.
+int Ctx::cells_adamw32(int n, const CellPtr *grads, const CellPtr *avgs, const CellPtr *avg2s,
+                       const CellPtr *masters, const CellPtr *params, const float *sc)
+{
+    CACTI_REQUIRE(n >= 0 && (n == 0 || (grads && avgs && avg2s && masters && params && sc)), CACTI_E_INVALID,
+                  "cells_adamw32: null argument");
+    if (n == 0) return 0;
+    size_t off;
+    int rc = pool_alloc(cacti_hip_adamw32_scratch_bytes(n), &off);
+    if (rc) return rc;
+    std::vector<const void *> g((size_t)n);
+    std::vector<void *> a((size_t)n), b((size_t)n), w((size_t)n), p((size_t)n);
+    std::vector<int64_t> ns((size_t)n);
+    int done = 0;
+    while (done < n && rc == 0) {
+        int m = 0;
+        for (int i = done; i < n; i++) {
+            const CellPtr five[5] = {grads[i], avgs[i], avg2s[i], masters[i], params[i]};
+            size_t elems = 0;
+            for (int k = 0; k < 5 && rc == 0; k++) {
+                const CellPtr ci = five[k];
+                const bool ok = ci > 0 && (size_t)ci < cells_.size() && cells_[ci].alive &&
+                                cells_[ci].ty.dtype == ((k == 0 || k == 4) ? F16 : F32);
+                const size_t e = ok ? cells_[ci].ty.bytes() / ((k == 0 || k == 4) ? 2 : 4) : 0;
+                if (!ok || (k > 0 && e != elems)) {
+                    set_error("cells_adamw32: tensor %d: cell %d has the wrong type, size or is dead", i, ci);
+                    rc = CACTI_E_INVALID;
+                }
+                elems = e;
+            }
+            if (rc) break;
+            int pinned = 0;
+            for (; pinned < 5 && rc == 0; pinned++) {
+                cells_[five[pinned]].pin++;
+                rc = ensure_vmem(five[pinned], pinned != 4);      // the parameter is only written
+            }
+            if (rc) {
+                for (int k = 0; k < pinned; k++) cells_[five[k]].pin--;
+                if (m > 0 && rc == CACTI_E_OOM) rc = 0;          // update what fits, then go on
+                break;
+            }
+            g[(size_t)m] = dev_ptr(cells_[five[0]].voff);
+            a[(size_t)m] = dev_ptr(cells_[five[1]].voff);
+            b[(size_t)m] = dev_ptr(cells_[five[2]].voff);
+            w[(size_t)m] = dev_ptr(cells_[five[3]].voff);
+            p[(size_t)m] = dev_ptr(cells_[five[4]].voff);
+            ns[(size_t)m] = (int64_t)elems;
+            m++;
+        }
+        if (rc == 0 && m > 0)
+            rc = cacti_hip_adamw32_step_f16_batch(m, g.data(), a.data(), b.data(), w.data(), p.data(), ns.data(), sc,
+                                                  dev_ptr(off), stream_);
+        for (int i = done; i < done + m; i++) {
+            const CellPtr five[5] = {grads[i], avgs[i], avg2s[i], masters[i], params[i]};
+            for (int k = 0; k < 5; k++) cells_[five[k]].pin--;
+            if (rc == 0)
+                for (int k = 1; k < 5; k++) {
+                    cells_[five[k]].v_valid = true;
+                    cells_[five[k]].h_valid = false;
+                }
+        }
+        if (rc == 0 && m == 0) rc = CACTI_E_OOM;
+        done += m;
+    }
+    pool_.free(off);                                             // reuse is ordered on the stream
+    return rc;
+}
+
 // VMem -> Mem: keep (or make) a host copy of the current version, then drop the device
 // replica.  PCell::read_loc(.., Locus::Mem) + yeet, src/pctx/nvgpu.rs:2198-2251.
 int Ctx::evict(CellPtr ci)

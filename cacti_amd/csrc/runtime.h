@@ -137,6 +137,13 @@ class Ctx {
     // NaN count and abs-log2 histogram (int64 [256]) of n f16 cells, one stream sync for all;
     // x.nan_count(), x.abs_log2_hist8() of the reference's example (open_llama_3b_train.rs:409-424)
     int cells_digest(const CellPtr *cells, int n, int64_t *hist, int64_t *nan);
+    // one AdamW32 step of n tensors in one launch: grads f16 (read), avgs / avg2s / masters f32
+    // (updated), params f16 (written); sc = the seven scalars of cacti_adamw32_scalars.  Returns
+    // without synchronising.
+    int cells_adamw32(int n, const CellPtr *grads, const CellPtr *avgs, const CellPtr *avg2s,
+                      const CellPtr *masters, const CellPtr *params, const float *sc);
+    int cell_cast_f16_f32(CellPtr src, CellPtr dst);              // set_cast, src/op.rs:1085-1096
+    int cell_zero(CellPtr c);                                    // set_zeros, src/op.rs:1137-1146
     int cell_free_all(CellPtr c);
     void *dev_ptr(size_t off) { return base_ + off; }
     // make the VMem replica exist (evicting others if needed) and, if `need_value`, hold

@@ -71,6 +71,14 @@ SIGNATURES = {
     "cacti_hip_abs_log2_hist8_f16": (ci, [i64, vp, vp, vp]),
     "cacti_hip_digests_scratch_bytes": (sz, [ci]),
     "cacti_hip_digests_f16_batch": (ci, [ci, vp, vp, vp, vp, vp]),
+    "cacti_hip_online_average_scale_f16_f32": (ci, [i64, vp, vp, f32, f32, vp]),
+    "cacti_hip_online_average_square_scale_f16_f32": (ci, [i64, vp, vp, f32, f32, vp]),
+    "cacti_hip_online_adamw_update_f32": (ci, [i64, vp, vp, vp, f32, f32, f32, f32, vp]),
+    "cacti_hip_cast_f32_f16": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_cast_f16_f32": (ci, [i64, vp, vp, vp]),
+    "cacti_adamw32_scalars": (ci, [ci, f32, f32, f32, f32, f32, f32, vp]),
+    "cacti_hip_adamw32_scratch_bytes": (sz, [ci]),
+    "cacti_hip_adamw32_step_f16_batch": (ci, [ci, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
     # ---- runtime (include/cacti_hip_runtime.h)
     "cacti_ctx_create": (ci, [pvp, ci, sz, ci]),
     "cacti_ctx_destroy": (ci, [vp]),
@@ -101,10 +109,18 @@ SIGNATURES = {
     "cacti_llama_param_put": (ci, [vp, ci, vp, sz]),
     "cacti_llama_grad_get": (ci, [vp, ci, vp, sz]),
     "cacti_llama_digests": (ci, [vp, ci, vp, vp]),
+    "cacti_llama_adamw_init": (ci, [vp]),
+    "cacti_llama_adamw_step": (ci, [vp, ci, vp, ci]),
+    "cacti_llama_adamw_state_get": (ci, [vp, ci, ci, vp, sz]),
     "cacti_llama_io_cells": (ci, [vp] + [C.POINTER(ci)] * 7),
     "cacti_llama_stage": (ci, [vp, ci, ci]),
     "cacti_llama_step": (ci, [vp, vp, vp, vp, ci, ci, vp]),
 }
+
+
+class AdamW32(C.Structure):
+    """cacti_adamw32 (AdamW32, src/librarium/adamw.rs:4-28)."""
+    _fields_ = [("grad_scale", f32), ("lr", f32), ("wd", f32), ("a1", f32), ("a2", f32), ("eps", f32)]
 
 
 class LlamaCfg(C.Structure):

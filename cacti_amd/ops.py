@@ -269,3 +269,78 @@ def digests(xs):
     ffi.call("cacti_hip_digests_f16_batch", n, C.cast(ptrs, C.c_void_p), C.cast(ns, C.c_void_p),
              out.data_ptr(), scratch.data_ptr(), _stream())
     return out[:, :256], out[:, 256]
+
+
+# ---------------------------------------------------------------- optimiser thunks (AdamW32)
+def _f(x):
+    return _chk(x, torch.float32)
+
+
+def online_average_scale_(u, v, src_scale, rate):
+    """v += rate * (src_scale * f32(u) - v) in place (src/thunk/op.rs:3884-3939)."""
+    _chk(u), _f(v)
+    assert u.numel() == v.numel()
+    ffi.call("cacti_hip_online_average_scale_f16_f32", u.numel(), u.data_ptr(), v.data_ptr(), src_scale, rate,
+             _stream())
+    return v
+
+
+def online_average_square_scale_(u, v, src_scale, rate):
+    """v += rate * ((src_scale * f32(u))^2 - v) in place (src/thunk/op.rs:3941-4002)."""
+    _chk(u), _f(v)
+    assert u.numel() == v.numel()
+    ffi.call("cacti_hip_online_average_square_scale_f16_f32", u.numel(), u.data_ptr(), v.data_ptr(), src_scale,
+             rate, _stream())
+    return v
+
+
+def online_adamw_update_(g1, g2, w, signed_lr, lr_unbias, lamda, eps):
+    """w += signed_lr * (lr_unbias * (g1 / (sqrt(g2) + eps)) + lamda * w) in place
+    (src/thunk/op.rs:4004-4062)."""
+    _f(g1), _f(g2), _f(w)
+    assert g1.numel() == g2.numel() == w.numel()
+    ffi.call("cacti_hip_online_adamw_update_f32", w.numel(), g1.data_ptr(), g2.data_ptr(), w.data_ptr(),
+             signed_lr, lr_unbias, lamda, eps, _stream())
+    return w
+
+
+def cast_f32_f16(x):
+    _f(x)
+    y = torch.empty(x.shape, dtype=torch.float16, device=x.device)
+    ffi.call("cacti_hip_cast_f32_f16", x.numel(), x.data_ptr(), y.data_ptr(), _stream())
+    return y
+
+
+def cast_f16_f32(x):
+    _chk(x)
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    ffi.call("cacti_hip_cast_f16_f32", x.numel(), x.data_ptr(), y.data_ptr(), _stream())
+    return y
+
+
+def adamw32_scalars(iter_nr, grad_scale, lr, wd, a1, a2, eps):
+    """The seven f32 scalars of one AdamW32 step (host arithmetic of src/librarium/adamw.rs:45-60 and
+    src/op.rs:984-1023) as a list; raises for iter_nr <= 0."""
+    import ctypes as C
+    out = (C.c_float * 7)()
+    ffi.call("cacti_adamw32_scalars", int(iter_nr), grad_scale or 0.0, lr, wd, a1, a2, eps, C.cast(out, C.c_void_p))
+    return list(out)
+
+
+def adamw32_step_(grads, avgs, avg2s, masters, params, scalars):
+    """One AdamW32 step of a list of tensors in one launch, in place (avgs, avg2s, masters updated,
+    params overwritten with f16(master))."""
+    import ctypes as C
+    n = len(grads)
+    assert len(avgs) == len(avg2s) == len(masters) == len(params) == n
+    if n == 0:
+        return
+    for g, a, b, w, p in zip(grads, avgs, avg2s, masters, params):
+        _chk(g), _f(a), _f(b), _f(w), _chk(p)
+        assert g.numel() == a.numel() == b.numel() == w.numel() == p.numel()
+    arr = lambda ts: C.cast((C.c_void_p * n)(*[t.data_ptr() for t in ts]), C.c_void_p)
+    ns = (C.c_int64 * n)(*[g.numel() for g in grads])
+    sc = (C.c_float * 7)(*scalars)
+    scratch = torch.empty(ffi.lib().cacti_hip_adamw32_scratch_bytes(n), dtype=torch.uint8, device=grads[0].device)
+    ffi.call("cacti_hip_adamw32_step_f16_batch", n, arr(grads), arr(avgs), arr(avg2s), arr(masters), arr(params),
+             C.cast(ns, C.c_void_p), C.cast(sc, C.c_void_p), scratch.data_ptr(), _stream())

@@ -162,6 +162,29 @@ class Llama:
         ffi.call("cacti_llama_digests", self._m, int(of_grads), hist.ctypes.data, nan.ctypes.data)
         return hist, nan
 
+    def param(self, i):
+        """Current value of parameter i (f16), read back from its cell."""
+        cell = C.c_int(0)
+        ffi.call("cacti_llama_param_info", self._m, i, None, 0, None, None, C.byref(cell), None)
+        return self.ctx.cell_get(cell.value, np.float16, self.params[i][1])
+
+    def adamw_init(self):
+        """master = set_cast(param), grad_avg = grad2_avg = 0 (examples/open_llama_3b_train.rs:230-243)."""
+        ffi.call("cacti_llama_adamw_init", self._m)
+
+    def adamw_step(self, iter_nr, grad_scale=None, lr=1e-3, wd=0.0, a1=0.1, a2=1e-3, eps=1e-8, skip_embed=False):
+        """One AdamW32 step of every parameter from its current gradient, then the cast of the master
+        weights back to f16 (examples/open_llama_3b_train.rs:252-268; defaults: AdamW32::default)."""
+        opt = ffi.AdamW32(grad_scale or 0.0, lr, wd, a1, a2, eps)
+        ffi.call("cacti_llama_adamw_step", self._m, int(iter_nr), C.byref(opt), int(skip_embed))
+
+    def adamw_state(self, i, which):
+        """master / grad_avg / grad2_avg (f32) of parameter i."""
+        out = np.empty(self.params[i][1], np.float32)
+        ffi.call("cacti_llama_adamw_state_get", self._m, i, ("master", "grad_avg", "grad2_avg").index(which),
+                 out.ctypes.data, out.nbytes)
+        return out
+
     def io_cells(self):
         v = [C.c_int(0) for _ in range(7)]
         ffi.call("cacti_llama_io_cells", self._m, *[C.byref(x) for x in v])

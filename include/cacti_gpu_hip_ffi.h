@@ -257,6 +257,49 @@ size_t cacti_hip_digests_scratch_bytes(int count);
 int cacti_hip_digests_f16_batch(int count, const void *const *xs, const int64_t *ns, void *out_i64,
                                 void *scratch, void *stream);
 
+/* ---------------------------------------------------------------------------
+ * Optimiser thunks of AdamW32 (src/librarium/adamw.rs:45-60).  They are Initialize-mode thunks:
+ * the output is read and overwritten in place.  n elements, contiguous, 16-byte aligned; every
+ * f32 operation is rounded on its own, in the order the reference's lambda is written.
+ *
+ * online_average_scale: v += rate * (src_scale * f32(u) - v); OnlineAverageScaleInitFutThunkSpec,
+ *   src/thunk/op.rs:3884-3939 (init_online_average_scale, src/op.rs:950-966).
+ * online_average_square_scale: v += rate * ((src_scale * f32(u)) * (src_scale * f32(u)) - v);
+ *   OnlineAverageSquareScaleInitFutThunkSpec, src/thunk/op.rs:3941-4002.
+ * online_adamw_update: w += signed_lr * (lr_unbias * (u / (sqrt(v) + eps)) + lamda * w);
+ *   OnlineAdamWUpdateInitFutThunkSpec, src/thunk/op.rs:4004-4062.
+ * cast_f32_f16 / cast_f16_f32: CastFutThunkSpec, src/thunk/op.rs:621-663, as staged by
+ *   set_lossy_cast / set_cast (src/op.rs:1085-1135); f32 -> f16 rounds to nearest even. */
+int cacti_hip_online_average_scale_f16_f32(int64_t n, const void *src_f16, void *dst_f32,
+                                           float src_scale, float rate, void *stream);
+int cacti_hip_online_average_square_scale_f16_f32(int64_t n, const void *src_f16, void *dst_f32,
+                                                  float src_scale, float rate, void *stream);
+int cacti_hip_online_adamw_update_f32(int64_t n, const void *grad1_avg_f32, const void *grad2_avg_f32,
+                                      void *master_f32, float signed_lr, float lr_unbias, float lamda,
+                                      float eps, void *stream);
+int cacti_hip_cast_f32_f16(int64_t n, const void *src_f32, void *dst_f16, void *stream);
+int cacti_hip_cast_f16_f32(int64_t n, const void *src_f16, void *dst_f32, void *stream);
+
+/* Host arithmetic of one AdamW32 step (AdamW32::step, src/librarium/adamw.rs:45-60, and
+ * init_online_adamw_update32, src/op.rs:984-1023): out7 = {grad_unscale, a1, a2, signed_lr,
+ * lr_unbias, lamda, eps * unbias2}, all f32, the powers taken as f32::powi does.  grad_scale <= 0
+ * stands for None.  iter_nr <= 0 is CACTI_E_INVALID (the reference panics). */
+int cacti_adamw32_scalars(int iter_nr, float grad_scale, float lr, float wd, float a1, float a2,
+                          float eps, float *out7);
+
+/* One AdamW32 step of `count` tensors in one launch: for each tensor the three thunks above and the
+ * cast of the master weights back to the f16 parameter (the loop of
+ * examples/open_llama_3b_train.rs:252-268), each element read and written once; bit-identical to
+ * the four separate thunks.  grads (f16, read), avgs, avg2s, masters (f32, updated), params (f16,
+ * written), ns (element counts) are host arrays of device pointers / sizes, read before the call
+ * returns; scalars7 as cacti_adamw32_scalars fills it; scratch: device memory of
+ * cacti_hip_adamw32_scratch_bytes(count) bytes, 8-byte aligned. */
+size_t cacti_hip_adamw32_scratch_bytes(int count);
+int cacti_hip_adamw32_step_f16_batch(int count, const void *const *grads_f16, void *const *avgs_f32,
+                                     void *const *avg2s_f32, void *const *masters_f32,
+                                     void *const *params_f16, const int64_t *ns, const float *scalars7,
+                                     void *scratch, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

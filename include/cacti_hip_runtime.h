@@ -106,6 +106,21 @@ int cacti_llama_grad_get(cacti_llama *model, int i, void *host, size_t bytes);
  * g.nan_count() (examples/open_llama_3b_train.rs:409-424, read at :587-650); bins as in
  * cacti_hip_abs_log2_hist8_f16.  One stream synchronisation for the whole call. */
 int cacti_llama_digests(cacti_llama *model, int of_grads, int64_t *hist, int64_t *nan);
+/* AdamW32 with f32 master weights and moment averages, as the reference's example sets it up
+ * (examples/open_llama_3b_train.rs:189-205, 230-243): adamw_init creates, per parameter, the f32
+ * cells master (= set_cast of the parameter), grad_avg and grad2_avg (= set_zeros).  adamw_step
+ * runs one step of every parameter from its current gradient (the loop at :252-268: adamw.step,
+ * then p.set_lossy_cast(master)) in one launch and returns without synchronising; skip_embed = 1
+ * leaves the embedding untouched as the example does (:262-263).  The new parameters are what the
+ * next cacti_llama_step reads.  adamw_state_get copies master (which = 0), grad_avg (1) or
+ * grad2_avg (2) of parameter i to host memory. */
+typedef struct {
+    float grad_scale;          /* <= 0: gradients are not scaled */
+    float lr, wd, a1, a2, eps;
+} cacti_adamw32;
+int cacti_llama_adamw_init(cacti_llama *model);
+int cacti_llama_adamw_step(cacti_llama *model, int iter_nr, const cacti_adamw32 *opt, int skip_embed);
+int cacti_llama_adamw_state_get(cacti_llama *model, int i, int which, void *host, size_t bytes);
 /* cells of the inputs (tok u16 [S], lm_tok u16 [S], loss_scale f32 [S]) and of the kept
  * outputs of the last staged cycle (logit f16 [S,V], loss f32 [S], amax u16 [S],
  * prob f32 [S,V] or 0) */

@@ -1022,6 +1022,101 @@ ORACLE_API void oracle_abs_log2_hist8_f16(i64 n, const h16 *x, i64 *hist /* [256
     for (i64 i = 0; i < n; i++) hist[oracle_abs_log2_bin(x[i])] += 1;
 }
 
+/* ------------------------------------------------------------------------- */
+/* optimiser thunks (Initialize mode: the output cell is read and overwritten)  */
+
+/* OnlineAverageScaleInitFutThunkSpec, src/thunk/op.rs:3884-3939:
+ * \u v -> v + rate * (src_scale * (f32.f16 u) - v) */
+ORACLE_API void th_online_average_scale_f16_f32(i64 n, const h16 *u, float *v, float src_scale, float rate)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) {
+        const float su = src_scale * h2f(u[i]);
+        const float d = su - v[i];
+        const float r = rate * d;
+        v[i] = v[i] + r;
+    }
+}
+
+/* OnlineAverageSquareScaleInitFutThunkSpec, src/thunk/op.rs:3941-4002:
+ * \u v -> v + rate * ((src_scale * (f32.f16 u)) * (src_scale * (f32.f16 u)) - v) */
+ORACLE_API void th_online_average_square_scale_f16_f32(i64 n, const h16 *u, float *v, float src_scale,
+                                                       float rate)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) {
+        const float su = src_scale * h2f(u[i]);
+        const float sq = su * su;
+        const float d = sq - v[i];
+        const float r = rate * d;
+        v[i] = v[i] + r;
+    }
+}
+
+/* OnlineAdamWUpdateInitFutThunkSpec, src/thunk/op.rs:4004-4062:
+ * \u v w -> w + signed_lr * (lr_unbias * (u / ((f32.sqrt v) + eps)) + lamda * w) */
+ORACLE_API void th_online_adamw_update_f32(i64 n, const float *u, const float *v, float *w, float signed_lr,
+                                           float lr_unbias, float lamda, float eps)
+{
+#pragma omp parallel for schedule(static)
+    for (i64 i = 0; i < n; i++) {
+        const float den = sqrtf(v[i]) + eps;
+        const float q = u[i] / den;
+        const float a = lr_unbias * q;
+        const float b = lamda * w[i];
+        const float c = a + b;
+        const float d = signed_lr * c;
+        w[i] = w[i] + d;
+    }
+}
+
+/* f32 integer power as compiler-rt's __powisf2 computes it (what Rust's f32::powi lowers to):
+ * square-and-multiply from the low bit, every product rounded to f32 */
+static float powi_f32(float a, int b)
+{
+    const int recip = b < 0;
+    float r = 1.0f;
+    for (;;) {
+        if (b & 1) r *= a;
+        b /= 2;
+        if (b == 0) break;
+        a *= a;
+    }
+    return recip ? 1.0f / r : r;
+}
+
+/* The seven f32 scalars one AdamW32 step passes to its three thunks: AdamW32::step,
+ * src/librarium/adamw.rs:45-60, and init_online_adamw_update32, src/op.rs:984-1023.
+ * out = {grad_unscale, a1, a2, signed_lr, lr_unbias, lamda, eps * unbias2}; grad_scale <= 0 means
+ * None.  Returns -1 for iter_nr <= 0 (the reference panics). */
+ORACLE_API int oracle_adamw32_scalars(int iter_nr, float grad_scale, float lr, float wd, float a1, float a2,
+                                      float eps, float *out)
+{
+    if (iter_nr <= 0) return -1;
+    const float unscale = grad_scale > 0.0f ? 1.0f / grad_scale : 1.0f;
+    const float unbias1 = iter_nr == 1 ? a1 : 1.0f - powi_f32(1.0f - a1, iter_nr);
+    const float unbias2 = iter_nr == 1 ? sqrtf(a2) : sqrtf(1.0f - powi_f32(1.0f - a2, iter_nr));
+    out[0] = unscale;
+    out[1] = a1;
+    out[2] = a2;
+    out[3] = -lr;
+    out[4] = unbias2 / unbias1;
+    out[5] = wd;
+    out[6] = eps * unbias2;
+    return 0;
+}
+
+/* One AdamW32 step of one tensor as the example stages it (examples/open_llama_3b_train.rs:252-268):
+ * adamw.step(..) then p.set_lossy_cast(master) (CastFutThunkSpec f32 -> f16, src/op.rs:1112-1135) */
+ORACLE_API void oracle_adamw32_step(i64 n, const h16 *grad, float *avg, float *avg2, float *master, h16 *param,
+                                    const float *sc /* [7] */)
+{
+    th_online_average_scale_f16_f32(n, grad, avg, sc[0], sc[1]);
+    th_online_average_square_scale_f16_f32(n, grad, avg2, sc[0], sc[2]);
+    th_online_adamw_update_f32(n, avg, avg2, master, sc[3], sc[4], sc[5], sc[6]);
+    th_cast_f32_f16(n, master, param);
+}
+
 ORACLE_API int oracle_num_threads(void)
 {
 #ifdef _OPENMP

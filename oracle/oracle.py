@@ -308,3 +308,60 @@ def abs_log2_hist8(x):
 def abs_log2_bin(bits):
     """Histogram bin of one f16 bit pattern."""
     return int(lib().oracle_abs_log2_bin(int(bits)))
+
+
+# ---------------------------------------------------------------- optimiser thunks
+def online_average_scale(u, v, src_scale, rate):
+    """v + rate * (src_scale * f32(u) - v) into a copy of v (src/thunk/op.rs:3884-3939)."""
+    u = h(u)
+    v = np.array(v, dtype=np.float32, copy=True, order="C")
+    lib().th_online_average_scale_f16_f32(i64(u.size), P(u), P(v), f32(src_scale), f32(rate))
+    return v
+
+
+def online_average_square_scale(u, v, src_scale, rate):
+    """v + rate * ((src_scale * f32(u))^2 - v) into a copy of v (src/thunk/op.rs:3941-4002)."""
+    u = h(u)
+    v = np.array(v, dtype=np.float32, copy=True, order="C")
+    lib().th_online_average_square_scale_f16_f32(i64(u.size), P(u), P(v), f32(src_scale), f32(rate))
+    return v
+
+
+def online_adamw_update(g1, g2, w, signed_lr, lr_unbias, lamda, eps):
+    """w + signed_lr * (lr_unbias * (g1 / (sqrt(g2) + eps)) + lamda * w) into a copy of w
+    (src/thunk/op.rs:4004-4062)."""
+    g1 = np.ascontiguousarray(g1, dtype=np.float32)
+    g2 = np.ascontiguousarray(g2, dtype=np.float32)
+    w = np.array(w, dtype=np.float32, copy=True, order="C")
+    lib().th_online_adamw_update_f32(i64(w.size), P(g1), P(g2), P(w), f32(signed_lr), f32(lr_unbias),
+                                     f32(lamda), f32(eps))
+    return w
+
+
+def cast_f32_f16(x):
+    """CastFutThunkSpec f32 -> f16, round to nearest even (src/thunk/op.rs:621-663)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.empty(x.shape, np.float16)
+    lib().th_cast_f32_f16(i64(x.size), P(x), P(y))
+    return y
+
+
+def adamw32_scalars(iter_nr, grad_scale, lr, wd, a1, a2, eps):
+    """{grad_unscale, a1, a2, signed_lr, lr_unbias, lamda, eps * unbias2} of one AdamW32 step
+    (src/librarium/adamw.rs:45-60, src/op.rs:984-1023); grad_scale None or <= 0 = unscaled."""
+    out = np.zeros(7, np.float32)
+    rc = lib().oracle_adamw32_scalars(int(iter_nr), f32(grad_scale or 0.0), f32(lr), f32(wd), f32(a1), f32(a2),
+                                      f32(eps), P(out))
+    if rc:
+        raise ValueError("adamw32: invalid iter_nr=%d (should be positive)" % iter_nr)
+    return out
+
+
+def adamw32_step(grad, avg, avg2, master, scalars):
+    """One step of one tensor: returns new (avg, avg2, master f32, param f16)."""
+    grad = h(grad)
+    avg, avg2, master = (np.array(x, dtype=np.float32, copy=True, order="C") for x in (avg, avg2, master))
+    param = np.empty(grad.shape, np.float16)
+    sc = np.ascontiguousarray(scalars, dtype=np.float32)
+    lib().oracle_adamw32_step(i64(grad.size), P(grad), P(avg), P(avg2), P(master), P(param), P(sc))
+    return avg, avg2, master, param

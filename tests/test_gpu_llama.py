@@ -165,6 +165,65 @@ def test_digests_of_parameters_and_gradients(oracle, capped):
     m.close(); ctx.close()
 
 
+@pytest.mark.parametrize("capped", [False, True])
+def test_adamw_steps_between_cycles(oracle, capped):
+    """The example's minibatch loop (examples/open_llama_3b_train.rs:230-268): master = cast(param),
+    zeroed averages, then cycle -> AdamW32 step -> cycle -> step.  Averages, master weights and the
+    f16 parameters are bit-exact against the oracle's thunks applied to the gradients the device
+    produced; the embedding stays as it was when skipped; the second cycle runs on the updated
+    parameters (its loss differs).  Also with a pool so small that the optimiser state spills."""
+    opt = dict(grad_scale=1024.0, lr=2.0e-3, wd=0.1, a1=0.1, a2=0.05, eps=1.0e-5)
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=6, norm_mean=1.0, grad_scale=1024.0)
+    ctx, m = _model(cfg)
+    m.put_params_flat(flat)
+    m.step(tok, lm_tok, scale)
+    if capped:
+        peak = ctx.stats()["pool_peak"]
+        m.close(); ctx.close()
+        ctx, m = _model(cfg, pool_bytes=int(peak))          # the cycle fits, the f32 optimiser state does not
+        m.put_params_flat(flat)
+    want_p = oracle.split_params(cfg, flat)
+    names = [n for n, _ in m.params]
+    master = {n: want_p[n].astype(np.float32) for n in names}
+    avg = {n: np.zeros(want_p[n].shape, np.float32) for n in names}
+    avg2 = {n: np.zeros(want_p[n].shape, np.float32) for n in names}
+    m.adamw_init()
+    losses = []
+    for it in (1, 2):
+        losses.append(m.step(tok, lm_tok, scale))
+        grads = m.grads()
+        m.adamw_step(it, skip_embed=(it == 1), **opt)
+        sc = oracle.adamw32_scalars(it, **opt)
+        for i, n in enumerate(names):
+            if it == 1 and n == "embed":
+                p16 = want_p[n]
+            else:
+                avg[n], avg2[n], master[n], p16 = oracle.adamw32_step(grads[n], avg[n], avg2[n], master[n], sc)
+                want_p[n] = p16
+            assert np.array_equal(m.adamw_state(i, "grad_avg").view(np.uint32), avg[n].view(np.uint32)), (it, n)
+            assert np.array_equal(m.adamw_state(i, "grad2_avg").view(np.uint32), avg2[n].view(np.uint32)), (it, n)
+            assert np.array_equal(m.adamw_state(i, "master").view(np.uint32), master[n].view(np.uint32)), (it, n)
+            assert np.array_equal(m.param(i).view(np.uint16), p16.view(np.uint16)), (it, n)
+    assert not np.array_equal(losses[0], losses[1])
+    if capped:
+        assert ctx.stats()["n_evict"] > 0
+    from cacti_amd.ffi import CactiError
+    with pytest.raises(CactiError) as e:
+        m.adamw_step(0, **opt)
+    assert e.value.code == -1
+    m.close(); ctx.close()
+
+
+def test_adamw_step_before_init_is_a_state_error(oracle):
+    from cacti_amd.ffi import CactiError
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=6)
+    ctx, m = _model(cfg)
+    with pytest.raises(CactiError) as e:
+        m.adamw_step(1)
+    assert e.value.code == -5
+    m.close(); ctx.close()
+
+
 def test_pool_too_small_is_a_clean_error(oracle):
     from cacti_amd.ffi import CactiError
     cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=3)
