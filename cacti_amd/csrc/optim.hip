@@ -9,8 +9,9 @@
 // per element instead of 24 + 18 over four launches per tensor, with the same f32 operations in the
 // same order, so the results are bit-identical to the separate thunks.
 //
-// All kernels stream: a lane owns 8 consecutive elements per step (one 16-byte f16 access, two
-// 16-byte f32 accesses per f32 tensor), non-temporal both ways since nothing is read twice.
+// All kernels stream: a lane owns 4 consecutive elements per step (one 8-byte f16 access, one
+// 16-byte access per f32 tensor), so every wave instruction covers one contiguous 512-byte or
+// 1-KiB run; non-temporal both ways since nothing is read twice.
 #include "common.h"
 #include <vector>
 
@@ -19,11 +20,11 @@ using namespace cacti;
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnits = 4;                       // 8-element units per lane
+constexpr int kUnits = 8;                       // 4-element units per lane
 constexpr int kChunk = kThreads * kUnits;       // units per workgroup (8192 elements)
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 enum Mode : int { M_AVG = 0, M_AVGSQ = 1, M_UPDATE = 2, M_CAST_F32_F16 = 3, M_CAST_F16_F32 = 4, M_STEP = 5 };
 
@@ -77,14 +78,14 @@ __device__ __forceinline__ float h2f_bits(uint32_t bits)
 __device__ __forceinline__ uint32_t f2h_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
 
 struct Unit {
-    float g[8], a[8], b[8], w[8];
+    float g[4], a[4], b[4], w[4];
 };
 
 template <int MODE>
-__device__ __forceinline__ void compute(Unit &u, uint32_t (&p)[8], const OptScalars &sc, int cnt)
+__device__ __forceinline__ void compute(Unit &u, uint32_t (&p)[4], const OptScalars &sc, int cnt)
 {
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int i = 0; i < 4; i++) {
         if (i >= cnt) break;
         if (MODE == M_AVG) u.a[i] = avg_step(u.g[i], u.a[i], sc.s[0], sc.s[1]);
         if (MODE == M_AVGSQ) u.a[i] = avgsq_step(u.g[i], u.a[i], sc.s[0], sc.s[2]);
@@ -112,26 +113,18 @@ struct Uses {
     static constexpr bool p_out = MODE == M_CAST_F32_F16 || MODE == M_STEP;
 };
 
-__device__ __forceinline__ void load8(const float *src, float (&d)[8])
+__device__ __forceinline__ void load4(const float *src, float (&d)[4])
 {
-    const f32x4 lo = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src));
-    const f32x4 hi = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src) + 1);
+    const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src));
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        d[i] = lo[i];
-        d[4 + i] = hi[i];
-    }
+    for (int i = 0; i < 4; i++) d[i] = v[i];
 }
-__device__ __forceinline__ void store8(float *dst, const float (&d)[8])
+__device__ __forceinline__ void store4(float *dst, const float (&d)[4])
 {
-    f32x4 lo, hi;
+    f32x4 v;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        lo[i] = d[i];
-        hi[i] = d[4 + i];
-    }
-    __builtin_nontemporal_store(lo, reinterpret_cast<f32x4 *>(dst));
-    __builtin_nontemporal_store(hi, reinterpret_cast<f32x4 *>(dst) + 1);
+    for (int i = 0; i < 4; i++) v[i] = d[i];
+    __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(dst));
 }
 
 // segs == nullptr: the one tensor `one`; otherwise nseg tensors, segs[] sorted by first_block
@@ -151,48 +144,48 @@ optim_kernel(OptSeg one, const OptSeg *__restrict__ segs, int nseg, OptScalars s
         sg = segs[lo];
     }
     const int64_t lb = (int64_t)blockIdx.x - sg.first_block;
-    const int64_t n8 = sg.n / 8;
+    const int64_t n4 = sg.n / 4;
     const int64_t u0 = lb * kChunk;
     Unit un[kUnits];
-    uint32_t pk[kUnits][8];
-    // all loads of the lane first (kUnits x up to 7 sixteen-byte loads in flight), then the arithmetic
+    uint32_t pk[kUnits][4];
+    // all loads of the lane first (kUnits x up to 4 loads in flight), then the arithmetic
 #pragma unroll
     for (int j = 0; j < kUnits; j++) {
         const int64_t u = u0 + j * kThreads + threadIdx.x;
-        if (u >= n8) break;
+        if (u >= n4) break;
         if (U::g_in) {
-            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(sg.g) + u);
+            const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(sg.g) + u);
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < 2; i++) {
                 un[j].g[2 * i] = h2f_bits(v[i] & 0xffff);
                 un[j].g[2 * i + 1] = h2f_bits(v[i] >> 16);
             }
         }
-        if (U::a_in) load8(sg.a + u * 8, un[j].a);
-        if (U::b_in) load8(sg.b + u * 8, un[j].b);
-        if (U::w_in) load8(sg.w + u * 8, un[j].w);
+        if (U::a_in) load4(sg.a + u * 4, un[j].a);
+        if (U::b_in) load4(sg.b + u * 4, un[j].b);
+        if (U::w_in) load4(sg.w + u * 4, un[j].w);
     }
 #pragma unroll
     for (int j = 0; j < kUnits; j++) {
         const int64_t u = u0 + j * kThreads + threadIdx.x;
-        if (u >= n8) break;
-        compute<MODE>(un[j], pk[j], sc, 8);
-        if (U::a_out) store8(sg.a + u * 8, un[j].a);
-        if (U::b_out) store8(sg.b + u * 8, un[j].b);
-        if (U::w_out) store8(sg.w + u * 8, un[j].w);
+        if (u >= n4) break;
+        compute<MODE>(un[j], pk[j], sc, 4);
+        if (U::a_out) store4(sg.a + u * 4, un[j].a);
+        if (U::b_out) store4(sg.b + u * 4, un[j].b);
+        if (U::w_out) store4(sg.w + u * 4, un[j].w);
         if (U::p_out) {
-            u32x4 v;
+            u32x2 v;
 #pragma unroll
-            for (int i = 0; i < 4; i++) v[i] = pk[j][2 * i] | (pk[j][2 * i + 1] << 16);
-            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(sg.p) + u);
+            for (int i = 0; i < 2; i++) v[i] = pk[j][2 * i] | (pk[j][2 * i + 1] << 16);
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x2 *>(sg.p) + u);
         }
     }
-    // the last n % 8 elements: one lane each of the tensor's first workgroup
-    const int rest = (int)(sg.n - n8 * 8);
+    // the last n % 4 elements: one lane each of the tensor's first workgroup
+    const int rest = (int)(sg.n - n4 * 4);
     if (lb == 0 && (int)threadIdx.x < rest) {
-        const int64_t e = n8 * 8 + threadIdx.x;
+        const int64_t e = n4 * 4 + threadIdx.x;
         Unit t;
-        uint32_t p1[8];
+        uint32_t p1[4];
         if (U::g_in) t.g[0] = h2f_bits(sg.g[e]);
         if (U::a_in) t.a[0] = sg.a[e];
         if (U::b_in) t.b[0] = sg.b[e];
@@ -207,7 +200,7 @@ optim_kernel(OptSeg one, const OptSeg *__restrict__ segs, int nseg, OptScalars s
 
 inline int64_t seg_blocks(int64_t n)
 {
-    const int64_t b = (n / 8 + kChunk - 1) / kChunk;
+    const int64_t b = (n / 4 + kChunk - 1) / kChunk;
     return b < 1 ? 1 : b;
 }
 
