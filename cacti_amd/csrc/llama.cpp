@@ -348,6 +348,80 @@ CACTI_API int cacti_llama_adamw_state_get(cacti_llama *m, int i, int which, void
     return m->ctx->c.cell_get(v[(size_t)i], host, bytes);
 }
 
+namespace cacti {
+
+int tensors_dir_keys(cacti_tensors_dir *dir, std::vector<const char *> *keys);
+int tensors_dir_lookup(cacti_tensors_dir *dir, int i, const char **dtype, const std::vector<int64_t> **shape,
+                       const void **data, size_t *bytes);
+
+int llama_load_tensors(cacti_llama *m, cacti_tensors_dir *dir, int *n_matched)
+{
+    Ctx &c = m->ctx->c;
+    // Llama::match_pickle_dir, src/librarium/llama.rs:284-302: one rule per parameter, in parameter order
+    std::vector<std::string> rules;
+    rules.push_back("embed");
+    static const char *const per_layer[9] = {"input_layernorm", "attn/q_proj", "attn/k_proj", "attn/v_proj", "attn/o_proj",
+                                             "post_attention_layernorm", "mlp/gate", "mlp/up", "mlp/down"};
+    for (size_t l = 0; l < m->layers.size(); l++)
+        for (const char *r : per_layer) rules.push_back("#" + std::to_string(l) + "/" + r);
+    rules.push_back("norm");
+    rules.push_back("lm_head");
+    CACTI_REQUIRE(rules.size() == m->params.size(), CACTI_E_STATE, "load_tensors: rule table out of step");
+    std::vector<const char *> keys, rp;
+    tensors_dir_keys(dir, &keys);
+    for (const std::string &r : rules) rp.push_back(r.c_str());
+    std::vector<int> match(rules.size(), -1);
+    int rc = cacti_cell_matcher_match(keys.data(), (int)keys.size(), rp.data(), (int)rp.size(), match.data());
+    if (rc) return rc;
+    int matched = 0;
+    for (size_t i = 0; i < m->params.size(); i++) {
+        if (match[i] < 0) continue;
+        const char *dtype;
+        const std::vector<int64_t> *shape;
+        const void *data;
+        size_t bytes;
+        tensors_dir_lookup(dir, match[i], &dtype, &shape, &data, &bytes);
+        const CellPtr p = m->params[i];
+        CACTI_REQUIRE(*shape == c.cell(p).ty.shape, CACTI_E_INVALID,
+                      "load_tensors: %s matched %s, whose shape differs from the parameter's", m->names[i].c_str(),
+                      keys[(size_t)match[i]]);
+        const int64_t n = c.cell(p).ty.numel();
+        if (!strcmp(dtype, "F16")) {
+            rc = c.cell_put(p, data, bytes);
+        } else if (!strcmp(dtype, "BF16") || !strcmp(dtype, "F32")) {
+            // a staging cell of the file's type, then the cast thunk into the parameter
+            const bool bf = dtype[0] == 'B';
+            const CellPtr t = c.cell_new(CellType(*shape, bf ? U16 : F32), false, "ingest");
+            rc = c.cell_put(t, data, bytes);
+            c.cell(t).pin++;
+            c.cell(p).pin++;
+            if (!rc) rc = c.ensure_vmem(t, true);
+            if (!rc) rc = c.ensure_vmem(p, false);
+            if (!rc)
+                rc = bf ? cacti_hip_raw_cast_bf16_f16(n, c.dev_ptr(c.cell(t).voff), c.dev_ptr(c.cell(p).voff), c.stream())
+                        : cacti_hip_cast_f32_f16(n, c.dev_ptr(c.cell(t).voff), c.dev_ptr(c.cell(p).voff), c.stream());
+            c.cell(t).pin--;
+            c.cell(p).pin--;
+            if (!rc) {
+                c.cell(p).v_valid = true;
+                c.cell(p).h_valid = false;
+                rc = c.sync();                          // the staging cell's host buffer is freed next
+            }
+            c.cell_free_all(t);
+            c.cell(t).alive = false;
+        } else {
+            set_error("load_tensors: %s: dtype %s cannot be stored into an f16 parameter", keys[(size_t)match[i]], dtype);
+            rc = CACTI_E_NOTIMPL;
+        }
+        if (rc) return rc;
+        matched++;
+    }
+    if (n_matched) *n_matched = matched;
+    return 0;
+}
+
+}  // namespace cacti
+
 CACTI_API int cacti_llama_io_cells(cacti_llama *m, int *tok, int *lm_tok, int *loss_scale,
                                    int *logit, int *loss, int *amax, int *prob)
 {

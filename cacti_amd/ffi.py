@@ -76,6 +76,10 @@ SIGNATURES = {
     "cacti_hip_online_adamw_update_f32": (ci, [i64, vp, vp, vp, f32, f32, f32, f32, vp]),
     "cacti_hip_cast_f32_f16": (ci, [i64, vp, vp, vp]),
     "cacti_hip_cast_f16_f32": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_raw_cast_bf16_f16": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_raw_cast_bf16_f32": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_raw_cast_f32_bf16": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_raw_cast_f16_bf16": (ci, [i64, vp, vp, vp]),
     "cacti_adamw32_scalars": (ci, [ci, f32, f32, f32, f32, f32, f32, vp]),
     "cacti_hip_adamw32_scratch_bytes": (sz, [ci]),
     "cacti_hip_adamw32_step_f16_batch": (ci, [ci, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
@@ -109,6 +113,13 @@ SIGNATURES = {
     "cacti_llama_param_put": (ci, [vp, ci, vp, sz]),
     "cacti_llama_grad_get": (ci, [vp, ci, vp, sz]),
     "cacti_llama_digests": (ci, [vp, ci, vp, vp]),
+    "cacti_tensors_dir_open": (ci, [C.c_char_p, pvp]),
+    "cacti_tensors_dir_close": (ci, [vp]),
+    "cacti_tensors_dir_count": (ci, [vp]),
+    "cacti_tensors_dir_entry": (ci, [vp, ci, C.c_char_p, sz, C.c_char_p, sz, C.POINTER(ci), C.POINTER(i64), pvp,
+                                C.POINTER(C.c_uint64)]),
+    "cacti_cell_matcher_match": (ci, [vp, ci, vp, ci, vp]),
+    "cacti_llama_load_tensors_dir": (ci, [vp, vp, C.POINTER(ci)]),
     "cacti_llama_adamw_init": (ci, [vp]),
     "cacti_llama_adamw_step": (ci, [vp, ci, vp, ci]),
     "cacti_llama_adamw_state_get": (ci, [vp, ci, ci, vp, sz]),

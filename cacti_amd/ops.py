@@ -344,3 +344,29 @@ def adamw32_step_(grads, avgs, avg2s, masters, params, scalars):
     scratch = torch.empty(ffi.lib().cacti_hip_adamw32_scratch_bytes(n), dtype=torch.uint8, device=grads[0].device)
     ffi.call("cacti_hip_adamw32_step_f16_batch", n, arr(grads), arr(avgs), arr(avg2s), arr(masters), arr(params),
              C.cast(ns, C.c_void_p), C.cast(sc, C.c_void_p), scratch.data_ptr(), _stream())
+
+
+# ---------------------------------------------------------------- bf16 raw casts (src/thunk/op.rs:665-803)
+def _raw_cast(name, x, in_dtype, out_dtype):
+    _chk(x, in_dtype)
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    ffi.call(name, x.numel(), x.data_ptr(), y.data_ptr(), _stream())
+    return y
+
+
+def raw_cast_bf16_f16(u):
+    """bf16 bit patterns (int16 tensor) -> f16."""
+    return _raw_cast("cacti_hip_raw_cast_bf16_f16", u, torch.int16, torch.float16)
+
+
+def raw_cast_bf16_f32(u):
+    return _raw_cast("cacti_hip_raw_cast_bf16_f32", u, torch.int16, torch.float32)
+
+
+def raw_cast_f32_bf16(x):
+    """f32 -> bf16 bit patterns (int16 tensor), truncating."""
+    return _raw_cast("cacti_hip_raw_cast_f32_bf16", x, torch.float32, torch.int16)
+
+
+def raw_cast_f16_bf16(x):
+    return _raw_cast("cacti_hip_raw_cast_f16_bf16", x, torch.float16, torch.int16)

@@ -168,6 +168,13 @@ class Llama:
         ffi.call("cacti_llama_param_info", self._m, i, None, 0, None, None, C.byref(cell), None)
         return self.ctx.cell_get(cell.value, np.float16, self.params[i][1])
 
+    def load_tensors_dir(self, tensors_dir):
+        """Stores every tensor of an open ingest.TensorsDir that Llama::match_pickle_dir's rules match
+        into its parameter (src/librarium/llama.rs:284-302); returns how many were matched."""
+        n = C.c_int(0)
+        ffi.call("cacti_llama_load_tensors_dir", self._m, tensors_dir._d, C.byref(n))
+        return n.value
+
     def adamw_init(self):
         """master = set_cast(param), grad_avg = grad2_avg = 0 (examples/open_llama_3b_train.rs:230-243)."""
         ffi.call("cacti_llama_adamw_init", self._m)

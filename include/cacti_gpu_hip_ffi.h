@@ -41,6 +41,8 @@ extern "C" {
 #define CACTI_E_INDEX (-3)     /* token / key id out of range (reference: assert)     */
 #define CACTI_E_OOM (-4)       /* pool exhausted even after eviction                  */
 #define CACTI_E_STATE (-5)     /* call not valid in the current state                 */
+#define CACTI_E_IO (-6)        /* a file cannot be opened or mapped                   */
+#define CACTI_E_FORMAT (-7)    /* a file does not have the expected layout            */
 
 /* Human-readable text for the last non-zero status returned on this thread. */
 const char *cacti_hip_last_error(void);
@@ -299,6 +301,19 @@ int cacti_hip_adamw32_step_f16_batch(int count, const void *const *grads_f16, vo
                                      void *const *avg2s_f32, void *const *masters_f32,
                                      void *const *params_f16, const int64_t *ns, const float *scalars7,
                                      void *scratch, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * bf16 held as raw u16 bit patterns <-> f16 / f32 (what set_lossy_cast stages for a bf16 source,
+ * src/op.rs:1112-1135).  n elements, contiguous, 16-byte aligned.
+ * bf16_f16: f16(f32 from (u << 16)), round to nearest even, overflow to inf;
+ *   RawCastBf16F16FutThunkSpec, src/thunk/op.rs:665-698.
+ * bf16_f32: f32 from (u << 16), exact; RawCastBf16F32FutThunkSpec, src/thunk/op.rs:700-733.
+ * f32_bf16: upper 16 bits of the f32 (truncation); RawCastF32Bf16FutThunkSpec, src/thunk/op.rs:735-768.
+ * f16_bf16: upper 16 bits of f32(x); RawCastF16Bf16FutThunkSpec, src/thunk/op.rs:770-803. */
+int cacti_hip_raw_cast_bf16_f16(int64_t n, const void *src_u16, void *dst_f16, void *stream);
+int cacti_hip_raw_cast_bf16_f32(int64_t n, const void *src_u16, void *dst_f32, void *stream);
+int cacti_hip_raw_cast_f32_bf16(int64_t n, const void *src_f32, void *dst_u16, void *stream);
+int cacti_hip_raw_cast_f16_bf16(int64_t n, const void *src_f16, void *dst_u16, void *stream);
 
 #ifdef __cplusplus
 }

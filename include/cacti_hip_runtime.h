@@ -121,6 +121,36 @@ typedef struct {
 int cacti_llama_adamw_init(cacti_llama *model);
 int cacti_llama_adamw_step(cacti_llama *model, int iter_nr, const cacti_adamw32 *opt, int skip_embed);
 int cacti_llama_adamw_state_get(cacti_llama *model, int i, int which, void *host, size_t bytes);
+/* ---- weight ingest: TensorsDir (src/util/safetensor.rs:45-160), CellMatcher (src/util/cell.rs:47-112),
+ * Llama::match_pickle_dir (src/librarium/llama.rs:284-302), resume_put (src/spine.rs:1714-1745).
+ *
+ * tensors_dir_open: `path` is a safetensors file, or a directory holding model.safetensors or the
+ * shards model-*-of-*.safetensors (taken in sorted order).  The files are memory-mapped, the
+ * headers parsed; a tensor name that occurs twice, a byte range that does not fit the file or the
+ * tensor's type, or a malformed header is CACTI_E_FORMAT, a missing file CACTI_E_IO.
+ * tensors_dir_entry: entry i in byte-wise sorted name order (the order CellMatcher scans): name,
+ * dtype as spelled in the file ("F16", "BF16", "F32", ...), shape (at most 8 dims), a pointer into
+ * the mapping (valid until close) and its length. */
+typedef struct cacti_tensors_dir cacti_tensors_dir;
+int cacti_tensors_dir_open(const char *path, cacti_tensors_dir **dir);
+int cacti_tensors_dir_close(cacti_tensors_dir *dir);
+int cacti_tensors_dir_count(cacti_tensors_dir *dir);
+int cacti_tensors_dir_entry(cacti_tensors_dir *dir, int i, char *name, size_t name_cap, char *dtype,
+                            size_t dtype_cap, int *ndim, int64_t *shape8, const void **data,
+                            uint64_t *bytes);
+/* CellMatcher::match_: rule r (components separated by '/', "#12" = the integer 12, anything else
+ * a string) takes the first key, in sorted order and not taken by an earlier rule, whose
+ * '.'-separated tokens consume the rule left to right: an integer needs a token equal to its
+ * decimal text, a string a token that equals or contains it.  match[r] = index into keys, or -1. */
+int cacti_cell_matcher_match(const char *const *keys, int nkeys, const char *const *rules, int nrules,
+                             int *match);
+/* Matches the model's parameters against the directory with the rules of Llama::match_pickle_dir
+ * and stores every matched tensor into its parameter cell: F16 as it is (resume_put), BF16 and F32
+ * through the device casts set_lossy_cast stages (src/op.rs:1112-1135).  A matched tensor whose
+ * shape differs from the parameter's is CACTI_E_INVALID (the reference panics on mismatched types),
+ * another dtype CACTI_E_NOTIMPL.  Parameters without a match keep their value; *n_matched counts the
+ * matched ones. */
+int cacti_llama_load_tensors_dir(cacti_llama *model, cacti_tensors_dir *dir, int *n_matched);
 /* cells of the inputs (tok u16 [S], lm_tok u16 [S], loss_scale f32 [S]) and of the kept
  * outputs of the last staged cycle (logit f16 [S,V], loss f32 [S], amax u16 [S],
  * prob f32 [S,V] or 0) */

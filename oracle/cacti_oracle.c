@@ -1117,6 +1117,51 @@ ORACLE_API void oracle_adamw32_step(i64 n, const h16 *grad, float *avg, float *a
     th_cast_f32_f16(n, master, param);
 }
 
+/* ------------------------------------------------------------------------- */
+/* bf16 raw casts, src/thunk/op.rs:665-803 (bf16 travels as u16 bit patterns)   */
+
+/* RawCastBf16F16: f16.f32 (f32.from_bits ((u32.u16 u) << 16)) */
+ORACLE_API void th_raw_cast_bf16_f16(i64 n, const uint16_t *x, h16 *y)
+{
+    for (i64 i = 0; i < n; i++) {
+        const uint32_t u = (uint32_t)x[i] << 16;
+        float f;
+        memcpy(&f, &u, 4);
+        y[i] = f2h(f);
+    }
+}
+/* RawCastBf16F32: f32.from_bits ((u32.u16 u) << 16) */
+ORACLE_API void th_raw_cast_bf16_f32(i64 n, const uint16_t *x, float *y)
+{
+    for (i64 i = 0; i < n; i++) {
+        const uint32_t u = (uint32_t)x[i] << 16;
+        memcpy(&y[i], &u, 4);
+    }
+}
+/* RawCastF32Bf16: u16.u32 ((f32.to_bits u) >> 16) */
+ORACLE_API void th_raw_cast_f32_bf16(i64 n, const float *x, uint16_t *y)
+{
+    for (i64 i = 0; i < n; i++) {
+        uint32_t u;
+        memcpy(&u, &x[i], 4);
+        y[i] = (uint16_t)(u >> 16);
+    }
+}
+/* RawCastF16Bf16: u16.u32 ((f32.to_bits (f32.f16 u)) >> 16) */
+ORACLE_API void th_raw_cast_f16_bf16(i64 n, const h16 *x, uint16_t *y)
+{
+    for (i64 i = 0; i < n; i++) {
+        const float f = h2f(x[i]);
+        uint32_t u;
+        memcpy(&u, &f, 4);
+        /* an IEEE conversion returns a quiet NaN for a signalling one (every convert instruction the
+         * reference can run on does); without it a NaN whose payload sits in the low 3 bits of the f16
+         * mantissa would be truncated to infinity */
+        if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x007fffffu)) u |= 0x00400000u;
+        y[i] = (uint16_t)(u >> 16);
+    }
+}
+
 ORACLE_API int oracle_num_threads(void)
 {
 #ifdef _OPENMP

@@ -365,3 +365,71 @@ def adamw32_step(grad, avg, avg2, master, scalars):
     sc = np.ascontiguousarray(scalars, dtype=np.float32)
     lib().oracle_adamw32_step(i64(grad.size), P(grad), P(avg), P(avg2), P(master), P(param), P(sc))
     return avg, avg2, master, param
+
+
+# ---------------------------------------------------------------- weight ingest
+def raw_cast(kind, x):
+    """The four bf16 raw casts (src/thunk/op.rs:665-803); bf16 travels as uint16 bit patterns."""
+    src, dst = {"bf16_f16": (np.uint16, np.float16), "bf16_f32": (np.uint16, np.float32),
+                "f32_bf16": (np.float32, np.uint16), "f16_bf16": (np.float16, np.uint16)}[kind]
+    x = np.ascontiguousarray(x, dtype=src)
+    y = np.empty(x.shape, dst)
+    getattr(lib(), "th_raw_cast_" + kind)(i64(x.size), P(x), P(y))
+    return y
+
+
+def cell_matcher_match(keys, rules):
+    """CellMatcher::match_ (src/util/cell.rs:63-112).  rules: tuples of int / str patterns.  Returns,
+    per rule, the matched key or None.  The key set is ordered; a matched key leaves it."""
+    left = sorted(set(keys), key=lambda k: k.encode())
+    out = []
+    for pat in rules:
+        pat = pat if isinstance(pat, tuple) else (pat,)
+        hit = None
+        for key in left:
+            idx = 0
+            for tok in key.split("."):
+                p = pat[idx]
+                if isinstance(p, int):
+                    if tok == "%d" % p:
+                        idx += 1
+                elif tok == p or p in tok:
+                    idx += 1
+                if idx == len(pat):
+                    break
+            if idx == len(pat):
+                hit = key
+                break
+        if hit is not None:
+            left.remove(hit)
+        out.append(hit)
+    return out
+
+
+def llama_rules(num_layers):
+    """The rules of Llama::match_pickle_dir in parameter order (src/librarium/llama.rs:284-302)."""
+    rules = [("embed",)]
+    for i in range(num_layers):
+        rules += [(i, "input_layernorm"), (i, "attn", "q_proj"), (i, "attn", "k_proj"), (i, "attn", "v_proj"),
+                  (i, "attn", "o_proj"), (i, "post_attention_layernorm"), (i, "mlp", "gate"), (i, "mlp", "up"),
+                  (i, "mlp", "down")]
+    return rules + [("norm",), ("lm_head",)]
+
+
+def read_safetensors_header(path):
+    """{name: (dtype string, shape, absolute byte range)} of one safetensors file, from the published
+    layout (u64 LE header length, JSON header, data); what TensorsDir::_reopen keeps per tensor
+    (src/util/safetensor.rs:88-113)."""
+    import json
+    import struct
+    with open(path, "rb") as f:
+        (n,) = struct.unpack("<Q", f.read(8))
+        hdr = json.loads(f.read(n).decode("utf-8"))
+    out = {}
+    for name, e in hdr.items():
+        if name == "__metadata__":
+            continue
+        b, e_ = e["data_offsets"]
+        out[name] = (e["dtype"], tuple(e["shape"]), (8 + n + b, 8 + n + e_))
+    return out
+
