@@ -535,6 +535,93 @@ def run_adamw(args):
     return out
 
 
+def run_ingest(args):
+    """Weight ingest (src/util/safetensor.rs:45-160 + resume_put + set_lossy_cast): a bf16 safetensors
+    checkpoint of the 3B model's embedding, first `--layers` (default 4) layers and LM head is written
+    to a temporary directory, then opened, matched and stored into the f16 parameter cells through
+    the device cast; value = checkpoint bytes per second from the page cache into device cells (the
+    path crosses PCIe: it is bound by the host copy into the staging cell and the upload, not by HBM)."""
+    import shutil
+    import struct
+    import tempfile
+    import torch
+    from cacti_amd import ingest
+    from cacti_amd.runtime import Ctx, Llama
+    from oracle import oracle as o
+    cfg = dict(LLAMA_3B)
+    cfg["L"] = args.layers if args.layers is not None else 4
+    ctx = Ctx(0, 0, True)
+    model = Llama(ctx, **cfg)
+    keys = ["model.embed_tokens.weight"]
+    for i in range(cfg["L"]):
+        p = "model.layers.%d." % i
+        keys += [p + "input_layernorm.weight", p + "self_attn.q_proj.weight", p + "self_attn.k_proj.weight",
+                 p + "self_attn.v_proj.weight", p + "self_attn.o_proj.weight", p + "post_attention_layernorm.weight",
+                 p + "mlp.gate_proj.weight", p + "mlp.up_proj.weight", p + "mlp.down_proj.weight"]
+    keys += ["model.norm.weight", "lm_head.weight"]
+    d = tempfile.mkdtemp(prefix="cacti_ingest_")
+    try:
+        r = np.random.default_rng(0)
+        hdr, off, blobs = {}, 0, []
+        for key, (_, shp) in zip(keys, model.params):
+            n = int(np.prod(shp))
+            bits = (r.standard_normal(n, dtype=np.float32) * 0.02).view(np.uint32) >> 16     # bf16 bit patterns
+            blobs.append(bits.astype(np.uint16))
+            hdr[key] = {"dtype": "BF16", "shape": list(shp), "data_offsets": [off, off + 2 * n]}
+            off += 2 * n
+        h = json.dumps(hdr).encode()
+        with open(os.path.join(d, "model.safetensors"), "wb") as f:
+            f.write(struct.pack("<Q", len(h)) + h)
+            for b in blobs:
+                f.write(b.tobytes())
+        nbytes = off
+
+        def load():
+            td = ingest.TensorsDir(d)
+            n = model.load_tensors_dir(td)
+            ctx.sync()
+            td.close()
+            return n
+        for _ in range(max(args.warmup, 1)):
+            assert load() == len(keys)
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            load()
+        dt = (time.perf_counter() - t0) / args.steps
+        # the cells hold f16(bf16) of the file: lm_head against the oracle's cast
+        want = o.raw_cast("bf16_f16", blobs[-1]).reshape(model.params[-1][1])
+        got = model.param(len(keys) - 1)
+        nan = np.isnan(want)
+        assert np.array_equal(got[~nan].view(np.uint16), want[~nan].view(np.uint16))
+        out = {"metric": "weight ingest: bf16 safetensors checkpoint -> f16 parameter cells on the device",
+               "value": nbytes / dt / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 1),
+               "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+               "dtype": "u16", "data": "synthetic (N(0, 0.02) bf16 weights, file in the page cache)",
+               "config": {"workload": "%d tensors, %.2f GB: embedding, %d layers, LM head of the 3B model"
+                                      % (len(keys), nbytes / 1e9, cfg["L"])},
+               "roofline": {"bound": "hbm", "achieved": 3 * nbytes / dt / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                            "frac": 3 * nbytes / dt / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                            "note": "device bytes per checkpoint byte: staging write + cast read + cast write; the "
+                                    "path is bound by the host copy and PCIe, not by HBM"}}
+        if not args.no_cpu_baseline:
+            t0 = time.time()
+            hd = o.read_safetensors_header(os.path.join(d, "model.safetensors"))
+            mm = np.memmap(os.path.join(d, "model.safetensors"), dtype=np.uint8, mode="r")
+            for k in keys:
+                b, e = hd[k][2]
+                o.raw_cast("bf16_f16", np.frombuffer(mm[b:e], dtype=np.uint16))
+            t = time.time() - t0
+            out["cpu_baseline"] = {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                                   "sample": "oracle header read + bf16->f16 cast of the same file into host arrays (%.2f s)" % t}
+        else:
+            out["cpu_baseline"] = None
+    finally:
+        shutil.rmtree(d, ignore_errors=True)
+    model.close()
+    ctx.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -544,7 +631,7 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -558,6 +645,8 @@ def main():
         out = run_digests(args)
     elif args.workload == "adamw":
         out = run_adamw(args)
+    elif args.workload == "ingest":
+        out = run_ingest(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)

@@ -445,12 +445,13 @@ int tensors_dir_keys(cacti_tensors_dir *dir, std::vector<const char *> *keys)
 }
 
 int tensors_dir_lookup(cacti_tensors_dir *dir, int i, const char **dtype, const std::vector<int64_t> **shape,
-                       const void **data, size_t *bytes)
+                       int *fd, uint64_t *off, size_t *bytes)
 {
     const TensorEntry &e = dir->tensors.at(*dir->sorted[(size_t)i]);
     *dtype = e.dtype.c_str();
     *shape = &e.shape;
-    *data = static_cast<const char *>(dir->files[(size_t)e.file].base) + e.off;
+    *fd = dir->files[(size_t)e.file].fd;
+    *off = e.off;
     *bytes = (size_t)(e.eoff - e.off);
     return 0;
 }

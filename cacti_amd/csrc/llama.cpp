@@ -352,7 +352,7 @@ namespace cacti {
 
 int tensors_dir_keys(cacti_tensors_dir *dir, std::vector<const char *> *keys);
 int tensors_dir_lookup(cacti_tensors_dir *dir, int i, const char **dtype, const std::vector<int64_t> **shape,
-                       const void **data, size_t *bytes);
+                       int *fd, uint64_t *off, size_t *bytes);
 
 int llama_load_tensors(cacti_llama *m, cacti_tensors_dir *dir, int *n_matched)
 {
@@ -378,46 +378,24 @@ int llama_load_tensors(cacti_llama *m, cacti_tensors_dir *dir, int *n_matched)
         if (match[i] < 0) continue;
         const char *dtype;
         const std::vector<int64_t> *shape;
-        const void *data;
+        int fd;
+        uint64_t off;
         size_t bytes;
-        tensors_dir_lookup(dir, match[i], &dtype, &shape, &data, &bytes);
+        tensors_dir_lookup(dir, match[i], &dtype, &shape, &fd, &off, &bytes);
         const CellPtr p = m->params[i];
         CACTI_REQUIRE(*shape == c.cell(p).ty.shape, CACTI_E_INVALID,
                       "load_tensors: %s matched %s, whose shape differs from the parameter's", m->names[i].c_str(),
                       keys[(size_t)match[i]]);
-        const int64_t n = c.cell(p).ty.numel();
-        if (!strcmp(dtype, "F16")) {
-            rc = c.cell_put(p, data, bytes);
-        } else if (!strcmp(dtype, "BF16") || !strcmp(dtype, "F32")) {
-            // a staging cell of the file's type, then the cast thunk into the parameter
-            const bool bf = dtype[0] == 'B';
-            const CellPtr t = c.cell_new(CellType(*shape, bf ? U16 : F32), false, "ingest");
-            rc = c.cell_put(t, data, bytes);
-            c.cell(t).pin++;
-            c.cell(p).pin++;
-            if (!rc) rc = c.ensure_vmem(t, true);
-            if (!rc) rc = c.ensure_vmem(p, false);
-            if (!rc)
-                rc = bf ? cacti_hip_raw_cast_bf16_f16(n, c.dev_ptr(c.cell(t).voff), c.dev_ptr(c.cell(p).voff), c.stream())
-                        : cacti_hip_cast_f32_f16(n, c.dev_ptr(c.cell(t).voff), c.dev_ptr(c.cell(p).voff), c.stream());
-            c.cell(t).pin--;
-            c.cell(p).pin--;
-            if (!rc) {
-                c.cell(p).v_valid = true;
-                c.cell(p).h_valid = false;
-                rc = c.sync();                          // the staging cell's host buffer is freed next
-            }
-            c.cell_free_all(t);
-            c.cell(t).alive = false;
-        } else {
-            set_error("load_tensors: %s: dtype %s cannot be stored into an f16 parameter", keys[(size_t)match[i]], dtype);
-            rc = CACTI_E_NOTIMPL;
-        }
+        // F16 as it is (resume_put); BF16 and F32 through the cast set_lossy_cast stages
+        const int cast = !strcmp(dtype, "F16") ? 0 : !strcmp(dtype, "BF16") ? 1 : !strcmp(dtype, "F32") ? 2 : -1;
+        CACTI_REQUIRE(cast >= 0, CACTI_E_NOTIMPL, "load_tensors: %s: dtype %s cannot be stored into an f16 parameter",
+                      keys[(size_t)match[i]], dtype);
+        rc = c.cell_ingest(p, fd, off, bytes, cast);
         if (rc) return rc;
         matched++;
     }
     if (n_matched) *n_matched = matched;
-    return 0;
+    return c.sync();
 }
 
 }  // namespace cacti

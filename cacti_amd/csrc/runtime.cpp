@@ -4,7 +4,10 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <unistd.h>
+
 #include <algorithm>
+#include <thread>
 
 #include "common.h"
 
@@ -100,6 +103,10 @@ Ctx::~Ctx()
     }
     if (ev0_) hipEventDestroy(ev0_);
     if (ev1_) hipEventDestroy(ev1_);
+    for (int k = 0; k < 2; k++) {
+        if (ingest_host_[k]) hipHostFree(ingest_host_[k]);
+        if (ingest_ev_[k]) hipEventDestroy(ingest_ev_[k]);
+    }
     if (base_) hipFree(base_);
     if (own_stream_ && stream_) hipStreamDestroy(stream_);
 }
@@ -308,6 +315,84 @@ int Ctx::cells_digest(const CellPtr *cells, int n, int64_t *hist, int64_t *nan)
         memcpy(hist + (size_t)i * 256, host.data() + (size_t)i * 257, 256 * sizeof(int64_t));
         nan[i] = host[(size_t)i * 257 + 256];
     }
+    return 0;
+}
+
+namespace {
+constexpr size_t kIngestChunk = 32u << 20;        // source bytes per staging buffer
+constexpr int kIngestThreads = 8;
+
+// pread the whole range, split over a few threads (the page cache copies at a few GB/s per core)
+bool read_range(int fd, uint64_t off, char *dst, size_t bytes)
+{
+    const int nt = bytes >= ((size_t)kIngestThreads << 20) ? kIngestThreads : 1;
+    std::vector<std::thread> th;
+    std::vector<char> ok((size_t)nt, 1);
+    const size_t per = ((bytes + (size_t)nt - 1) / (size_t)nt + 4095) & ~(size_t)4095;
+    for (int t = 0; t < nt; t++) {
+        const size_t b = std::min(bytes, per * (size_t)t), e = std::min(bytes, b + per);
+        auto work = [fd, off, dst, b, e, &ok, t]() {
+            size_t done = b;
+            while (done < e) {
+                const ssize_t r = pread(fd, dst + done, e - done, (off_t)(off + done));
+                if (r <= 0) {
+                    ok[(size_t)t] = 0;
+                    return;
+                }
+                done += (size_t)r;
+            }
+        };
+        if (t + 1 < nt) th.emplace_back(work);
+        else work();
+    }
+    for (std::thread &x : th) x.join();
+    for (char v : ok)
+        if (!v) return false;
+    return true;
+}
+}  // namespace
+
+int Ctx::cell_ingest(CellPtr ci, int fd, uint64_t off, size_t bytes, int cast)
+{
+    CACTI_REQUIRE(ci > 0 && (size_t)ci < cells_.size() && cells_[ci].alive, CACTI_E_INVALID, "cell_ingest: dead cell");
+    CACTI_REQUIRE(cast >= 0 && cast <= 2, CACTI_E_INVALID, "cell_ingest: unknown cast %d", cast);
+    const size_t dst_bytes = cast == 2 ? bytes / 2 : bytes;
+    CACTI_REQUIRE(dst_bytes == cells_[ci].ty.bytes() && (cast == 0 || cells_[ci].ty.dtype == F16), CACTI_E_INVALID,
+                  "cell_ingest: %zu source bytes do not fill cell %s", bytes, cells_[ci].name.c_str());
+    for (int k = 0; k < 2; k++) {
+        if (!ingest_host_[k]) CACTI_HIP(hipHostMalloc(&ingest_host_[k], kIngestChunk, hipHostMallocDefault));
+        if (!ingest_ev_[k]) CACTI_HIP(hipEventCreateWithFlags(&ingest_ev_[k], hipEventDisableTiming));
+    }
+    cells_[ci].pin++;
+    int rc = ensure_vmem(ci, false);
+    size_t scratch = kNoOffset;
+    if (!rc && cast) rc = pool_alloc(2 * kIngestChunk, &scratch);
+    char *dst = rc ? nullptr : static_cast<char *>(dev_ptr(cells_[ci].voff));
+    int buf = 0;
+    for (size_t done = 0; done < bytes && !rc; done += kIngestChunk, buf ^= 1) {
+        const size_t n = std::min(kIngestChunk, bytes - done);
+        // the upload that last read this staging buffer must have finished
+        rc = hip_status(hipEventSynchronize(ingest_ev_[buf]), "ingest wait");
+        if (rc) break;
+        if (!read_range(fd, off + done, static_cast<char *>(ingest_host_[buf]), n)) {
+            set_error("cell_ingest: short read at offset %llu", (unsigned long long)(off + done));
+            rc = CACTI_E_IO;
+            break;
+        }
+        char *stage = cast ? static_cast<char *>(dev_ptr(scratch)) + (size_t)buf * kIngestChunk : dst + done;
+        rc = hip_status(hipMemcpyAsync(stage, ingest_host_[buf], n, hipMemcpyHostToDevice, stream_), "ingest upload");
+        if (!rc) rc = hip_status(hipEventRecord(ingest_ev_[buf], stream_), "ingest record");
+        bytes_h2d_ += n;
+        if (!rc && cast == 1) rc = cacti_hip_raw_cast_bf16_f16((int64_t)(n / 2), stage, dst + done, stream_);
+        if (!rc && cast == 2) rc = cacti_hip_cast_f32_f16((int64_t)(n / 4), stage, dst + done / 2, stream_);
+    }
+    if (scratch != kNoOffset) pool_.free(scratch);               // reuse is ordered on the stream
+    cells_[ci].pin--;
+    if (rc) return rc;
+    Cell &c = cells_[ci];
+    host_free(c);
+    c.v_valid = true;
+    c.h_valid = false;
     return 0;
 }
 

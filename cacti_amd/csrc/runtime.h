@@ -142,6 +142,11 @@ class Ctx {
     // without synchronising.
     int cells_adamw32(int n, const CellPtr *grads, const CellPtr *avgs, const CellPtr *avg2s,
                       const CellPtr *masters, const CellPtr *params, const float *sc);
+    // Streams `bytes` of a file (at `off` of `fd`) into the device replica of cell c: the range is
+    // read by a few threads into two page-locked buffers in turn, uploaded, and (cast != 0)
+    // converted on the device: 0 = bytes as they are, 1 = bf16 bit patterns -> f16, 2 = f32 -> f16.
+    // The cell ends with a device value and no host replica.  Returns with the work queued.
+    int cell_ingest(CellPtr c, int fd, uint64_t off, size_t bytes, int cast);
     int cell_cast_f16_f32(CellPtr src, CellPtr dst);              // set_cast, src/op.rs:1085-1096
     int cell_zero(CellPtr c);                                    // set_zeros, src/op.rs:1137-1146
     int cell_free_all(CellPtr c);
@@ -231,6 +236,9 @@ class Ctx {
     std::vector<std::string> ev_keys_;
     std::map<std::string, std::pair<double, uint64_t>> times_;
     hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
+    // cell_ingest: two page-locked staging buffers and the event after the last upload from each
+    void *ingest_host_[2] = {nullptr, nullptr};
+    hipEvent_t ingest_ev_[2] = {nullptr, nullptr};
 };
 
 }  // namespace cacti
