@@ -303,6 +303,10 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nbl
     p.win = 0;
     if (vec >= 4 && !ta && tb && K <= 128 && beta == 0.f && tri <= 1)
         return gemm_nt_smallk_launch(p, nblk, st);
+    // one to four rows against a weight matrix (decoding): a stream over B
+    static const bool no_skinny = getenv("CACTI_GEMM_NO_SKINNY") != nullptr;
+    if (vec == 8 && !ta && tb && M <= 4 && nblk == 1 && beta == 0.f && tri == 0 && !no_skinny)
+        return gemm_skinny_nt_launch(M, N, K, alpha, p.A, lda, p.B, ldb, p.C, ldc, st);
     // The attention products with a [sequence, heads, head_dim] operand: A (probabilities or
     // their adjoint) is 16-byte aligned, B and C are per-head slabs whose offset (head_dim 100)
     // is only a multiple of 8 bytes.  Addressed from the 16-byte boundary below each slab they

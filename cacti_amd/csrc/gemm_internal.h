@@ -42,4 +42,9 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
 // 8-byte aligned, K % 4 == 0, beta = 0, tri 0 or 1
 int gemm_nt_smallk_launch(const GemmArgs &p, int64_t nblk, hipStream_t st);
 
+// C[M,N] = f16(alpha A B^T) for 1 <= M <= 4: a stream over B ([N,K] row-major, rows 16-byte
+// aligned, K % 8 == 0), beta = 0; A rows 16-byte aligned
+int gemm_skinny_nt_launch(int64_t M, int64_t N, int64_t K, float alpha, const half_t *A, int64_t lda,
+                          const half_t *B, int64_t ldb, half_t *C, int64_t ldc, hipStream_t st);
+
 }  // namespace cacti

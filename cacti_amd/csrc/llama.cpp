@@ -511,3 +511,219 @@ CACTI_API int cacti_llama_step(cacti_llama *m, const uint16_t *tok, const uint16
     TRY(c.check_status());
     return c.cell_get(m->out_loss, loss_out, S * 4);
 }
+
+// ---------------------------------------------------------------------------
+// KV-cached forward pass: LlamaCached, src/librarium/llama.rs:561-963 (batch 1, q_group 1).
+// The pass runs eagerly on the context's stream: temporaries come from the pool and go back at
+// the end of the call (reuse is ordered on the stream), parameters and caches are stable cells.
+struct cacti_llama_cached {
+    cacti_llama *base;                       // shares the parameter cells (LlamaCached::from(Llama))
+    int64_t cap;
+    std::vector<CellPtr> k_cache, v_cache;   // per layer [cap, H, Dh] f16
+    CellPtr in_tok;                          // [cap] u16
+    // outputs of the last apply (pool regions kept until the next apply or destroy)
+    size_t out_logit = kNoOffset, out_prob = kNoOffset, out_tok = kNoOffset;
+    int64_t out_rows = 0;
+};
+
+namespace {
+
+void cached_drop_outputs(cacti_llama_cached *k)
+{
+    Ctx &c = k->base->ctx->c;
+    for (size_t *o : {&k->out_logit, &k->out_prob, &k->out_tok})
+        if (*o != kNoOffset) {
+            c.pool_free(*o);
+            *o = kNoOffset;
+        }
+    k->out_rows = 0;
+}
+
+}  // namespace
+
+CACTI_API int cacti_llama_cached_create(cacti_llama *model, int64_t seq_cap, cacti_llama_cached **out)
+{
+    CACTI_REQUIRE(model && out, CACTI_E_INVALID, "llama_cached_create: null argument");
+    // the position tables are the model's (from_train keeps model.cos / model.sin, llama.rs:657-686)
+    CACTI_REQUIRE(seq_cap > 0 && seq_cap % 8 == 0 && seq_cap <= model->cfg.S, CACTI_E_INVALID,
+                  "llama_cached_create: seq_cap must be a multiple of 8 and at most the model's %lld",
+                  (long long)model->cfg.S);
+    Ctx &c = model->ctx->c;
+    cacti_llama_cached *k = new cacti_llama_cached();
+    k->base = model;
+    k->cap = seq_cap;
+    for (int64_t l = 0; l < model->cfg.L; l++) {
+        const std::string p = "l" + std::to_string(l) + ".";
+        k->k_cache.push_back(c.cell_new(CellType({seq_cap, model->cfg.H, model->cfg.Dh}, F16), true, (p + "k_cache").c_str()));
+        k->v_cache.push_back(c.cell_new(CellType({seq_cap, model->cfg.H, model->cfg.Dh}, F16), true, (p + "v_cache").c_str()));
+        c.set_const(k->k_cache.back());
+        c.set_const(k->v_cache.back());
+    }
+    k->in_tok = c.cell_new(CellType({seq_cap}, U16), true, "cached_in_tok");
+    c.set_const(k->in_tok);
+    int rc = cacti_llama_cached_reset_state(k);
+    if (!rc) rc = c.cell_zero(k->in_tok);
+    if (rc) {
+        delete k;
+        return rc;
+    }
+    *out = k;
+    return 0;
+}
+
+CACTI_API int cacti_llama_cached_destroy(cacti_llama_cached *k)
+{
+    if (!k) return 0;
+    Ctx &c = k->base->ctx->c;
+    cached_drop_outputs(k);
+    for (CellPtr x : k->k_cache) { c.cell_free_all(x); c.cell(x).alive = false; }
+    for (CellPtr x : k->v_cache) { c.cell_free_all(x); c.cell(x).alive = false; }
+    c.cell_free_all(k->in_tok);
+    c.cell(k->in_tok).alive = false;
+    delete k;
+    return 0;
+}
+
+// LlamaCached::reset_state, src/librarium/llama.rs:784-789
+CACTI_API int cacti_llama_cached_reset_state(cacti_llama_cached *k)
+{
+    CACTI_REQUIRE(k, CACTI_E_INVALID, "llama_cached_reset_state: null model");
+    Ctx &c = k->base->ctx->c;
+    for (size_t l = 0; l < k->k_cache.size(); l++) {
+        int rc = c.cell_zero(k->k_cache[l]);
+        if (!rc) rc = c.cell_zero(k->v_cache[l]);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+CACTI_API int cacti_llama_cached_set_tokens(cacti_llama_cached *k, const uint16_t *tok, int64_t n)
+{
+    CACTI_REQUIRE(k && (tok || n == 0) && n >= 0 && n <= k->cap, CACTI_E_INVALID,
+                  "llama_cached_set_tokens: %lld tokens do not fit the capacity", (long long)n);
+    std::vector<uint16_t> buf((size_t)k->cap, 0);                 // the rest of the input is the pad token 0
+    for (int64_t i = 0; i < n; i++) buf[(size_t)i] = tok[i];
+    return k->base->ctx->c.cell_put(k->in_tok, buf.data(), buf.size() * 2);
+}
+
+CACTI_API int cacti_llama_cached_get_tokens(cacti_llama_cached *k, uint16_t *tok)
+{
+    CACTI_REQUIRE(k && tok, CACTI_E_INVALID, "llama_cached_get_tokens: null argument");
+    return k->base->ctx->c.cell_get(k->in_tok, tok, (size_t)k->cap * 2);
+}
+
+CACTI_API int cacti_llama_cached_apply(cacti_llama_cached *k, int64_t prev, int64_t next, int want_prob)
+{
+    CACTI_REQUIRE(k, CACTI_E_INVALID, "llama_cached_apply: null model");
+    cacti_llama *m = k->base;
+    Ctx &c = m->ctx->c;
+    const cacti_llama_cfg &g = m->cfg;
+    const int64_t T = next - prev, D = g.D, H = g.H, Dh = g.Dh, F = g.F, V = g.V, cap = k->cap;
+    CACTI_REQUIRE(prev >= 0 && T > 0 && next <= cap, CACTI_E_INVALID,
+                  "llama_cached_apply: positions [%lld, %lld) outside the capacity %lld", (long long)prev,
+                  (long long)next, (long long)cap);
+    const int64_t Cw = (next + 7) / 8 * 8;                        // cached columns, rounded up to the vector width
+    const float alpha = 1.0f / sqrtf((float)Dh);
+    hipStream_t st = c.stream();
+    cached_drop_outputs(k);
+
+    // every cell the pass touches is made resident and pinned for the duration of the call
+    std::vector<CellPtr> used = m->params;
+    used.insert(used.end(), k->k_cache.begin(), k->k_cache.end());
+    used.insert(used.end(), k->v_cache.begin(), k->v_cache.end());
+    used.push_back(k->in_tok);
+    used.push_back(m->cos);
+    used.push_back(m->sin);
+    int rc = 0;
+    size_t npinned = 0;
+    for (; npinned < used.size() && !rc; npinned++) {
+        c.cell(used[npinned]).pin++;
+        rc = c.ensure_vmem(used[npinned], true);
+    }
+    std::vector<size_t> temps;
+    auto tmp = [&](int64_t elems, size_t esz) -> char * {
+        size_t off;
+        if (rc) return nullptr;
+        rc = c.pool_alloc((size_t)elems * esz, &off);
+        if (rc) return nullptr;
+        temps.push_back(off);
+        return static_cast<char *>(c.dev_ptr(off));
+    };
+    auto P = [&](CellPtr x) { return c.dev_ptr(c.cell(x).voff); };
+    char *x = tmp(T * D, 2), *pre = tmp(T * D, 2), *q = tmp(T * D, 2), *qr = tmp(T * D, 2), *kk = tmp(T * D, 2),
+         *kr = tmp(T * D, 2), *v = tmp(T * D, 2), *attn = tmp(T * D, 2), *o = tmp(T * D, 2), *x1 = tmp(T * D, 2),
+         *post = tmp(T * D, 2), *up = tmp(T * F, 2), *gate = tmp(T * F, 2), *h = tmp(T * F, 2), *down = tmp(T * D, 2),
+         *s16 = tmp(T * H * Cw, 2);
+    // outputs
+    if (!rc) rc = c.pool_alloc((size_t)(T * V) * 2, &k->out_logit);
+    if (!rc) rc = c.pool_alloc((size_t)T * 2, &k->out_tok);
+    if (!rc && want_prob) rc = c.pool_alloc((size_t)(T * V) * 4, &k->out_prob);
+#define STEP(call)          \
+    do {                    \
+        if (!rc) rc = (call); \
+    } while (0)
+    if (!rc) {
+        const char *cosr = static_cast<const char *>(P(m->cos)) + prev * Dh * 2;
+        const char *sinr = static_cast<const char *>(P(m->sin)) + prev * Dh * 2;
+        char *tok = static_cast<char *>(P(k->in_tok));
+        // stream = embed.outer_select(in_tok[prev .. next])
+        STEP(cacti_hip_embed_fwd(V, D, P(m->embed), T, tok + prev * 2, x, c.status_ptr(), st));
+        STEP(cacti_hip_rms_norm_fwd(T, D, x, P(m->layers.empty() ? m->head_norm : m->layers[0].pre_norm), g.eps, pre, st));
+        for (size_t l = 0; l < m->layers.size() && !rc; l++) {
+            const LayerCells &w = m->layers[l];
+            char *kc = static_cast<char *>(P(k->k_cache[l])), *vc = static_cast<char *>(P(k->v_cache[l]));
+            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.q), D, 0.f, q, D, st));
+            STEP(cacti_hip_rope_fwd(T, H, Dh, q, cosr, sinr, qr, st));
+            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.k), D, 0.f, kk, D, st));
+            STEP(cacti_hip_rope_fwd(T, H, Dh, kk, cosr, sinr, kr, st));
+            // k_cache[prev .. next] += k, v_cache[prev .. next] += v
+            STEP(cacti_hip_add_f16(T * D, kc + prev * D * 2, kr, kc + prev * D * 2, st));
+            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.v), D, 0.f, v, D, st));
+            STEP(cacti_hip_add_f16(T * D, vc + prev * D * 2, v, vc + prev * D * 2, st));
+            // scores against the cache, row-causal mask + softmax (in place), P V.  Columns from
+            // `next` on are masked for every row, so only the first Cw of the cap columns are formed.
+            STEP(cacti_hip_gemm_f16_strided_batched(0, 1, H, T, Cw, Dh, alpha, qr, D, Dh, kc, D, Dh, 0.f, s16, H * Cw, Cw, st));
+            STEP(cacti_hip_row_causal_softmax_fwd(T, H, Cw, Cw, prev, s16, s16, st));
+            STEP(cacti_hip_gemm_f16_strided_batched(0, 0, H, T, Dh, Cw, 1.f, s16, H * Cw, Cw, vc, D, Dh, 0.f, attn, D, Dh, st));
+            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, attn, D, P(w.o), D, 0.f, o, D, st));
+            STEP(cacti_hip_add_rms_norm_fwd(T, D, x, o, P(w.post_norm), g.eps, x1, post, st));
+            STEP(cacti_hip_gemm_f16(0, 1, T, F, D, 1.f, post, D, P(w.up), D, 0.f, up, F, st));
+            STEP(cacti_hip_gemm_f16(0, 1, T, F, D, 1.f, post, D, P(w.gate), D, 0.f, gate, F, st));
+            STEP(cacti_hip_silu_gate_fwd(T * F, gate, up, h, st));
+            STEP(cacti_hip_gemm_f16(0, 1, T, D, F, 1.f, h, F, P(w.down), F, 0.f, down, D, st));
+            const CellPtr wn = l + 1 < m->layers.size() ? m->layers[l + 1].pre_norm : m->head_norm;
+            STEP(cacti_hip_add_rms_norm_fwd(T, D, x1, down, P(wn), g.eps, x, pre, st));
+        }
+        void *logit = c.dev_ptr(k->out_logit), *otok = c.dev_ptr(k->out_tok);
+        STEP(cacti_hip_gemm_f16(0, 1, T, V, D, 1.f, pre, D, P(m->lm_head), D, 0.f, logit, V, st));
+        STEP(cacti_hip_softmax_ce_fwd(T, V, logit, nullptr, want_prob ? c.dev_ptr(k->out_prob) : nullptr, nullptr,
+                                      otok, nullptr, st));
+        // in_tok[next] += out_lm_tok[T - 1]
+        if (next < cap) STEP(cacti_hip_append_token_u16(tok, next, otok, T - 1, st));
+        if (!rc) {
+            c.cell(k->in_tok).h_valid = false;
+            for (size_t l = 0; l < m->layers.size(); l++)
+                c.cell(k->k_cache[l]).h_valid = c.cell(k->v_cache[l]).h_valid = false;
+            k->out_rows = T;
+        }
+    }
+#undef STEP
+    for (size_t off : temps) c.pool_free(off);                   // reuse is ordered on the stream
+    for (size_t i = 0; i < npinned; i++) c.cell(used[i]).pin--;
+    if (rc) cached_drop_outputs(k);
+    return rc;
+}
+
+CACTI_API int cacti_llama_cached_outputs(cacti_llama_cached *k, void *logit_f16, float *prob, uint16_t *tok)
+{
+    CACTI_REQUIRE(k && k->out_rows > 0, CACTI_E_STATE, "llama_cached_outputs: no apply has run");
+    CACTI_REQUIRE(!prob || k->out_prob != kNoOffset, CACTI_E_STATE, "llama_cached_outputs: the last apply kept no probabilities");
+    Ctx &c = k->base->ctx->c;
+    hipStream_t st = c.stream();
+    const int64_t T = k->out_rows, V = k->base->cfg.V;
+    if (logit_f16) CACTI_HIP(hipMemcpyAsync(logit_f16, c.dev_ptr(k->out_logit), (size_t)(T * V) * 2, hipMemcpyDeviceToHost, st));
+    if (prob) CACTI_HIP(hipMemcpyAsync(prob, c.dev_ptr(k->out_prob), (size_t)(T * V) * 4, hipMemcpyDeviceToHost, st));
+    if (tok) CACTI_HIP(hipMemcpyAsync(tok, c.dev_ptr(k->out_tok), (size_t)T * 2, hipMemcpyDeviceToHost, st));
+    return c.check_status();                                     // syncs; raises a token id out of range
+}
+

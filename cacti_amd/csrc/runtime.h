@@ -155,6 +155,7 @@ class Ctx {
     // the current version (uploading from the host replica)
     int ensure_vmem(CellPtr c, bool need_value);
     int pool_alloc(size_t bytes, size_t *off);                   // with soft-OOM eviction
+    void pool_free(size_t off) { pool_.free(off); }              // later reuse is ordered on the stream
     int try_soft_oom(size_t need);
     int evict(CellPtr c);                                        // VMem -> Mem, drop VMem
 

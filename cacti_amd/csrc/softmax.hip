@@ -321,6 +321,92 @@ __global__ void check_tok_kernel(int64_t N, int V, const uint16_t *tok, int *sta
         default: { constexpr int CH = 16; CALL; } break;             \
     }
 
+namespace {
+
+// Row-causal softmax for the cached forward pass: T new rows at positions row0 .. row0 + T - 1
+// against C cached columns; column j of row t is live when j <= t + row0.  One wave per row
+// (t, h); the row is read three times (it is short and stays in cache): maximum, sum, quotient.
+// The per-lane partial sums run over the same 8-column pieces in the same order as in
+// causal_softmax_kernel, so a whole sequence processed as one block gives the same bits.
+__global__ void __launch_bounds__(kRowsPerBlock * 64)
+row_causal_softmax_kernel(int64_t T, int H, int64_t C, int64_t ld, int64_t row0, const half_t *__restrict__ s16,
+                          half_t *__restrict__ p16)
+{
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + wid;
+    if (row >= T * H) return;
+    const int64_t i = row / H + row0;             // last live column
+    const half_t *sr = s16 + row * ld;
+    half_t *pr = p16 + row * ld;
+    const int64_t live = (i + 1 < C ? i + 1 : C); // number of live columns
+    float mx = -INFINITY;
+    for (int64_t j0 = (int64_t)lane * 8; j0 < live; j0 += 512) {
+        const h8 v = ld8(sr + j0);
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            if (j0 + k < live) mx = fmaxf(mx, h2f(v.v[k]));
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int64_t j0 = (int64_t)lane * 8; j0 < live; j0 += 512) {
+        const h8 v = ld8(sr + j0);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float t = exp_nonpos(fmaxf(h2f(v.v[k]) - mx, -100.0f));
+            sum += (j0 + k < live) ? t : 0.f;
+        }
+    }
+    sum = wave_sum(sum);
+    const RowDivide div(sum);
+    for (int64_t j0 = (int64_t)lane * 8; j0 < C; j0 += 512) {
+        h8 o;
+        if (j0 < live) {
+            const h8 v = ld8(sr + j0);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float t = exp_nonpos(fmaxf(h2f(v.v[k]) - mx, -100.0f));
+                o.v[k] = (j0 + k < live) ? f2h(div(t)) : (half_t)0.f;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k++) o.v[k] = (half_t)0.f;
+        }
+        st8(pr + j0, o);
+    }
+}
+
+// in_tok[pos] += out_tok[last]: the generated token appended to the input (u16 add as the
+// reference's `+=` on a zero-filled slot, src/librarium/llama.rs:958-959)
+__global__ void append_token_kernel(uint16_t *in_tok, int64_t pos, const uint16_t *out_tok, int64_t last)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) in_tok[pos] = (uint16_t)(in_tok[pos] + out_tok[last]);
+}
+
+}  // namespace
+
+CACTI_API int cacti_hip_row_causal_softmax_fwd(int64_t T, int64_t H, int64_t C, int64_t ld, int64_t initial_row,
+                                               const void *s16, void *p16, void *stream)
+{
+    CACTI_REQUIRE(T > 0 && H > 0 && C > 0 && s16 && p16 && initial_row >= 0, CACTI_E_INVALID,
+                  "row_causal_softmax_fwd: null pointer or empty shape");
+    CACTI_REQUIRE(C % 8 == 0 && ld % 8 == 0 && ld >= C, CACTI_E_NOTIMPL,
+                  "row_causal_softmax_fwd: need C %% 8 == 0 and a row pitch that is a multiple of 8 and >= C");
+    CACTI_REQUIRE(aligned(s16, 16) && aligned(p16, 16), CACTI_E_INVALID,
+                  "row_causal_softmax_fwd: tensors must be 16-byte aligned");
+    const unsigned grid = (unsigned)((T * H + kRowsPerBlock - 1) / kRowsPerBlock);
+    hipLaunchKernelGGL(row_causal_softmax_kernel, dim3(grid), dim3(kRowsPerBlock * 64), 0, (hipStream_t)stream, T,
+                       (int)H, C, ld, initial_row, (const half_t *)s16, (half_t *)p16);
+    return launch_status("row_causal_softmax_fwd");
+}
+
+CACTI_API int cacti_hip_append_token_u16(void *in_tok, int64_t pos, const void *out_tok, int64_t last, void *stream)
+{
+    CACTI_REQUIRE(in_tok && out_tok && pos >= 0 && last >= 0, CACTI_E_INVALID, "append_token: bad argument");
+    hipLaunchKernelGGL(append_token_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (uint16_t *)in_tok, pos,
+                       (const uint16_t *)out_tok, last);
+    return launch_status("append_token");
+}
+
 static int causal_check(int64_t S, int64_t H, const void *a, const void *b, const char *who)
 {
     CACTI_REQUIRE(S > 0 && H > 0 && a && b, CACTI_E_INVALID, "%s: null pointer or empty shape", who);

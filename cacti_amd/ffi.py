@@ -76,6 +76,8 @@ SIGNATURES = {
     "cacti_hip_online_adamw_update_f32": (ci, [i64, vp, vp, vp, f32, f32, f32, f32, vp]),
     "cacti_hip_cast_f32_f16": (ci, [i64, vp, vp, vp]),
     "cacti_hip_cast_f16_f32": (ci, [i64, vp, vp, vp]),
+    "cacti_hip_row_causal_softmax_fwd": (ci, [i64, i64, i64, i64, i64, vp, vp, vp]),
+    "cacti_hip_append_token_u16": (ci, [vp, i64, vp, i64, vp]),
     "cacti_hip_raw_cast_bf16_f16": (ci, [i64, vp, vp, vp]),
     "cacti_hip_raw_cast_bf16_f32": (ci, [i64, vp, vp, vp]),
     "cacti_hip_raw_cast_f32_bf16": (ci, [i64, vp, vp, vp]),
@@ -120,6 +122,13 @@ SIGNATURES = {
                                 C.POINTER(C.c_uint64)]),
     "cacti_cell_matcher_match": (ci, [vp, ci, vp, ci, vp]),
     "cacti_llama_load_tensors_dir": (ci, [vp, vp, C.POINTER(ci)]),
+    "cacti_llama_cached_create": (ci, [vp, i64, pvp]),
+    "cacti_llama_cached_destroy": (ci, [vp]),
+    "cacti_llama_cached_reset_state": (ci, [vp]),
+    "cacti_llama_cached_set_tokens": (ci, [vp, vp, i64]),
+    "cacti_llama_cached_get_tokens": (ci, [vp, vp]),
+    "cacti_llama_cached_apply": (ci, [vp, i64, i64, ci]),
+    "cacti_llama_cached_outputs": (ci, [vp, vp, vp, vp]),
     "cacti_llama_adamw_init": (ci, [vp]),
     "cacti_llama_adamw_step": (ci, [vp, ci, vp, ci]),
     "cacti_llama_adamw_state_get": (ci, [vp, ci, ci, vp, sz]),

@@ -235,3 +235,48 @@ class Llama:
         if want_prob:
             out["prob"] = c.cell_get(io["prob"], np.float32, (S, V))
         return out
+
+
+class LlamaCached:
+    """LlamaCached (src/librarium/llama.rs:561-963) on the parameters of a Llama: incremental forward
+    passes over a key / value cache."""
+
+    def __init__(self, model, seq_cap):
+        self.model = model
+        self.cap = int(seq_cap)
+        self._k = C.c_void_p()
+        ffi.call("cacti_llama_cached_create", model._m, self.cap, C.byref(self._k))
+        self._rows, self._prob = 0, False
+
+    def close(self):
+        if self._k:
+            ffi.lib().cacti_llama_cached_destroy(self._k)
+            self._k = None
+
+    def reset_state(self):
+        ffi.call("cacti_llama_cached_reset_state", self._k)
+
+    def set_tokens(self, tok):
+        tok = np.ascontiguousarray(tok, dtype=np.uint16)
+        ffi.call("cacti_llama_cached_set_tokens", self._k, tok.ctypes.data, tok.size)
+
+    def tokens(self):
+        out = np.empty(self.cap, np.uint16)
+        ffi.call("cacti_llama_cached_get_tokens", self._k, out.ctypes.data)
+        return out
+
+    def apply(self, prev, next_, want_prob=False):
+        """Queues positions prev .. next_-1; read the results with outputs()."""
+        ffi.call("cacti_llama_cached_apply", self._k, int(prev), int(next_), int(want_prob))
+        self._rows, self._prob = int(next_) - int(prev), bool(want_prob)
+
+    def outputs(self, want_logit=True):
+        """dict(logit [T,V] f16 or None, tok [T] u16, prob [T,V] f32 or None) of the last apply."""
+        T, V = self._rows, self.model.cfg.V
+        logit = np.empty((T, V), np.float16) if want_logit else None
+        prob = np.empty((T, V), np.float32) if self._prob else None
+        tok = np.empty(T, np.uint16)
+        ffi.call("cacti_llama_cached_outputs", self._k, logit.ctypes.data if want_logit else None,
+                 prob.ctypes.data if self._prob else None, tok.ctypes.data)
+        return dict(logit=logit, tok=tok, prob=prob)
+

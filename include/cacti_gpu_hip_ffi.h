@@ -201,6 +201,18 @@ int cacti_hip_causal_softmax_fwd(int64_t S, int64_t H, const void *s16, void *p1
 int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const void *dp16,
                                  void *ds16, void *stream);
 
+/* Row-causal softmax of the cached forward pass, src/librarium/llama.rs:905-907:
+ * P16 = f16(softmax_j(mask(f32(S16)))) with mask j > t + initial_row -> -inf
+ * (Cast, RowCausalAttentionMaskFutThunkSpec src/librarium/llama.rs:1052-1112, InnerSoftmax, Cast).
+ * s16, p16: [T,H,ld] f16, columns 0 .. C-1 of each row used (C % 8 == 0, ld % 8 == 0, ld >= C);
+ * row (t, h) belongs to sequence position t + initial_row.  All C columns of p16 are written
+ * (zeros at the masked ones). */
+int cacti_hip_row_causal_softmax_fwd(int64_t T, int64_t H, int64_t C, int64_t ld, int64_t initial_row,
+                                     const void *s16, void *p16, void *stream);
+/* in_tok[pos] += out_tok[last] (u16): the token generated for the last position appended to the
+ * input sequence on the device, src/librarium/llama.rs:958-959. */
+int cacti_hip_append_token_u16(void *in_tok, int64_t pos, const void *out_tok, int64_t last, void *stream);
+
 /* LM loss, src/librarium/llama.rs:541-546 on logit16 [N,V] f16, tok [N] u16:
  * prob [N,V] f32 = softmax(f32(logit)) (InnerSoftmax), loss [N] f32
  * (InnerSoftmaxCategoricalNLLFutThunkSpec op.rs:3460-3569), amax [N] u16

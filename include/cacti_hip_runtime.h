@@ -151,6 +151,26 @@ int cacti_cell_matcher_match(const char *const *keys, int nkeys, const char *con
  * another dtype CACTI_E_NOTIMPL.  Parameters without a match keep their value; *n_matched counts the
  * matched ones. */
 int cacti_llama_load_tensors_dir(cacti_llama *model, cacti_tensors_dir *dir, int *n_matched);
+/* ---- KV-cached forward pass: LlamaCached, src/librarium/llama.rs:561-963 (batch 1, q_group 1).
+ * cached_create shares the model's parameters and position tables (LlamaCached::from(Llama) /
+ * from_train, llama.rs:618-686) and adds zeroed k / v caches [seq_cap, H, Dh] per layer and an
+ * input token cell [seq_cap] (u16, zeros = pad); seq_cap % 8 == 0, seq_cap <= the model's S.
+ * reset_state zeroes the caches (llama.rs:784-789).  set_tokens writes the first n input tokens
+ * and pads the rest with 0 (the example's resume_put_mem_with, open_llama_3b_deploy.rs:221-231).
+ * apply runs positions prev .. next-1 (llama.rs:805-963): embeds in_tok[prev .. next], adds the new
+ * keys and values to the caches, attends over the cache with the row-causal mask, and keeps logit
+ * [T,V] f16, tok [T] u16 (arg max) and, if asked, prob [T,V] f32 for the T = next - prev rows; the
+ * token generated for the last row is added to in_tok[next] when next < seq_cap.  It returns with
+ * the work queued on the context's stream.  outputs copies what the last apply kept (any pointer
+ * may be NULL) and synchronises; a token id >= V is reported there as CACTI_E_INDEX. */
+typedef struct cacti_llama_cached cacti_llama_cached;
+int cacti_llama_cached_create(cacti_llama *model, int64_t seq_cap, cacti_llama_cached **cached);
+int cacti_llama_cached_destroy(cacti_llama_cached *cached);
+int cacti_llama_cached_reset_state(cacti_llama_cached *cached);
+int cacti_llama_cached_set_tokens(cacti_llama_cached *cached, const uint16_t *tok, int64_t n);
+int cacti_llama_cached_get_tokens(cacti_llama_cached *cached, uint16_t *tok);
+int cacti_llama_cached_apply(cacti_llama_cached *cached, int64_t prev, int64_t next, int want_prob);
+int cacti_llama_cached_outputs(cacti_llama_cached *cached, void *logit_f16, float *prob, uint16_t *tok);
 /* cells of the inputs (tok u16 [S], lm_tok u16 [S], loss_scale f32 [S]) and of the kept
  * outputs of the last staged cycle (logit f16 [S,V], loss f32 [S], amax u16 [S],
  * prob f32 [S,V] or 0) */

@@ -976,6 +976,95 @@ ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const ui
     return 0;
 }
 
+/* ------------------------------------------------------------------------- */
+/* KV-cached forward pass: LlamaCached::apply, src/librarium/llama.rs:805-963,   */
+/* batch 1, q_group 1, no param_scale.                                          */
+
+/* RowCausalAttentionMaskFutThunkSpec, src/librarium/llama.rs:1052-1112, on [1,T,H,C] f32:
+ * if (row_idx + initial_row) >= col_idx then u else -inf */
+ORACLE_API void th_row_causal_mask_f32(i64 T, i64 H, i64 C, i64 initial_row, const float *x, float *y)
+{
+    for (i64 t = 0; t < T; t++)
+        for (i64 h = 0; h < H; h++)
+            for (i64 j = 0; j < C; j++) {
+                const i64 i = (t * H + h) * C + j;
+                y[i] = (t + initial_row) >= j ? x[i] : -INFINITY;
+            }
+}
+
+/* One chunk of positions prev .. next-1.  k_cache, v_cache: [L][cap,H,Dh] f16, updated in place
+ * (`+=` of the new rows); in_tok: [cap] u16, in_tok[next] += the token generated for position
+ * next-1 when next < cap (the reference's slice would be out of range otherwise).  Outputs for the
+ * T = next - prev rows: logit [T,V] f16, prob [T,V] f32 (may be NULL), out_tok [T] u16.
+ * Returns 0, or 1 + row for a token id out of range. */
+ORACLE_API i64 oracle_llama_cached_apply(const oracle_cfg *c, const h16 *param, h16 *k_cache, h16 *v_cache,
+                                         uint16_t *in_tok, i64 prev, i64 next, h16 *logit_out, float *prob_out,
+                                         uint16_t *tok_out)
+{
+    const i64 cap = c->S, D = c->D, H = c->H, Dh = c->Dh, F = c->F, V = c->V, L = c->L;
+    const i64 T = next - prev;
+    const float alpha = 1.0f / sqrtf((float)Dh);
+    if (H * Dh != D || prev < 0 || T <= 0 || next > cap) return -1;
+    const h16 *embed = param;
+    const h16 *layers = param + V * D;
+    const i64 lsz = oracle_layer_elems(c);
+    const h16 *head_norm = layers + L * lsz;
+    const h16 *lm_head = head_norm + D;
+    h16 *cos16 = halloc(cap * Dh), *sin16 = halloc(cap * Dh);
+    oracle_rope_tables(cap, Dh, cos16, sin16);
+    const h16 *cosr = cos16 + prev * Dh, *sinr = sin16 + prev * Dh;        /* rows prev .. next-1 */
+
+    h16 *stream = halloc(T * D);
+    i64 rc = th_outer_select_f16(V, D, embed, T, in_tok + prev, stream);
+    if (rc) return rc;
+    float *tsave = falloc(T * D), *ssave = falloc(T);
+    h16 *pre = halloc(T * D), *q = halloc(T * D), *k = halloc(T * D), *v = halloc(T * D), *qr = halloc(T * D),
+        *kr = halloc(T * D), *attn = halloc(T * D), *o = halloc(T * D), *x1 = halloc(T * D), *post = halloc(T * D),
+        *up = halloc(T * F), *gate = halloc(T * F), *y = halloc(T * F), *hh = halloc(T * F), *down = halloc(T * D);
+    h16 *s16 = halloc(T * H * cap), *p16 = halloc(T * H * cap);
+    float *s32 = falloc(T * H * cap), *m32 = falloc(T * H * cap);
+    for (i64 l = 0; l < L; l++) {
+        const h16 *P = layers + l * lsz;
+        const h16 *w_pre = P, *wq = P + D, *wk = wq + D * D, *wv = wk + D * D, *wo = wv + D * D;
+        const h16 *w_post = wo + D * D, *wg = w_post + D, *wu = wg + F * D, *wd = wu + F * D;
+        h16 *kc = k_cache + l * cap * D, *vc = v_cache + l * cap * D;
+        oracle_rmsnorm_fwd(T, D, stream, w_pre, c->eps, pre, tsave, ssave);
+        th_matmul_f16(0, 1, T, D, D, 1.0f, pre, D, wq, D, 0.0f, q, D);
+        oracle_rope_fwd(T, H, Dh, q, cosr, sinr, qr);
+        th_matmul_f16(0, 1, T, D, D, 1.0f, pre, D, wk, D, 0.0f, k, D);
+        oracle_rope_fwd(T, H, Dh, k, cosr, sinr, kr);
+        th_add_f16(T * D, kc + prev * D, kr, kc + prev * D);                 /* k_cache[prev..next] += k */
+        th_matmul_f16(0, 1, T, D, D, 1.0f, pre, D, wv, D, 0.0f, v, D);
+        th_add_f16(T * D, vc + prev * D, v, vc + prev * D);                  /* v_cache[prev..next] += v */
+        /* scores against the whole cache (all cap rows), mask, softmax, P V */
+        th_block_matmul_f16(0, 1, H, T, cap, Dh, alpha, qr, D, Dh, kc, D, Dh, 0.0f, s16, H * cap, cap);
+        th_cast_f16_f32(T * H * cap, s16, s32);
+        th_row_causal_mask_f32(T, H, cap, prev, s32, m32);
+        th_softmax_f32(T * H, cap, m32, s32);
+        th_cast_f32_f16(T * H * cap, s32, p16);
+        th_block_matmul_f16(0, 0, H, T, Dh, cap, 1.0f, p16, H * cap, cap, vc, D, Dh, 0.0f, attn, D, Dh);
+        th_matmul_f16(0, 1, T, D, D, 1.0f, attn, D, wo, D, 0.0f, o, D);
+        th_add_f16(T * D, stream, o, x1);
+        oracle_rmsnorm_fwd(T, D, x1, w_post, c->eps, post, tsave, ssave);
+        th_matmul_f16(0, 1, T, F, D, 1.0f, post, D, wu, D, 0.0f, up, F);
+        th_matmul_f16(0, 1, T, F, D, 1.0f, post, D, wg, D, 0.0f, gate, F);
+        oracle_silu_gate_fwd(T * F, gate, up, y, hh);
+        th_matmul_f16(0, 1, T, D, F, 1.0f, hh, F, wd, F, 0.0f, down, D);
+        th_add_f16(T * D, x1, down, stream);
+    }
+    h16 *hn = halloc(T * D), *logit = halloc(T * V);
+    oracle_rmsnorm_fwd(T, D, stream, head_norm, c->eps, hn, tsave, ssave);
+    th_matmul_f16(0, 1, T, V, D, 1.0f, hn, D, lm_head, D, 0.0f, logit, V);
+    /* out_lm_prob = softmax(f32(logit)); out_lm_tok = u16(argmax(logit)) */
+    rc = oracle_softmax_ce_fwd(T, V, logit, NULL, prob_out, NULL, tok_out);
+    if (logit_out) memcpy(logit_out, logit, (size_t)(T * V) * 2);
+    if (next < cap) in_tok[next] = (uint16_t)(in_tok[next] + tok_out[T - 1]);
+    free(cos16); free(sin16); free(stream); free(tsave); free(ssave); free(pre); free(q); free(k); free(v);
+    free(qr); free(kr); free(attn); free(o); free(x1); free(post); free(up); free(gate); free(y); free(hh);
+    free(down); free(s16); free(p16); free(s32); free(m32); free(hn); free(logit);
+    return rc;
+}
+
 /* ---------------------------------------------------------------------------
  * Numerical-health digests over f16 tensors (integer-exact).
  * NanCountFutThunkSpec, src/thunk/op.rs:273-349: elements whose exponent field is all ones and

@@ -433,3 +433,28 @@ def read_safetensors_header(path):
         out[name] = (e["dtype"], tuple(e["shape"]), (8 + n + b, 8 + n + e_))
     return out
 
+
+# ---------------------------------------------------------------- KV-cached forward pass
+def llama_cached_state(cfg):
+    """Zeroed k / v caches [L, cap, H*Dh] f16 (LlamaCached::init_state, src/librarium/llama.rs:762-782)."""
+    shape = (cfg.L, cfg.S, cfg.D)
+    return np.zeros(shape, np.float16), np.zeros(shape, np.float16)
+
+
+def llama_cached_apply(cfg, param, k_cache, v_cache, in_tok, prev, next_, want_prob=False):
+    """LlamaCached::apply (src/librarium/llama.rs:805-963) for positions prev .. next_-1; cfg.S is the
+    sequence capacity.  Updates k_cache, v_cache and in_tok (the generated token is appended) in
+    place; returns dict(logit [T,V] f16, tok [T] u16, prob [T,V] f32 or None)."""
+    T = next_ - prev
+    assert param.dtype == np.float16 and in_tok.dtype == np.uint16 and in_tok.size == cfg.S
+    assert k_cache.flags["C_CONTIGUOUS"] and v_cache.flags["C_CONTIGUOUS"]
+    logit = np.empty((T, cfg.V), np.float16)
+    prob = np.empty((T, cfg.V), np.float32) if want_prob else None
+    tok = np.empty((T,), np.uint16)
+    lib().oracle_llama_cached_apply.restype = i64
+    rc = lib().oracle_llama_cached_apply(C.byref(cfg), P(param), P(k_cache), P(v_cache), P(in_tok), i64(prev),
+                                         i64(next_), P(logit), P(prob), P(tok))
+    if rc:
+        raise ValueError("oracle_llama_cached_apply: status %d" % rc)
+    return dict(logit=logit, tok=tok, prob=prob)
+

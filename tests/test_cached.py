@@ -1,0 +1,263 @@
+"""KV-cached forward pass (LlamaCached::apply, src/librarium/llama.rs:805-963; the row-causal mask,
+src/librarium/llama.rs:1052-1112).
+
+CPU: the oracle's cached pass is pinned against the oracle's own full forward pass, which other tests
+pin: one call over the whole sequence reproduces its logits bit for bit (same thunks; the row-causal
+mask with initial row 0 is the causal mask), and any split into chunks reproduces the one-call result
+bit for bit (rows of a product do not depend on how many rows are computed with them), which fixes the
+offsets of the cache rows, of the position tables and of the mask.  GPU: the HIP pass against the
+oracle, chunk by chunk."""
+import numpy as np
+import pytest
+
+from tests.util import assert_parity, rng
+
+
+def _inputs(seed=4):
+    from tests.test_gpu_llama import TINY, make_inputs
+    return make_inputs(TINY, seed=seed, norm_mean=1.0, grad_scale=1024.0)
+
+
+def test_oracle_cached_pass_equals_the_full_forward_pass(oracle):
+    cfg, flat, tok, lm_tok, scale = _inputs()
+    ref = oracle.llama_step(cfg, flat, tok, lm_tok, scale, want_grad=False)
+    kc, vc = oracle.llama_cached_state(cfg)
+    full = oracle.llama_cached_apply(cfg, flat, kc, vc, tok.copy(), 0, cfg.S, want_prob=True)
+    assert np.array_equal(full["logit"].view(np.uint16), ref["logit"].view(np.uint16))
+    assert np.array_equal(full["tok"], ref["amax"])
+    assert np.allclose(full["prob"].sum(axis=1), 1.0, atol=1e-5)
+    assert np.array_equal(full["prob"].argmax(axis=1), full["tok"])
+    # the caches hold every position's rotated keys and plain values
+    assert np.mean(kc != 0) > 0.99 and np.mean(vc != 0) > 0.99
+    # chunks of any size, including single rows, give the same bits and the same caches
+    kc2, vc2 = oracle.llama_cached_state(cfg)
+    cuts = [0, 5, 6, 7, 40, cfg.S - 3, cfg.S]
+    parts = []
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        it = tok.copy()
+        out = oracle.llama_cached_apply(cfg, flat, kc2, vc2, it, a, b)
+        parts.append(out["logit"])
+        if b < cfg.S:                                     # the generated token is added to the next input slot
+            assert it[b] == (int(tok[b]) + int(out["tok"][-1])) % 65536
+            assert np.array_equal(np.delete(it, b), np.delete(tok, b))
+    assert np.array_equal(np.concatenate(parts).view(np.uint16), full["logit"].view(np.uint16))
+    assert np.array_equal(kc, kc2) and np.array_equal(vc, vc2)
+    # rows beyond `next` of a partly filled cache stay zero
+    kc3, vc3 = oracle.llama_cached_state(cfg)
+    oracle.llama_cached_apply(cfg, flat, kc3, vc3, tok.copy(), 0, 9)
+    assert np.all(kc3[:, 9:] == 0) and np.all(vc3[:, 9:] == 0) and np.array_equal(kc3[:, :9], kc[:, :9])
+
+
+def test_oracle_row_causal_mask(oracle):
+    import ctypes as C
+    T, H, Cc = 3, 2, 7
+    x = np.arange(T * H * Cc, dtype=np.float32).reshape(T, H, Cc) + 1
+    for row0 in (0, 2, 6, 100):
+        y = np.empty_like(x)
+        oracle.lib().th_row_causal_mask_f32(oracle.i64(T), oracle.i64(H), oracle.i64(Cc), oracle.i64(row0), oracle.P(x), oracle.P(y))
+        for t in range(T):
+            live = min(Cc, t + row0 + 1)
+            assert np.array_equal(y[t, :, :live], x[t, :, :live]) and np.all(np.isneginf(y[t, :, live:]))
+
+
+# ------------------------------------------------------------------------------------------ GPU
+def _row_softmax_oracle(oracle, s16, row0):
+    T, H, Cc = s16.shape
+    s32 = s16.astype(np.float32)
+    m = np.empty_like(s32)
+    oracle.lib().th_row_causal_mask_f32(oracle.i64(T), oracle.i64(H), oracle.i64(Cc), oracle.i64(row0), oracle.P(s32), oracle.P(m))
+    p = np.empty_like(s32)
+    oracle.lib().th_softmax_f32(oracle.i64(T * H), oracle.i64(Cc), oracle.P(m), oracle.P(p))
+    return oracle.cast_f32_f16(p)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,H,Cc,row0", [(1, 4, 8, 0), (1, 32, 2048, 2047), (1, 32, 1032, 1024), (5, 3, 520, 100),
+                                         (64, 4, 64, 0), (3, 2, 16, 40)])
+def test_row_causal_softmax_matches_the_oracle(oracle, T, H, Cc, row0):
+    import torch
+    from cacti_amd import ffi
+    print("row causal softmax", T, H, Cc, row0, flush=True)
+    r = rng(T + H + Cc + row0)
+    s16 = (r.standard_normal((T, H, Cc)) * 3).astype(np.float16)
+    want = _row_softmax_oracle(oracle, s16, row0)
+    d = torch.from_numpy(s16.view(np.int16)).cuda()
+    out = torch.full_like(d, 0x7e00)                       # NaN patterns: every column must be written
+    ffi.call("cacti_hip_row_causal_softmax_fwd", T, H, Cc, Cc, row0, d.data_ptr(), out.data_ptr(), None)
+    got = out.cpu().numpy().view(np.float16)
+    assert_parity(got, want, "row causal softmax")
+    live = np.arange(Cc)[None, :] <= (np.arange(T)[:, None] + row0)
+    assert np.all(got[~np.broadcast_to(live[:, None, :], got.shape)] == 0)
+    assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.99
+    # in place
+    ffi.call("cacti_hip_row_causal_softmax_fwd", T, H, Cc, Cc, row0, d.data_ptr(), d.data_ptr(), None)
+    assert np.array_equal(d.cpu().numpy(), out.cpu().numpy())
+
+
+def _gpu_model(cfg, flat):
+    from tests.test_gpu_llama import _model
+    ctx, m = _model(cfg)
+    m.put_params_flat(flat)
+    return ctx, m
+
+
+@pytest.mark.gpu
+def test_cached_pass_matches_the_oracle_chunk_by_chunk(oracle):
+    """Teacher-forced input: a prompt chunk, single tokens, a mid-sized chunk, the rest; logits,
+    probabilities and arg-max tokens of every chunk against the oracle's cached pass."""
+    from cacti_amd.runtime import LlamaCached
+    cfg, flat, tok, lm_tok, scale = _inputs(seed=5)
+    ctx, m = _gpu_model(cfg, flat)
+    k = LlamaCached(m, cfg.S)
+    kc, vc = oracle.llama_cached_state(cfg)
+    cuts = [0, 13, 14, 15, 16, 48, 51, cfg.S]
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        print("cached chunk", a, b, flush=True)
+        k.set_tokens(tok)
+        k.apply(a, b, want_prob=True)
+        got = k.outputs()
+        it = tok.copy()
+        want = oracle.llama_cached_apply(cfg, flat, kc, vc, it, a, b, want_prob=True)
+        assert_parity(got["logit"], want["logit"], "logit %d:%d" % (a, b))
+        assert np.abs(got["prob"] - want["prob"]).max() < 2e-3 and np.allclose(got["prob"].sum(axis=1), 1, atol=1e-4)
+        top2 = np.sort(want["logit"].astype(np.float32), axis=1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 0.02
+        assert np.array_equal(got["tok"][clear], want["tok"][clear]) and clear.mean() > 0.5
+        assert np.array_equal(got["tok"], got["logit"].astype(np.float32).argmax(axis=1))
+        if b < cfg.S:                                     # the appended token
+            toks = k.tokens()
+            assert toks[b] == (int(tok[b]) + int(got["tok"][-1])) % 65536
+            assert np.array_equal(np.delete(toks, b), np.delete(tok, b))
+    k.close(); m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_cached_pass_in_one_call_matches_the_training_forward_pass(oracle):
+    from cacti_amd.runtime import LlamaCached
+    cfg, flat, tok, lm_tok, scale = _inputs(seed=6)
+    ctx, m = _gpu_model(cfg, flat)
+    m.step(tok, lm_tok, scale, want_grad=False)
+    io = m.io_cells()
+    ref = ctx.cell_get(io["logit"], np.float16, (cfg.S, cfg.V))
+    k = LlamaCached(m, cfg.S)
+    k.set_tokens(tok)
+    k.apply(0, cfg.S)
+    got = k.outputs()["logit"]
+    assert_parity(got, ref, "cached vs training forward")
+    assert np.mean(got.view(np.uint16) == ref.view(np.uint16)) > 0.95
+    k.close(); m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_greedy_generation_feeds_its_own_tokens(oracle):
+    """The deploy loop (examples/open_llama_3b_deploy.rs:195-206): prompt, then one position per
+    cycle; every cycle's input token is the previous cycle's arg max (asserted by the example), the
+    cache is reset between two runs, and the run matches the oracle's while its arg max is clear."""
+    from cacti_amd.runtime import LlamaCached
+    cfg, flat, tok, lm_tok, scale = _inputs(seed=7)
+    ctx, m = _gpu_model(cfg, flat)
+    k = LlamaCached(m, cfg.S)
+    P, n_new = 9, 12
+    runs = []
+    for _ in range(2):
+        k.reset_state()
+        k.set_tokens(tok[:P])
+        k.apply(0, P)
+        outs = [int(k.outputs(want_logit=False)["tok"][-1])]
+        for i in range(1, n_new):
+            k.apply(P + i - 1, P + i)
+            outs.append(int(k.outputs(want_logit=False)["tok"][0]))
+        toks = k.tokens()
+        assert np.array_equal(toks[:P], tok[:P]) and list(toks[P:P + n_new]) == outs and np.all(toks[P + n_new:] == 0)
+        runs.append(outs)
+    assert runs[0] == runs[1]
+    kc, vc = oracle.llama_cached_state(cfg)
+    it = np.zeros(cfg.S, np.uint16)
+    it[:P] = tok[:P]
+    a, b = 0, P
+    for i in range(n_new):
+        want = oracle.llama_cached_apply(cfg, flat, kc, vc, it, a, b)
+        top2 = np.sort(want["logit"][-1].astype(np.float32))[-2:]
+        if top2[1] - top2[0] < 0.02 or int(want["tok"][-1]) != runs[0][i]:
+            assert top2[1] - top2[0] < 0.02, (i, want["tok"][-1], runs[0][i])
+            break
+        a, b = b, b + 1
+    assert i >= 2
+    k.close(); m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_cached_pass_error_paths(oracle):
+    from cacti_amd.ffi import CactiError
+    from cacti_amd.runtime import LlamaCached
+    cfg, flat, tok, lm_tok, scale = _inputs(seed=5)
+    ctx, m = _gpu_model(cfg, flat)
+    for bad_cap in (cfg.S + 8, 12, 0):
+        with pytest.raises(CactiError) as e:
+            LlamaCached(m, bad_cap)
+        assert e.value.code == -1
+    k = LlamaCached(m, 64)                                 # a capacity below the model's
+    with pytest.raises(CactiError) as e:
+        k.outputs()
+    assert e.value.code == -5
+    for a, b in ((0, 65), (-1, 3), (5, 5), (7, 3)):
+        with pytest.raises(CactiError) as e:
+            k.apply(a, b)
+        assert e.value.code == -1, (a, b)
+    with pytest.raises(CactiError) as e:
+        k.set_tokens(np.zeros(65, np.uint16))
+    assert e.value.code == -1
+    bad = tok[:64].copy()
+    bad[3] = cfg.V                                        # token id out of range: reported at the next sync
+    k.set_tokens(bad)
+    k.apply(0, 8)
+    with pytest.raises(CactiError) as e:
+        k.outputs()
+    assert e.value.code == -3
+    k.set_tokens(tok[:64])
+    k.reset_state()
+    k.apply(0, 64)                                         # next == capacity: nothing is appended
+    out = k.outputs()
+    assert np.array_equal(k.tokens(), tok[:64]) and np.isfinite(out["logit"].astype(np.float32)).all()
+    k.close(); m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_full_size_decode_agrees_with_one_call_over_the_same_tokens():
+    """3B shapes (hidden 3200, 32 heads x 100, ffn 8640, vocabulary 32000), 2 layers, capacity 2048,
+    no oracle run: a 515-token sequence processed as prompt + three single-token cycles (the
+    streaming product kernels and the attention over the cache at one row) gives the logits of one
+    call over all 515 positions (the tiled kernels) up to summation order (the bar between two
+    device paths is wider than against the oracle: both carry their own rounding)."""
+    from cacti_amd.runtime import Ctx, Llama, LlamaCached
+    cfg = dict(S=2048, D=3200, H=32, Dh=100, F=8640, V=32000, L=2)
+    ctx = Ctx(0, 0, True)
+    m = Llama(ctx, **cfg)
+    r = np.random.default_rng(0)
+    for i, (name, shp) in enumerate(m.params):
+        w = r.standard_normal(shp, dtype=np.float32) * 0.02
+        if name.endswith("norm"):
+            w += 1.0
+        m.put_param(i, w.astype(np.float16))
+    tok = r.integers(0, cfg["V"], 515).astype(np.uint16)
+    k = LlamaCached(m, 2048)
+    k.set_tokens(tok)
+    k.apply(0, 515)
+    ref = k.outputs()["logit"]
+    k.reset_state()
+    k.set_tokens(tok)
+    k.apply(0, 512)
+    head = k.outputs()["logit"]
+    rows = [head]
+    for p in (512, 513, 514):
+        print("decode position", p, flush=True)
+        k.set_tokens(tok)
+        k.apply(p, p + 1)
+        rows.append(k.outputs()["logit"])
+    got = np.concatenate(rows)
+    assert np.isfinite(ref.astype(np.float32)).all()
+    assert_parity(got[:512], ref[:512], "prefill rows")
+    # two summation orders of the same fp32 products, each rounded to f16 after every thunk: the
+    # distance between them is twice the distance of either from exact arithmetic
+    assert_parity(got[512:], ref[512:], "decoded rows", l2=3e-3, mx=6e-2)
+    k.close(); m.close(); ctx.close()

@@ -309,6 +309,26 @@ def test_gemm_direct_load_kernels(ops, oracle, ta, tb, M, N, K):
         assert exact_frac(got, want) > 0.98
 
 
+# one to four rows against a weight matrix (decoding): the streaming kernel, including a row count
+# of columns that is not a multiple of its 4 rows per workgroup, a short K, and a padded weight matrix
+SKINNY_SHAPES = [(1, 3200, 3200, 0), (2, 8640, 3200, 0), (3, 3200, 8640, 8), (4, 1000, 136, 0), (1, 32000, 3200, 0),
+                 (4, 24, 136, 16)]
+
+
+@pytest.mark.parametrize("M,N,K,pad", SKINNY_SHAPES)
+def test_gemm_few_rows_streams_the_weights(ops, oracle, M, N, K, pad):
+    say("gemm skinny", M, N, K, pad)
+    r = rng(400 + M + N + K)
+    A = randn16(r, (M, K))
+    Bp = randn16(r, (N, K + pad), 0.05)
+    B = Bp[:, :K]
+    for alpha in (1.0, 0.125):
+        want = oracle.matmul(0, 1, A, np.ascontiguousarray(B), alpha, 0.0, None)
+        got = host(ops.gemm(dev(A), dev(Bp)[:, :K], False, True, alpha, 0.0))
+        assert_parity(got, want, "gemm skinny")
+        assert exact_frac(got, want) > 0.98
+
+
 @pytest.mark.parametrize("case", ["fwd", "dgrad", "wgrad"])
 def test_gemm_projection_shapes(ops, oracle, case):
     """The three GEMMs of one projection at a reduced token count (oracle finishes in seconds)."""
