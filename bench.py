@@ -622,6 +622,94 @@ def run_ingest(args):
     return out
 
 
+def run_decode(args):
+    """Single-stream greedy decoding with the key / value cache (examples/open_llama_3b_deploy.rs:195-206):
+    a prompt of 1024 positions in one call, then one position per call, each feeding the previous
+    call's arg max.  value = generated tokens per second over the timed single-position calls (each
+    returns queued; one synchronisation at the end).  A position streams every weight matrix once
+    (6.65 GB: all parameters but the embedding, of which one row is read) plus the cached keys and
+    values of the positions before it."""
+    import torch
+    from cacti_amd.runtime import Ctx, Llama, LlamaCached
+    cfg = dict(LLAMA_3B)
+    if args.layers is not None:
+        cfg["L"] = args.layers
+    prompt = 1024
+    steps = max(args.steps, 32)
+    ctx = Ctx(0, 0, True)
+    model = Llama(ctx, **cfg)
+    synth_params(model)
+    tok, _, _ = synth_inputs(cfg)
+    k = LlamaCached(model, cfg["S"])
+    k.set_tokens(tok[:prompt])
+    k.apply(0, prompt)
+    ctx.sync()
+    t0 = time.perf_counter()
+    k.reset_state()
+    k.set_tokens(tok[:prompt])
+    k.apply(0, prompt)
+    ctx.sync()
+    prefill = time.perf_counter() - t0
+    pos = prompt
+    for _ in range(max(args.warmup, 2)):
+        k.apply(pos, pos + 1)
+        pos += 1
+    ctx.sync()
+    torch.cuda.synchronize()
+    first = pos
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        k.apply(pos, pos + 1)
+        pos += 1
+    ctx.sync()
+    dt = (time.perf_counter() - t0) / steps
+    toks = k.tokens()
+    last = k.outputs(want_logit=False)["tok"]
+    assert toks[pos] == last[0] and np.all(toks[pos + 1:] == 0) and np.array_equal(toks[:prompt], tok[:prompt])
+    D, F, V, L = cfg["D"], cfg["F"], cfg["V"], cfg["L"]
+    wbytes = 2 * (L * (4 * D * D + 3 * F * D + 2 * D) + D + V * D)
+    ctx_mid = first + steps / 2.0
+    kvbytes = 2 * 2 * L * ctx_mid * D
+    out = {"metric": "greedy decoding tokens/sec with the key / value cache, 1 sequence", "value": 1.0 / dt,
+           "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": max(args.warmup, 2), "ms_per_step": dt * 1e3,
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+           "data": "synthetic (seeded N(0,0.02) weights, uniform prompt ids)",
+           "config": {"workload": "OpenLLaMA-3B shapes, %d layers, prompt %d positions then %d single positions "
+                                  "(context %d .. %d), capacity %d" % (L, prompt, steps, first, pos, cfg["S"]),
+                      "prefill_ms": prefill * 1e3, "prefill_tokens_per_s": prompt / prefill},
+           "roofline": {"bound": "hbm", "achieved": (wbytes + kvbytes) / dt / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": (wbytes + kvbytes) / dt / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "note": "whole position: %.2f GB of weights + %.2f GB of cached keys and values over the "
+                                "wall time of a call (about 15 launches per layer); per-kernel figures are in "
+                                "profiles/" % (wbytes / 1e9, kvbytes / 1e9)}}
+    k.close()
+    model.close()
+    ctx.close()
+    if not args.no_cpu_baseline:
+        from oracle import oracle as o
+        from tests.llama_ref import make_inputs
+        times = {}
+        for Lc in (0, 2):
+            ocfg, flat, otok, _, _ = make_inputs(dict(cfg, L=Lc), seed=0, norm_mean=1.0, grad_scale=1024.0)
+            kc, vc = o.llama_cached_state(ocfg)
+            it = np.zeros(ocfg.S, np.uint16)
+            it[:8] = otok[:8]
+            o.llama_cached_apply(ocfg, flat, kc, vc, it, 0, 8)
+            t0 = time.time()
+            for p in range(8, 12):
+                o.llama_cached_apply(ocfg, flat, kc, vc, it, p, p + 1)
+            times[Lc] = (time.time() - t0) / 4
+        layer = max(times[2] - times[0], 1e-9) / 2
+        full = times[0] + cfg["L"] * layer
+        out["cpu_baseline"] = {"value": 1.0 / full, "unit": "tokens/s", "cores": o.num_threads(), "kind": "port",
+                               "sample": "oracle cached pass, one position per call at full shapes: LM head alone (%.3f s) "
+                                         "and with 2 layers (%.3f s per layer), extrapolated to %d layers"
+                                         % (times[0], layer, cfg["L"])}
+    else:
+        out["cpu_baseline"] = None
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -631,7 +719,7 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest", "decode"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -647,6 +735,8 @@ def main():
         out = run_adamw(args)
     elif args.workload == "ingest":
         out = run_ingest(args)
+    elif args.workload == "decode":
+        out = run_decode(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)

@@ -1,12 +1,21 @@
-// C[M,N] = f16(alpha * A[M,K] B[N,K]^T) for M <= 4 rows (decoding: one or a few tokens against a
-// weight matrix).  The product is a stream over B: every byte of the weights is read once and
+// C[M,N] = f16(alpha * A[M,K] B[N,K]^T) for M <= 4 rows (decoding: one or a few positions against
+// a weight matrix).  The product is a stream over B: every byte of the weights is read once and
 // used M times, so the kernel is built for HBM, not for the matrix cores.
 //
 // A workgroup of 256 lanes owns R = 4 rows of B (4 output columns) and splits K over its lanes
-// in 16-byte pieces; each lane issues its 4 row loads together, accumulates M x 4 fp32 sums, and
-// the sums are reduced over the wave (cross-lane adds) and over the 4 waves (LDS).  N / 4
-// workgroups: 800 for N = 3200, 8 resident per CU, i.e. some 200 KiB of weight loads in flight
-// per CU.  A (a few KiB) is re-read from L2 by every workgroup.
+// in 16-byte pieces; a lane issues the loads of 2 or 4 pieces x 4 rows before it uses the first,
+// accumulates M x 4 fp32 sums with v_dot2_f32_f16 (the scalar form, 3 instructions per product
+// with the conversions, made the kernel compute-bound), and the sums are reduced over the wave (cross-lane adds) and
+// over the 4 waves (LDS).  N / 4 workgroups: 800 for N = 3200, 8 resident per CU.  A (a few KiB)
+// is re-read from L2 by every workgroup.
+//
+// Two fusions keep a decoding step from paying a launch for every small thunk:
+//  * NORM: A is not read but formed per workgroup as the RMSNorm of a row x (optionally of the
+//    residual sum f16(x + x2), which workgroup 0 also writes out): the lanes' own pieces of the
+//    row give the sum of squares (every piece of the row belongs to exactly one lane), one
+//    workgroup reduction, then a = f16(w * (x * rinv)) exactly as the RMSNorm kernel rounds it.
+//  * GATE: two weight matrices share the rows (gate and up projection); the epilogue stores
+//    f16(f16(silu(g)) * u) of the two rounded products, as the SiLU-gate kernel computes it.
 #include "gemm_internal.h"
 
 namespace cacti {
@@ -15,57 +24,200 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kRows = 4;
+constexpr int kMaxPre = 4;                 // pieces of K per lane whose loads are in flight together (2 or 4)
 
-template <int M>
-__global__ void __launch_bounds__(kThreads)
-gemm_skinny_nt_kernel(int64_t N, int64_t K, float alpha, const half_t *__restrict__ A, int64_t lda,
-                      const half_t *__restrict__ B, int64_t ldb, half_t *__restrict__ C, int64_t ldc)
+struct SkinnyArgs {
+    int64_t N, K;
+    float alpha;
+    const half_t *A;         // [M, lda] (plain) or the row source x (NORM)
+    int64_t lda;
+    const half_t *x2;        // NORM: optional second summand of the row
+    const half_t *w;         // NORM: norm weights [K]
+    float eps;
+    half_t *sum_out;         // NORM with x2: the residual sum [M, lda], written by workgroup 0
+    const half_t *B;         // [N, ldb]
+    const half_t *B2;        // GATE: the second weight matrix [N, ldb]
+    int64_t ldb;
+    half_t *C;
+    int64_t ldc;
+};
+
+__device__ __forceinline__ float block_sum(float v, float *scratch)
 {
-    __shared__ float part[kThreads / 64][M * kRows];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) scratch[wid] = v;
+    __syncthreads();
+    float r = scratch[0];
+#pragma unroll
+    for (int w = 1; w < kThreads / 64; w++) r += scratch[w];
+    return r;
+}
+
+// sum of 8 products, fp32 accumulate: four v_dot2_f32_f16 (no conversions, two products each)
+__device__ __forceinline__ float dot8(const half8_t &a, const half8_t &b, float acc)
+{
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const half2_t a2 = {a[2 * i], a[2 * i + 1]}, b2 = {b[2 * i], b[2 * i + 1]};
+        acc = __builtin_amdgcn_fdot2(a2, b2, acc, false);
+    }
+    return acc;
+}
+
+template <int M, bool NORM, bool GATE, int kPre>
+__global__ void __launch_bounds__(kThreads)
+gemm_skinny_nt_kernel(SkinnyArgs p)
+{
+    constexpr int NB = GATE ? 2 : 1;
+    __shared__ float part[kThreads / 64][NB * M * kRows];
+    __shared__ float scratch[kThreads / 64];
     const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
     const int64_t n0 = (int64_t)blockIdx.x * kRows;
-    float acc[M][kRows];
+    float acc[NB][M][kRows];
 #pragma unroll
-    for (int m = 0; m < M; m++)
-#pragma unroll
-        for (int r = 0; r < kRows; r++) acc[m][r] = 0.f;
-    // rows past N re-read the last row (their sums are dropped)
-    const half_t *brow[kRows];
-#pragma unroll
-    for (int r = 0; r < kRows; r++) brow[r] = B + (n0 + r < N ? n0 + r : N - 1) * ldb;
-    const int64_t chunks = K / 8;
-    for (int64_t c = tid; c < chunks; c += kThreads) {
-        half8_t b[kRows];
-        h8 a[M];
-#pragma unroll
-        for (int r = 0; r < kRows; r++)
-            b[r] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(brow[r]) + c);
-#pragma unroll
-        for (int m = 0; m < M; m++) a[m] = ld8(A + m * lda + c * 8);
+    for (int b = 0; b < NB; b++)
 #pragma unroll
         for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int r = 0; r < kRows; r++)
+            for (int r = 0; r < kRows; r++) acc[b][m][r] = 0.f;
+    // rows past N re-read the last row (their sums are dropped)
+    const half_t *brow[NB][kRows];
 #pragma unroll
-                for (int k = 0; k < 8; k++) acc[m][r] += h2f(a[m].v[k]) * h2f(b[r][k]);
+    for (int r = 0; r < kRows; r++) {
+        const int64_t n = n0 + r < p.N ? n0 + r : p.N - 1;
+        brow[0][r] = p.B + n * p.ldb;
+        if (GATE) brow[NB - 1][r] = p.B2 + n * p.ldb;
+    }
+    const int64_t chunks = p.K / 8;
+    for (int64_t base = 0; base < chunks; base += (int64_t)kPre * kThreads) {
+        half8_t b[kPre][NB][kRows];
+        h8 a[kPre][M];
+        // every load of the batch is issued before the first use
+#pragma unroll
+        for (int j = 0; j < kPre; j++) {
+            const int64_t c = base + j * kThreads + tid;
+            if (c < chunks) {
+#pragma unroll
+                for (int q = 0; q < NB; q++)
+#pragma unroll
+                    for (int r = 0; r < kRows; r++)
+                        b[j][q][r] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(brow[q][r]) + c);
+#pragma unroll
+                for (int m = 0; m < M; m++) a[j][m] = ld8(p.A + m * p.lda + c * 8);
+            }
+        }
+        if (NORM) {
+            // the whole row is in this one batch (K <= 8 * kPre * kThreads, seen to by the launcher)
+            h8 wv[kPre];
+#pragma unroll
+            for (int j = 0; j < kPre; j++) {
+                const int64_t c = base + j * kThreads + tid;
+                if (c < chunks) wv[j] = ld8(p.w + c * 8);
+            }
+#pragma unroll
+            for (int m = 0; m < M; m++) {
+                float ss = 0.f;
+#pragma unroll
+                for (int j = 0; j < kPre; j++) {
+                    const int64_t c = base + j * kThreads + tid;
+                    if (c < chunks) {
+                        if (p.x2) {
+                            const h8 x2v = ld8(p.x2 + m * p.lda + c * 8);
+#pragma unroll
+                            for (int i = 0; i < 8; i++) a[j][m].v[i] = f2h(h2f(a[j][m].v[i]) + h2f(x2v.v[i]));
+                            if (blockIdx.x == 0 && p.sum_out) st8(p.sum_out + m * p.lda + c * 8, a[j][m]);
+                        }
+#pragma unroll
+                        for (int i = 0; i < 8; i++) {
+                            const float f = h2f(a[j][m].v[i]);
+                            ss += f * f;
+                        }
+                    }
+                }
+                ss = block_sum(ss, scratch);
+                const float rinv = 1.0f / sqrtf(ss / (float)p.K + p.eps);
+#pragma unroll
+                for (int j = 0; j < kPre; j++) {
+                    const int64_t c = base + j * kThreads + tid;
+                    if (c < chunks) {
+#pragma unroll
+                        for (int i = 0; i < 8; i++) a[j][m].v[i] = f2h(h2f(wv[j].v[i]) * (h2f(a[j][m].v[i]) * rinv));
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kPre; j++) {
+            const int64_t c = base + j * kThreads + tid;
+            if (c < chunks) {
+#pragma unroll
+                for (int m = 0; m < M; m++) {
+                    half8_t av;
+#pragma unroll
+                    for (int k = 0; k < 8; k++) av[k] = a[j][m].v[k];
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+#pragma unroll
+                        for (int r = 0; r < kRows; r++) acc[q][m][r] = dot8(av, b[j][q][r], acc[q][m][r]);
+                }
+            }
+        }
     }
 #pragma unroll
-    for (int m = 0; m < M; m++)
+    for (int q = 0; q < NB; q++)
 #pragma unroll
-        for (int r = 0; r < kRows; r++) {
-            float v = acc[m][r];
+        for (int m = 0; m < M; m++)
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-            if (lane == 0) part[wid][m * kRows + r] = v;
-        }
+            for (int r = 0; r < kRows; r++) {
+                float v = acc[q][m][r];
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+                if (lane == 0) part[wid][(q * M + m) * kRows + r] = v;
+            }
     __syncthreads();
     if (tid < M * kRows) {
         const int m = tid / kRows, r = tid % kRows;
-        float v = 0.f;
+        float v[NB];
 #pragma unroll
-        for (int w = 0; w < kThreads / 64; w++) v += part[w][tid];
-        if (n0 + r < N) C[m * ldc + n0 + r] = f2h(alpha * v);
+        for (int q = 0; q < NB; q++) {
+            v[q] = 0.f;
+#pragma unroll
+            for (int w = 0; w < kThreads / 64; w++) v[q] += part[w][(q * M + m) * kRows + r];
+        }
+        if (n0 + r < p.N) {
+            if (GATE) {
+                // g = f16(alpha dot_g), u = f16(alpha dot_u); h = f16(f16(silu g) * u)
+                const float g = rnd16(p.alpha * v[0]), u = rnd16(p.alpha * v[NB - 1]);
+                const float y = rnd16(g / (1.0f + expf(-g)));
+                p.C[m * p.ldc + n0 + r] = f2h(y * u);
+            } else {
+                p.C[m * p.ldc + n0 + r] = f2h(p.alpha * v[0]);
+            }
+        }
     }
+}
+
+template <bool NORM, bool GATE, int kPre>
+int launch_pre(int64_t M, const SkinnyArgs &p, hipStream_t st)
+{
+    const dim3 grid((unsigned)((p.N + kRows - 1) / kRows)), block(kThreads);
+    switch (M) {
+        case 1: hipLaunchKernelGGL((gemm_skinny_nt_kernel<1, NORM, GATE, kPre>), grid, block, 0, st, p); break;
+        case 2: hipLaunchKernelGGL((gemm_skinny_nt_kernel<2, NORM, GATE, kPre>), grid, block, 0, st, p); break;
+        case 3: hipLaunchKernelGGL((gemm_skinny_nt_kernel<3, NORM, GATE, kPre>), grid, block, 0, st, p); break;
+        default: hipLaunchKernelGGL((gemm_skinny_nt_kernel<4, NORM, GATE, kPre>), grid, block, 0, st, p); break;
+    }
+    return launch_status("gemm_skinny_nt");
+}
+
+// rows of at most 4096 elements fit two pieces per lane: fewer registers, more workgroups per CU
+template <bool NORM, bool GATE>
+int launch(int64_t M, const SkinnyArgs &p, hipStream_t st)
+{
+    return p.K <= 8 * 2 * kThreads ? launch_pre<NORM, GATE, 2>(M, p, st) : launch_pre<NORM, GATE, kMaxPre>(M, p, st);
 }
 
 }  // namespace
@@ -74,14 +226,28 @@ gemm_skinny_nt_kernel(int64_t N, int64_t K, float alpha, const half_t *__restric
 int gemm_skinny_nt_launch(int64_t M, int64_t N, int64_t K, float alpha, const half_t *A, int64_t lda,
                           const half_t *B, int64_t ldb, half_t *C, int64_t ldc, hipStream_t st)
 {
-    const dim3 grid((unsigned)((N + kRows - 1) / kRows)), block(kThreads);
-    switch (M) {
-        case 1: hipLaunchKernelGGL((gemm_skinny_nt_kernel<1>), grid, block, 0, st, N, K, alpha, A, lda, B, ldb, C, ldc); break;
-        case 2: hipLaunchKernelGGL((gemm_skinny_nt_kernel<2>), grid, block, 0, st, N, K, alpha, A, lda, B, ldb, C, ldc); break;
-        case 3: hipLaunchKernelGGL((gemm_skinny_nt_kernel<3>), grid, block, 0, st, N, K, alpha, A, lda, B, ldb, C, ldc); break;
-        default: hipLaunchKernelGGL((gemm_skinny_nt_kernel<4>), grid, block, 0, st, N, K, alpha, A, lda, B, ldb, C, ldc); break;
-    }
-    return launch_status("gemm_skinny_nt");
+    SkinnyArgs p = {N, K, alpha, A, lda, nullptr, nullptr, 0.f, nullptr, B, nullptr, ldb, C, ldc};
+    return launch<false, false>(M, p, st);
 }
 
 }  // namespace cacti
+
+using namespace cacti;
+
+CACTI_API int cacti_hip_rows_norm_matmul_f16(int64_t M, int64_t N, int64_t K, const void *x, const void *x2,
+                                             const void *w_norm, float eps, void *sum_out, const void *B,
+                                             const void *B_mul, void *C, void *stream)
+{
+    CACTI_REQUIRE(M >= 1 && M <= 4, CACTI_E_NOTIMPL, "rows_norm_matmul: 1 to 4 rows are handled here (M=%lld)", (long long)M);
+    CACTI_REQUIRE(N > 0 && K > 0 && K % 8 == 0 && K <= 8 * kMaxPre * kThreads, CACTI_E_NOTIMPL,
+                  "rows_norm_matmul: need K %% 8 == 0 and K <= %d (K=%lld)", 8 * kMaxPre * kThreads, (long long)K);
+    CACTI_REQUIRE(x && B && C && (w_norm || (!x2 && !sum_out)), CACTI_E_INVALID, "rows_norm_matmul: null pointer");
+    CACTI_REQUIRE(aligned(x, 16) && aligned(x2, 16) && aligned(w_norm, 16) && aligned(sum_out, 16) && aligned(B, 16) &&
+                      aligned(B_mul, 16) && aligned(C, 2),
+                  CACTI_E_INVALID, "rows_norm_matmul: operands must be 16-byte aligned");
+    SkinnyArgs p = {N, K, 1.0f, (const half_t *)x, K, (const half_t *)x2, (const half_t *)w_norm, eps,
+                    (half_t *)sum_out, (const half_t *)B, (const half_t *)B_mul, K, (half_t *)C, N};
+    hipStream_t st = (hipStream_t)stream;
+    if (w_norm) return B_mul ? launch<true, true>(M, p, st) : launch<true, false>(M, p, st);
+    return B_mul ? launch<false, true>(M, p, st) : launch<false, false>(M, p, st);
+}

@@ -563,6 +563,7 @@ CACTI_API int cacti_llama_cached_create(cacti_llama *model, int64_t seq_cap, cac
     c.set_const(k->in_tok);
     int rc = cacti_llama_cached_reset_state(k);
     if (!rc) rc = c.cell_zero(k->in_tok);
+
     if (rc) {
         delete k;
         return rc;
@@ -653,7 +654,12 @@ CACTI_API int cacti_llama_cached_apply(cacti_llama_cached *k, int64_t prev, int6
     char *x = tmp(T * D, 2), *pre = tmp(T * D, 2), *q = tmp(T * D, 2), *qr = tmp(T * D, 2), *kk = tmp(T * D, 2),
          *kr = tmp(T * D, 2), *v = tmp(T * D, 2), *attn = tmp(T * D, 2), *o = tmp(T * D, 2), *x1 = tmp(T * D, 2),
          *post = tmp(T * D, 2), *up = tmp(T * F, 2), *gate = tmp(T * F, 2), *h = tmp(T * F, 2), *down = tmp(T * D, 2),
-         *s16 = tmp(T * H * Cw, 2);
+         *s16 = nullptr, *aws = nullptr;
+    // one to four rows: the fused decoding attention; more: scores, softmax and P V as three products
+    const bool fused_attn = T <= 4 && Dh % 4 == 0 && Dh <= 100 && next <= 8192;
+    const size_t aws_bytes = fused_attn ? cacti_hip_attn_decode_workspace(T, H, Dh, next) : 0;
+    if (fused_attn) aws = tmp((int64_t)aws_bytes, 1);
+    else s16 = tmp(T * H * Cw, 2);
     // outputs
     if (!rc) rc = c.pool_alloc((size_t)(T * V) * 2, &k->out_logit);
     if (!rc) rc = c.pool_alloc((size_t)T * 2, &k->out_tok);
@@ -668,34 +674,65 @@ CACTI_API int cacti_llama_cached_apply(cacti_llama_cached *k, int64_t prev, int6
         char *tok = static_cast<char *>(P(k->in_tok));
         // stream = embed.outer_select(in_tok[prev .. next])
         STEP(cacti_hip_embed_fwd(V, D, P(m->embed), T, tok + prev * 2, x, c.status_ptr(), st));
-        STEP(cacti_hip_rms_norm_fwd(T, D, x, P(m->layers.empty() ? m->head_norm : m->layers[0].pre_norm), g.eps, pre, st));
-        for (size_t l = 0; l < m->layers.size() && !rc; l++) {
-            const LayerCells &w = m->layers[l];
-            char *kc = static_cast<char *>(P(k->k_cache[l])), *vc = static_cast<char *>(P(k->v_cache[l]));
-            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.q), D, 0.f, q, D, st));
-            STEP(cacti_hip_rope_fwd(T, H, Dh, q, cosr, sinr, qr, st));
-            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.k), D, 0.f, kk, D, st));
-            STEP(cacti_hip_rope_fwd(T, H, Dh, kk, cosr, sinr, kr, st));
-            // k_cache[prev .. next] += k, v_cache[prev .. next] += v
-            STEP(cacti_hip_add_f16(T * D, kc + prev * D * 2, kr, kc + prev * D * 2, st));
-            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.v), D, 0.f, v, D, st));
-            STEP(cacti_hip_add_f16(T * D, vc + prev * D * 2, v, vc + prev * D * 2, st));
-            // scores against the cache, row-causal mask + softmax (in place), P V.  Columns from
-            // `next` on are masked for every row, so only the first Cw of the cap columns are formed.
-            STEP(cacti_hip_gemm_f16_strided_batched(0, 1, H, T, Cw, Dh, alpha, qr, D, Dh, kc, D, Dh, 0.f, s16, H * Cw, Cw, st));
-            STEP(cacti_hip_row_causal_softmax_fwd(T, H, Cw, Cw, prev, s16, s16, st));
-            STEP(cacti_hip_gemm_f16_strided_batched(0, 0, H, T, Dh, Cw, 1.f, s16, H * Cw, Cw, vc, D, Dh, 0.f, attn, D, Dh, st));
-            STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, attn, D, P(w.o), D, 0.f, o, D, st));
-            STEP(cacti_hip_add_rms_norm_fwd(T, D, x, o, P(w.post_norm), g.eps, x1, post, st));
-            STEP(cacti_hip_gemm_f16(0, 1, T, F, D, 1.f, post, D, P(w.up), D, 0.f, up, F, st));
-            STEP(cacti_hip_gemm_f16(0, 1, T, F, D, 1.f, post, D, P(w.gate), D, 0.f, gate, F, st));
-            STEP(cacti_hip_silu_gate_fwd(T * F, gate, up, h, st));
-            STEP(cacti_hip_gemm_f16(0, 1, T, D, F, 1.f, h, F, P(w.down), F, 0.f, down, D, st));
-            const CellPtr wn = l + 1 < m->layers.size() ? m->layers[l + 1].pre_norm : m->head_norm;
-            STEP(cacti_hip_add_rms_norm_fwd(T, D, x1, down, P(wn), g.eps, x, pre, st));
+        void *logit = c.dev_ptr(k->out_logit);
+        if (fused_attn && D <= 8192) {
+            // One to four rows: the norms, the residual adds and the SiLU gate ride in the product
+            // kernels (cacti_hip_rows_norm_matmul_f16), which stream each weight matrix once.
+            // The residual stream is (xa) or the pending sum f16(xa + xb).
+            const char *xa = x, *xb = nullptr;
+            for (size_t l = 0; l < m->layers.size() && !rc; l++) {
+                const LayerCells &w = m->layers[l];
+                char *kc = static_cast<char *>(P(k->k_cache[l])), *vc = static_cast<char *>(P(k->v_cache[l]));
+                STEP(cacti_hip_rows_norm_matmul_f16(T, D, D, xa, xb, P(w.pre_norm), g.eps, xb ? x : nullptr, P(w.q), nullptr, q, st));
+                STEP(cacti_hip_rope_fwd(T, H, Dh, q, cosr, sinr, qr, st));
+                STEP(cacti_hip_rows_norm_matmul_f16(T, D, D, xa, xb, P(w.pre_norm), g.eps, nullptr, P(w.k), nullptr, kk, st));
+                STEP(cacti_hip_rope_fwd(T, H, Dh, kk, cosr, sinr, kr, st));
+                STEP(cacti_hip_add_f16(T * D, kc + prev * D * 2, kr, kc + prev * D * 2, st));
+                STEP(cacti_hip_rows_norm_matmul_f16(T, D, D, xa, xb, P(w.pre_norm), g.eps, nullptr, P(w.v), nullptr, v, st));
+                STEP(cacti_hip_add_f16(T * D, vc + prev * D * 2, v, vc + prev * D * 2, st));
+                STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, attn, D, aws, aws_bytes, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, attn, D, P(w.o), D, 0.f, o, D, st));
+                // x1 = stream + o; post = rms_norm(x1); h = silu(post gate^T) * (post up^T)
+                STEP(cacti_hip_rows_norm_matmul_f16(T, F, D, x, o, P(w.post_norm), g.eps, x1, P(w.gate), P(w.up), h, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, F, 1.f, h, F, P(w.down), F, 0.f, down, D, st));
+                xa = x1;                                          // stream = x1 + down, formed by the next consumer
+                xb = down;
+            }
+            STEP(cacti_hip_rows_norm_matmul_f16(T, V, D, xa, xb, P(m->head_norm), g.eps, nullptr, P(m->lm_head), nullptr, logit, st));
+        } else {
+            STEP(cacti_hip_rms_norm_fwd(T, D, x, P(m->layers.empty() ? m->head_norm : m->layers[0].pre_norm), g.eps, pre, st));
+            for (size_t l = 0; l < m->layers.size() && !rc; l++) {
+                const LayerCells &w = m->layers[l];
+                char *kc = static_cast<char *>(P(k->k_cache[l])), *vc = static_cast<char *>(P(k->v_cache[l]));
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.q), D, 0.f, q, D, st));
+                STEP(cacti_hip_rope_fwd(T, H, Dh, q, cosr, sinr, qr, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.k), D, 0.f, kk, D, st));
+                STEP(cacti_hip_rope_fwd(T, H, Dh, kk, cosr, sinr, kr, st));
+                // k_cache[prev .. next] += k, v_cache[prev .. next] += v
+                STEP(cacti_hip_add_f16(T * D, kc + prev * D * 2, kr, kc + prev * D * 2, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, pre, D, P(w.v), D, 0.f, v, D, st));
+                STEP(cacti_hip_add_f16(T * D, vc + prev * D * 2, v, vc + prev * D * 2, st));
+                // scores against the cache, row-causal mask + softmax (in place), P V.  Columns from
+                // `next` on are masked for every row, so only the first Cw of the cap columns are formed.
+                if (fused_attn) {
+                    STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, attn, D, aws, aws_bytes, st));
+                } else {
+                    STEP(cacti_hip_gemm_f16_strided_batched(0, 1, H, T, Cw, Dh, alpha, qr, D, Dh, kc, D, Dh, 0.f, s16, H * Cw, Cw, st));
+                    STEP(cacti_hip_row_causal_softmax_fwd(T, H, Cw, Cw, prev, s16, s16, st));
+                    STEP(cacti_hip_gemm_f16_strided_batched(0, 0, H, T, Dh, Cw, 1.f, s16, H * Cw, Cw, vc, D, Dh, 0.f, attn, D, Dh, st));
+                }
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, attn, D, P(w.o), D, 0.f, o, D, st));
+                STEP(cacti_hip_add_rms_norm_fwd(T, D, x, o, P(w.post_norm), g.eps, x1, post, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, F, D, 1.f, post, D, P(w.up), D, 0.f, up, F, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, F, D, 1.f, post, D, P(w.gate), D, 0.f, gate, F, st));
+                STEP(cacti_hip_silu_gate_fwd(T * F, gate, up, h, st));
+                STEP(cacti_hip_gemm_f16(0, 1, T, D, F, 1.f, h, F, P(w.down), F, 0.f, down, D, st));
+                const CellPtr wn = l + 1 < m->layers.size() ? m->layers[l + 1].pre_norm : m->head_norm;
+                STEP(cacti_hip_add_rms_norm_fwd(T, D, x1, down, P(wn), g.eps, x, pre, st));
+            }
+            STEP(cacti_hip_gemm_f16(0, 1, T, V, D, 1.f, pre, D, P(m->lm_head), D, 0.f, logit, V, st));
         }
-        void *logit = c.dev_ptr(k->out_logit), *otok = c.dev_ptr(k->out_tok);
-        STEP(cacti_hip_gemm_f16(0, 1, T, V, D, 1.f, pre, D, P(m->lm_head), D, 0.f, logit, V, st));
+        void *otok = c.dev_ptr(k->out_tok);
         STEP(cacti_hip_softmax_ce_fwd(T, V, logit, nullptr, want_prob ? c.dev_ptr(k->out_prob) : nullptr, nullptr,
                                       otok, nullptr, st));
         // in_tok[next] += out_lm_tok[T - 1]

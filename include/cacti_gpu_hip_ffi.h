@@ -209,6 +209,32 @@ int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const vo
  * (zeros at the masked ones). */
 int cacti_hip_row_causal_softmax_fwd(int64_t T, int64_t H, int64_t C, int64_t ld, int64_t initial_row,
                                      const void *s16, void *p16, void *stream);
+/* One to four rows through a chain of small thunks and a weight matrix in ONE pass over the
+ * weights (decoding), with the rounding points of the separate thunks:
+ *   r = x                      or f16(x + x2), which is also stored to sum_out (AddFutThunkSpec)
+ *   a = rms_norm(r, w_norm)    as cacti_hip_rms_norm_fwd; skipped (a = r) when w_norm is NULL
+ *   C = f16(a B^T)             matmul(false, B, true), src/librarium/llama.rs:857-937
+ *   or, with B_mul:  C = f16(f16(silu(f16(a B^T))) * f16(a B_mul^T))   the gate / up pair and
+ *                    standard_silu + mul of src/librarium/llama.rs:926-935
+ * x, x2, sum_out: [M,K] f16; w_norm: [K]; B, B_mul: [N,K]; C: [M,N]; all contiguous, 16-byte
+ * aligned; 1 <= M <= 4, K % 8 == 0, K <= 8192. */
+int cacti_hip_rows_norm_matmul_f16(int64_t M, int64_t N, int64_t K, const void *x, const void *x2,
+                                   const void *w_norm, float eps, void *sum_out, const void *B,
+                                   const void *B_mul, void *C, void *stream);
+
+/* Attention of T = 1..4 new positions over the key / value cache in three small launches: the chain
+ * block_matmul_scale(q, k_cache^T, alpha) -> f32 -> row-causal mask -> softmax -> f16 ->
+ * block_matmul(., v_cache) of src/librarium/llama.rs:895-915 with its rounding points (f16 scores
+ * and probabilities, fp32 accumulation, one rounding of the output).  q: [T, ldq] f16 with head h
+ * at columns h*Dh..; k_cache, v_cache: [C, ldkv] f16 likewise (C cached positions, those beyond
+ * T + initial_row - 1 are not read); out: [T, ldo] f16.  Dh % 4 == 0, Dh <= 100; pointers 8-byte
+ * aligned, pitches multiples of 4; C <= 8192.  workspace: cacti_hip_attn_decode_workspace bytes,
+ * 16-byte aligned, contents undefined on return. */
+size_t cacti_hip_attn_decode_workspace(int64_t T, int64_t H, int64_t Dh, int64_t C);
+int cacti_hip_attn_decode_f16(int64_t T, int64_t H, int64_t Dh, int64_t C, int64_t initial_row, float alpha,
+                              const void *q, int64_t ldq, const void *k_cache, const void *v_cache,
+                              int64_t ldkv, void *out, int64_t ldo, void *workspace, size_t workspace_bytes,
+                              void *stream);
 /* in_tok[pos] += out_tok[last] (u16): the token generated for the last position appended to the
  * input sequence on the device, src/librarium/llama.rs:958-959. */
 int cacti_hip_append_token_u16(void *in_tok, int64_t pos, const void *out_tok, int64_t last, void *stream);

@@ -94,6 +94,95 @@ def test_row_causal_softmax_matches_the_oracle(oracle, T, H, Cc, row0):
     assert np.array_equal(d.cpu().numpy(), out.cpu().numpy())
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,H,Dh,Cc,row0", [(1, 4, 64, 8, 0), (1, 32, 100, 2048, 2047), (1, 32, 100, 1031, 1030), (4, 3, 100, 300, 296),
+                                            (2, 5, 36, 129, 50), (3, 2, 4, 700, 0), (1, 2, 100, 128, 127)])
+def test_decoding_attention_matches_the_oracle_chain(oracle, T, H, Dh, Cc, row0):
+    """scores -> mask -> softmax -> P V for one to four rows against the oracle's thunks over the
+    whole cache; rows of the cache beyond the last position hold garbage that must not be read into
+    the result; called twice on the same workspace."""
+    import torch
+    from cacti_amd import ffi
+    print("attn decode", T, H, Dh, Cc, row0, flush=True)
+    r = rng(T * 7 + H + Dh + Cc + row0)
+    D = H * Dh
+    q = (r.standard_normal((T, D))).astype(np.float16)
+    kc = (r.standard_normal((Cc, D))).astype(np.float16)
+    vc = (r.standard_normal((Cc, D))).astype(np.float16)
+    alpha = 1.0 / np.sqrt(Dh)
+    lib, i64, P = oracle.lib(), oracle.i64, oracle.P
+    s16 = np.empty((T, H, Cc), np.float16)
+    lib.th_block_matmul_f16(0, 1, i64(H), i64(T), i64(Cc), i64(Dh), oracle.f32(alpha), P(q), i64(D), i64(Dh), P(kc), i64(D), i64(Dh),
+                            oracle.f32(0.0), P(s16), i64(H * Cc), i64(Cc))
+    p16 = _row_softmax_oracle(oracle, s16, row0)
+    want = np.empty((T, D), np.float16)
+    lib.th_block_matmul_f16(0, 0, i64(H), i64(T), i64(Dh), i64(Cc), oracle.f32(1.0), P(p16), i64(H * Cc), i64(Cc), P(vc), i64(D), i64(Dh),
+                            oracle.f32(0.0), P(want), i64(D), i64(Dh))
+    live = min(Cc, T + row0)
+    kc_d, vc_d = kc.copy(), vc.copy()
+    kc_d[live:] = np.float16("nan")
+    vc_d[live:] = np.float16("nan")
+    dev = lambda a: torch.from_numpy(a.view(np.int16)).cuda()
+    dq, dk, dv = dev(q), dev(kc_d), dev(vc_d)
+    out = torch.zeros((T, D), dtype=torch.int16, device="cuda")
+    nb = ffi.lib().cacti_hip_attn_decode_workspace(T, H, Dh, Cc)
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    for _ in range(2):
+        ffi.call("cacti_hip_attn_decode_f16", T, H, Dh, Cc, row0, alpha, dq.data_ptr(), D, dk.data_ptr(), dv.data_ptr(), D,
+                 out.data_ptr(), D, ws.data_ptr(), nb, None)
+        got = out.cpu().numpy().view(np.float16)
+        assert_parity(got, want, "attn decode")
+        out.zero_()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,add,gate", [(1, 3200, 3200, False, False), (1, 8640, 3200, True, True), (2, 96, 256, True, False),
+                                            (4, 250, 1024, False, True), (3, 32000, 3200, True, False), (1, 64, 8192, True, True),
+                                            (1, 100, 136, False, False)])
+def test_rows_norm_matmul_matches_the_separate_thunks(oracle, M, N, K, add, gate):
+    """residual add -> RMSNorm -> product (-> SiLU gate with a second product) in one kernel against
+    the oracle's thunks one after the other; the residual sum is stored bit-exactly."""
+    import torch
+    from cacti_amd import ffi
+    print("rows norm matmul", M, N, K, add, gate, flush=True)
+    r = rng(M + N + K + add + 2 * gate)
+    x = r.standard_normal((M, K)).astype(np.float16)
+    x2 = (r.standard_normal((M, K)) * 0.5).astype(np.float16) if add else None
+    w = (1 + 0.1 * r.standard_normal(K)).astype(np.float16)
+    B = (r.standard_normal((N, K)) * 0.05).astype(np.float16)
+    B2 = (r.standard_normal((N, K)) * 0.05).astype(np.float16) if gate else None
+    lib, i64, P, f32 = oracle.lib(), oracle.i64, oracle.P, oracle.f32
+    rsum = x
+    if add:
+        rsum = np.empty_like(x)
+        lib.th_add_f16(i64(M * K), P(x), P(x2), P(rsum))
+    a = np.empty_like(x)
+    ts, ss = np.empty((M, K), np.float32), np.empty(M, np.float32)
+    lib.oracle_rmsnorm_fwd(i64(M), i64(K), P(rsum), P(w), f32(1e-6), P(a), P(ts), P(ss))
+    want = oracle.matmul(0, 1, a, B)
+    if gate:
+        up = oracle.matmul(0, 1, a, B2)
+        y, hh = np.empty_like(want), np.empty_like(want)
+        lib.oracle_silu_gate_fwd(i64(M * N), P(want), P(up), P(y), P(hh))
+        want = hh
+    dev = lambda v: torch.from_numpy(v.view(np.int16)).cuda() if v is not None else None
+    dx, dx2, dw, dB, dB2 = dev(x), dev(x2), dev(w), dev(B), dev(B2)
+    out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    sout = torch.zeros((M, K), dtype=torch.int16, device="cuda") if add else None
+    ptr = lambda v: v.data_ptr() if v is not None else None
+    ffi.call("cacti_hip_rows_norm_matmul_f16", M, N, K, ptr(dx), ptr(dx2), ptr(dw), 1e-6, ptr(sout), ptr(dB), ptr(dB2),
+             out.data_ptr(), None)
+    got = out.cpu().numpy().view(np.float16)
+    assert_parity(got, want, "rows norm matmul")
+    assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.9        # the rest differ by one f16 ulp
+    if add:
+        assert np.array_equal(sout.cpu().numpy().view(np.uint16), rsum.view(np.uint16))
+    # without the norm: the plain product of the (summed) rows
+    if not add and not gate:
+        ffi.call("cacti_hip_rows_norm_matmul_f16", M, N, K, ptr(dx), None, None, 0.0, None, ptr(dB), None, out.data_ptr(), None)
+        assert_parity(out.cpu().numpy().view(np.float16), oracle.matmul(0, 1, x, B), "rows matmul")
+
+
 def _gpu_model(cfg, flat):
     from tests.test_gpu_llama import _model
     ctx, m = _model(cfg)
