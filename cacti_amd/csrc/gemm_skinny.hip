@@ -16,6 +16,9 @@
 //    workgroup reduction, then a = f16(w * (x * rinv)) exactly as the RMSNorm kernel rounds it.
 //  * GATE: two weight matrices share the rows (gate and up projection); the epilogue stores
 //    f16(f16(silu(g)) * u) of the two rounded products, as the SiLU-gate kernel computes it.
+//  * QKV: one launch covers the query, key and value projections; a workgroup owns two rotation
+//    pairs of a head, rotates queries and keys in the epilogue and adds keys and values to the
+//    cache rows of the new positions.
 #include "gemm_internal.h"
 
 namespace cacti {
@@ -36,11 +39,18 @@ struct SkinnyArgs {
     float eps;
     half_t *sum_out;         // NORM with x2: the residual sum [M, lda], written by workgroup 0
     const half_t *B;         // [N, ldb]
-    const half_t *B2;        // GATE: the second weight matrix [N, ldb]
+    const half_t *B2;        // GATE: the second weight matrix [N, ldb]; QKV: the key projection
     int64_t ldb;
-    half_t *C;
+    half_t *C;               // QKV: the rotated queries [M, ldc]
     int64_t ldc;
+    // QKV: value projection, position tables (row 0 = the first new position), caches (row 0 = the
+    // first new position, pitch ldc), heads
+    const half_t *B3;
+    const half_t *cos16, *sin16;
+    half_t *kc, *vc;
+    int H, Dh;
 };
+enum : int { E_PLAIN = 0, E_GATE = 1, E_QKV = 2 };
 
 __device__ __forceinline__ float block_sum(float v, float *scratch)
 {
@@ -67,10 +77,11 @@ __device__ __forceinline__ float dot8(const half8_t &a, const half8_t &b, float 
     return acc;
 }
 
-template <int M, bool NORM, bool GATE, int kPre>
+template <int M, bool NORM, int EPI, int kPre>
 __global__ void __launch_bounds__(kThreads)
 gemm_skinny_nt_kernel(SkinnyArgs p)
 {
+    constexpr bool GATE = EPI == E_GATE;
     constexpr int NB = GATE ? 2 : 1;
     __shared__ float part[kThreads / 64][NB * M * kRows];
     __shared__ float scratch[kThreads / 64];
@@ -85,11 +96,26 @@ gemm_skinny_nt_kernel(SkinnyArgs p)
             for (int r = 0; r < kRows; r++) acc[b][m][r] = 0.f;
     // rows past N re-read the last row (their sums are dropped)
     const half_t *brow[NB][kRows];
+    int64_t col[kRows];
+    if (EPI == E_QKV) {
+        // the workgroup owns two rotation pairs of one head: columns d, d + 1, d + Dh/2, d + 1 + Dh/2;
+        // blockIdx.y picks the query, key or value projection
+        const int hf = p.Dh / 2, per_head = hf / 2;
+        const int head = blockIdx.x / per_head, d0 = 2 * (blockIdx.x - head * per_head);
+        const half_t *Bsel = blockIdx.y == 0 ? p.B : blockIdx.y == 1 ? p.B2 : p.B3;
 #pragma unroll
-    for (int r = 0; r < kRows; r++) {
-        const int64_t n = n0 + r < p.N ? n0 + r : p.N - 1;
-        brow[0][r] = p.B + n * p.ldb;
-        if (GATE) brow[NB - 1][r] = p.B2 + n * p.ldb;
+        for (int r = 0; r < kRows; r++) {
+            col[r] = (int64_t)head * p.Dh + d0 + (r & 1) + (r >> 1) * hf;
+            brow[0][r] = Bsel + col[r] * p.ldb;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < kRows; r++) {
+            col[r] = n0 + r;
+            const int64_t n = n0 + r < p.N ? n0 + r : p.N - 1;
+            brow[0][r] = p.B + n * p.ldb;
+            if (GATE) brow[NB - 1][r] = p.B2 + n * p.ldb;
+        }
     }
     const int64_t chunks = p.K / 8;
     for (int64_t base = 0; base < chunks; base += (int64_t)kPre * kThreads) {
@@ -128,7 +154,7 @@ gemm_skinny_nt_kernel(SkinnyArgs p)
                             const h8 x2v = ld8(p.x2 + m * p.lda + c * 8);
 #pragma unroll
                             for (int i = 0; i < 8; i++) a[j][m].v[i] = f2h(h2f(a[j][m].v[i]) + h2f(x2v.v[i]));
-                            if (blockIdx.x == 0 && p.sum_out) st8(p.sum_out + m * p.lda + c * 8, a[j][m]);
+                            if (blockIdx.x == 0 && blockIdx.y == 0 && p.sum_out) st8(p.sum_out + m * p.lda + c * 8, a[j][m]);
                         }
 #pragma unroll
                         for (int i = 0; i < 8; i++) {
@@ -178,6 +204,36 @@ gemm_skinny_nt_kernel(SkinnyArgs p)
                 if (lane == 0) part[wid][(q * M + m) * kRows + r] = v;
             }
     __syncthreads();
+    if (EPI == E_QKV) {
+        // rotate (queries, keys) and add to the caches (keys, values) with the rounding points of
+        // the separate thunks: y = f16(f16(x cos) + f16(rot(x) sin)), cache = f16(cache + y)
+        __shared__ float xr[M][kRows];
+        const int m = tid / kRows, r = tid % kRows;
+        if (tid < M * kRows) {
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < kThreads / 64; w++) v += part[w][m * kRows + r];
+            xr[m][r] = rnd16(p.alpha * v);
+        }
+        __syncthreads();
+        if (tid < M * kRows) {
+            float y = xr[m][r];
+            if (blockIdx.y < 2) {
+                const bool left = r < 2;
+                const float xp = xr[m][r ^ 2];
+                const int64_t d = col[r] % p.Dh;
+                const float cs = h2f(p.cos16[m * p.Dh + d]), sn = h2f(p.sin16[m * p.Dh + d]);
+                y = rnd16(rnd16(y * cs) + rnd16((left ? -xp : xp) * sn));
+            }
+            if (blockIdx.y == 0) {
+                p.C[m * p.ldc + col[r]] = f2h(y);
+            } else {
+                half_t *dst = (blockIdx.y == 1 ? p.kc : p.vc) + m * p.ldc + col[r];
+                *dst = f2h(h2f(*dst) + y);
+            }
+        }
+        return;
+    }
     if (tid < M * kRows) {
         const int m = tid / kRows, r = tid % kRows;
         float v[NB];
@@ -200,24 +256,24 @@ gemm_skinny_nt_kernel(SkinnyArgs p)
     }
 }
 
-template <bool NORM, bool GATE, int kPre>
+template <bool NORM, int EPI, int kPre>
 int launch_pre(int64_t M, const SkinnyArgs &p, hipStream_t st)
 {
-    const dim3 grid((unsigned)((p.N + kRows - 1) / kRows)), block(kThreads);
+    const dim3 grid((unsigned)((p.N + kRows - 1) / kRows), EPI == E_QKV ? 3 : 1), block(kThreads);
     switch (M) {
-        case 1: hipLaunchKernelGGL((gemm_skinny_nt_kernel<1, NORM, GATE, kPre>), grid, block, 0, st, p); break;
-        case 2: hipLaunchKernelGGL((gemm_skinny_nt_kernel<2, NORM, GATE, kPre>), grid, block, 0, st, p); break;
-        case 3: hipLaunchKernelGGL((gemm_skinny_nt_kernel<3, NORM, GATE, kPre>), grid, block, 0, st, p); break;
-        default: hipLaunchKernelGGL((gemm_skinny_nt_kernel<4, NORM, GATE, kPre>), grid, block, 0, st, p); break;
+        case 1: hipLaunchKernelGGL((gemm_skinny_nt_kernel<1, NORM, EPI, kPre>), grid, block, 0, st, p); break;
+        case 2: hipLaunchKernelGGL((gemm_skinny_nt_kernel<2, NORM, EPI, kPre>), grid, block, 0, st, p); break;
+        case 3: hipLaunchKernelGGL((gemm_skinny_nt_kernel<3, NORM, EPI, kPre>), grid, block, 0, st, p); break;
+        default: hipLaunchKernelGGL((gemm_skinny_nt_kernel<4, NORM, EPI, kPre>), grid, block, 0, st, p); break;
     }
     return launch_status("gemm_skinny_nt");
 }
 
 // rows of at most 4096 elements fit two pieces per lane: fewer registers, more workgroups per CU
-template <bool NORM, bool GATE>
+template <bool NORM, int EPI>
 int launch(int64_t M, const SkinnyArgs &p, hipStream_t st)
 {
-    return p.K <= 8 * 2 * kThreads ? launch_pre<NORM, GATE, 2>(M, p, st) : launch_pre<NORM, GATE, kMaxPre>(M, p, st);
+    return p.K <= 8 * 2 * kThreads ? launch_pre<NORM, EPI, 2>(M, p, st) : launch_pre<NORM, EPI, kMaxPre>(M, p, st);
 }
 
 }  // namespace
@@ -226,8 +282,9 @@ int launch(int64_t M, const SkinnyArgs &p, hipStream_t st)
 int gemm_skinny_nt_launch(int64_t M, int64_t N, int64_t K, float alpha, const half_t *A, int64_t lda,
                           const half_t *B, int64_t ldb, half_t *C, int64_t ldc, hipStream_t st)
 {
-    SkinnyArgs p = {N, K, alpha, A, lda, nullptr, nullptr, 0.f, nullptr, B, nullptr, ldb, C, ldc};
-    return launch<false, false>(M, p, st);
+    SkinnyArgs p = {N, K, alpha, A, lda, nullptr, nullptr, 0.f, nullptr, B, nullptr, ldb, C, ldc,
+                    nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+    return launch<false, E_PLAIN>(M, p, st);
 }
 
 }  // namespace cacti
@@ -246,8 +303,31 @@ CACTI_API int cacti_hip_rows_norm_matmul_f16(int64_t M, int64_t N, int64_t K, co
                       aligned(B_mul, 16) && aligned(C, 2),
                   CACTI_E_INVALID, "rows_norm_matmul: operands must be 16-byte aligned");
     SkinnyArgs p = {N, K, 1.0f, (const half_t *)x, K, (const half_t *)x2, (const half_t *)w_norm, eps,
-                    (half_t *)sum_out, (const half_t *)B, (const half_t *)B_mul, K, (half_t *)C, N};
+                    (half_t *)sum_out, (const half_t *)B, (const half_t *)B_mul, K, (half_t *)C, N,
+                    nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
     hipStream_t st = (hipStream_t)stream;
-    if (w_norm) return B_mul ? launch<true, true>(M, p, st) : launch<true, false>(M, p, st);
-    return B_mul ? launch<false, true>(M, p, st) : launch<false, false>(M, p, st);
+    if (w_norm) return B_mul ? launch<true, E_GATE>(M, p, st) : launch<true, E_PLAIN>(M, p, st);
+    return B_mul ? launch<false, E_GATE>(M, p, st) : launch<false, E_PLAIN>(M, p, st);
+}
+
+CACTI_API int cacti_hip_rows_qkv_rope_cache_f16(int64_t M, int64_t H, int64_t Dh, const void *x, const void *x2,
+                                                const void *w_norm, float eps, void *sum_out, const void *Wq,
+                                                const void *Wk, const void *Wv, const void *cos16, const void *sin16,
+                                                void *q_rot, void *k_cache_rows, void *v_cache_rows, void *stream)
+{
+    const int64_t D = H * Dh;
+    CACTI_REQUIRE(M >= 1 && M <= 4, CACTI_E_NOTIMPL, "rows_qkv: 1 to 4 rows are handled here (M=%lld)", (long long)M);
+    CACTI_REQUIRE(H > 0 && Dh > 0 && Dh % 4 == 0 && D % 8 == 0 && D <= 8 * kMaxPre * kThreads, CACTI_E_NOTIMPL,
+                  "rows_qkv: need Dh %% 4 == 0, H*Dh %% 8 == 0 and H*Dh <= %d", 8 * kMaxPre * kThreads);
+    CACTI_REQUIRE(x && w_norm && Wq && Wk && Wv && cos16 && sin16 && q_rot && k_cache_rows && v_cache_rows, CACTI_E_INVALID,
+                  "rows_qkv: null pointer");
+    CACTI_REQUIRE(aligned(x, 16) && aligned(x2, 16) && aligned(w_norm, 16) && aligned(sum_out, 16) && aligned(Wq, 16) &&
+                      aligned(Wk, 16) && aligned(Wv, 16) && aligned(cos16, 2) && aligned(sin16, 2) && aligned(q_rot, 2) &&
+                      aligned(k_cache_rows, 2) && aligned(v_cache_rows, 2),
+                  CACTI_E_INVALID, "rows_qkv: rows and weights must be 16-byte aligned");
+    SkinnyArgs p = {D, D, 1.0f, (const half_t *)x, D, (const half_t *)x2, (const half_t *)w_norm, eps,
+                    (half_t *)sum_out, (const half_t *)Wq, (const half_t *)Wk, D, (half_t *)q_rot, D,
+                    (const half_t *)Wv, (const half_t *)cos16, (const half_t *)sin16, (half_t *)k_cache_rows,
+                    (half_t *)v_cache_rows, (int)H, (int)Dh};
+    return launch<true, E_QKV>(M, p, (hipStream_t)stream);
 }

@@ -683,13 +683,9 @@ CACTI_API int cacti_llama_cached_apply(cacti_llama_cached *k, int64_t prev, int6
             for (size_t l = 0; l < m->layers.size() && !rc; l++) {
                 const LayerCells &w = m->layers[l];
                 char *kc = static_cast<char *>(P(k->k_cache[l])), *vc = static_cast<char *>(P(k->v_cache[l]));
-                STEP(cacti_hip_rows_norm_matmul_f16(T, D, D, xa, xb, P(w.pre_norm), g.eps, xb ? x : nullptr, P(w.q), nullptr, q, st));
-                STEP(cacti_hip_rope_fwd(T, H, Dh, q, cosr, sinr, qr, st));
-                STEP(cacti_hip_rows_norm_matmul_f16(T, D, D, xa, xb, P(w.pre_norm), g.eps, nullptr, P(w.k), nullptr, kk, st));
-                STEP(cacti_hip_rope_fwd(T, H, Dh, kk, cosr, sinr, kr, st));
-                STEP(cacti_hip_add_f16(T * D, kc + prev * D * 2, kr, kc + prev * D * 2, st));
-                STEP(cacti_hip_rows_norm_matmul_f16(T, D, D, xa, xb, P(w.pre_norm), g.eps, nullptr, P(w.v), nullptr, v, st));
-                STEP(cacti_hip_add_f16(T * D, vc + prev * D * 2, v, vc + prev * D * 2, st));
+                // q, k, v projections of the normed stream, rotation, k_cache[prev ..] += k, v_cache[prev ..] += v
+                STEP(cacti_hip_rows_qkv_rope_cache_f16(T, H, Dh, xa, xb, P(w.pre_norm), g.eps, xb ? x : nullptr, P(w.q), P(w.k),
+                                                       P(w.v), cosr, sinr, qr, kc + prev * D * 2, vc + prev * D * 2, st));
                 STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, attn, D, aws, aws_bytes, st));
                 STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, attn, D, P(w.o), D, 0.f, o, D, st));
                 // x1 = stream + o; post = rms_norm(x1); h = silu(post gate^T) * (post up^T)

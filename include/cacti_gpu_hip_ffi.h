@@ -222,6 +222,20 @@ int cacti_hip_rows_norm_matmul_f16(int64_t M, int64_t N, int64_t K, const void *
                                    const void *w_norm, float eps, void *sum_out, const void *B,
                                    const void *B_mul, void *C, void *stream);
 
+/* The head of a cached attention block for one to four rows in ONE launch
+ * (src/librarium/llama.rs:855-893): a = rms_norm(x or f16(x + x2), w_norm) as above, then
+ *   q_rot                = symplectic_embed(f16(a Wq^T))
+ *   k_cache_rows        += symplectic_embed(f16(a Wk^T))
+ *   v_cache_rows        += f16(a Wv^T)
+ * with the rounding points of the separate thunks (product, cos / sin products, their sum, the
+ * accumulation into the cache).  x, x2, sum_out, q_rot: [M, H*Dh] f16; Wq, Wk, Wv: [H*Dh, H*Dh];
+ * cos16, sin16: rows of the position tables for the M positions ([M, Dh]); k_cache_rows,
+ * v_cache_rows: the cache rows of the M positions ([M, H*Dh]).  Dh % 4 == 0, H*Dh <= 8192. */
+int cacti_hip_rows_qkv_rope_cache_f16(int64_t M, int64_t H, int64_t Dh, const void *x, const void *x2,
+                                      const void *w_norm, float eps, void *sum_out, const void *Wq,
+                                      const void *Wk, const void *Wv, const void *cos16, const void *sin16,
+                                      void *q_rot, void *k_cache_rows, void *v_cache_rows, void *stream);
+
 /* Attention of T = 1..4 new positions over the key / value cache in three small launches: the chain
  * block_matmul_scale(q, k_cache^T, alpha) -> f32 -> row-causal mask -> softmax -> f16 ->
  * block_matmul(., v_cache) of src/librarium/llama.rs:895-915 with its rounding points (f16 scores

@@ -183,6 +183,55 @@ def test_rows_norm_matmul_matches_the_separate_thunks(oracle, M, N, K, add, gate
         assert_parity(out.cpu().numpy().view(np.float16), oracle.matmul(0, 1, x, B), "rows matmul")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,H,Dh,add", [(1, 32, 100, True), (1, 4, 64, False), (4, 6, 36, True), (2, 16, 128, False)])
+def test_rows_qkv_rope_cache_matches_the_separate_thunks(oracle, M, H, Dh, add):
+    """norm -> q, k, v products -> rotation -> cache accumulation in one launch against the oracle's
+    thunks; the cache rows already hold values (the reference accumulates into them)."""
+    import torch
+    from cacti_amd import ffi
+    print("rows qkv", M, H, Dh, add, flush=True)
+    r = rng(M + H + Dh + add)
+    D, pos0, cap = H * Dh, 5, 16
+    x = r.standard_normal((M, D)).astype(np.float16)
+    x2 = (r.standard_normal((M, D)) * 0.5).astype(np.float16) if add else None
+    w = (1 + 0.1 * r.standard_normal(D)).astype(np.float16)
+    Wq, Wk, Wv = ((r.standard_normal((D, D)) * 0.05).astype(np.float16) for _ in range(3))
+    kc0, vc0 = ((r.standard_normal((M, D)) * 0.3).astype(np.float16) for _ in range(2))
+    lib, i64, P, f32 = oracle.lib(), oracle.i64, oracle.P, oracle.f32
+    cos16, sin16 = np.empty((cap, Dh), np.float16), np.empty((cap, Dh), np.float16)
+    lib.oracle_rope_tables(i64(cap), i64(Dh), P(cos16), P(sin16))
+    cr, sr = np.ascontiguousarray(cos16[pos0:pos0 + M]), np.ascontiguousarray(sin16[pos0:pos0 + M])
+    rsum = x
+    if add:
+        rsum = np.empty_like(x)
+        lib.th_add_f16(i64(M * D), P(x), P(x2), P(rsum))
+    a = np.empty_like(x)
+    ts, ss = np.empty((M, D), np.float32), np.empty(M, np.float32)
+    lib.oracle_rmsnorm_fwd(i64(M), i64(D), P(rsum), P(w), f32(1e-6), P(a), P(ts), P(ss))
+    q, kk, v = oracle.matmul(0, 1, a, Wq), oracle.matmul(0, 1, a, Wk), oracle.matmul(0, 1, a, Wv)
+    qr, kr = np.empty_like(q), np.empty_like(kk)
+    lib.oracle_rope_fwd(i64(M), i64(H), i64(Dh), P(q), P(cr), P(sr), P(qr))
+    lib.oracle_rope_fwd(i64(M), i64(H), i64(Dh), P(kk), P(cr), P(sr), P(kr))
+    want_k, want_v = np.empty_like(kc0), np.empty_like(vc0)
+    lib.th_add_f16(i64(M * D), P(kc0), P(kr), P(want_k))
+    lib.th_add_f16(i64(M * D), P(vc0), P(v), P(want_v))
+    dev = lambda t_: torch.from_numpy(np.ascontiguousarray(t_).view(np.int16)).cuda() if t_ is not None else None
+    ptr = lambda t_: t_.data_ptr() if t_ is not None else None
+    dx, dx2, dw, dq, dk, dv, dc, ds, dkc, dvc = (dev(t_) for t_ in (x, x2, w, Wq, Wk, Wv, cr, sr, kc0, vc0))
+    out = torch.zeros((M, D), dtype=torch.int16, device="cuda")
+    sout = torch.zeros((M, D), dtype=torch.int16, device="cuda") if add else None
+    ffi.call("cacti_hip_rows_qkv_rope_cache_f16", M, H, Dh, ptr(dx), ptr(dx2), ptr(dw), 1e-6, ptr(sout), ptr(dq), ptr(dk), ptr(dv),
+             ptr(dc), ptr(ds), out.data_ptr(), ptr(dkc), ptr(dvc), None)
+    h16 = lambda t_: t_.cpu().numpy().view(np.float16)
+    assert_parity(h16(out), qr, "rotated queries")
+    assert_parity(h16(dkc), want_k, "key cache rows")
+    assert_parity(h16(dvc), want_v, "value cache rows")
+    assert np.mean(h16(out).view(np.uint16) == qr.view(np.uint16)) > 0.95
+    if add:
+        assert np.array_equal(sout.cpu().numpy().view(np.uint16), rsum.view(np.uint16))
+
+
 def _gpu_model(cfg, flat):
     from tests.test_gpu_llama import _model
     ctx, m = _model(cfg)
