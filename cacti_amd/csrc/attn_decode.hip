@@ -34,26 +34,26 @@ struct __attribute__((aligned(8))) h4 {
 template <int T>
 __global__ void __launch_bounds__(kThreads)
 decode_scores_kernel(int C, int H, int Dh, float alpha, const half_t *__restrict__ q, int64_t ldq,
-                     const half_t *__restrict__ kc, int64_t ldk, half_t *__restrict__ s16, int64_t ld)
+                     const half_t *__restrict__ kc, int64_t ldk, int64_t hsk, half_t *__restrict__ s16, int64_t ld)
 {
     __shared__ float part[T][kSlice * 25 + kSlice];        // [t][row * pieces + piece], pieces <= 26 here
     const int tid = threadIdx.x, h = blockIdx.y, j0 = blockIdx.x * kSlice;
     const int pieces = Dh / 4;
     const int nrow = min(kSlice, C - j0);
     const int total = nrow * pieces;
-    // all of the lane's loads are issued before the first use: at most 13 pieces of K of 8 bytes,
-    // each with the matching piece of every query row (those hit in L2)
+    // All of the lane's loads are issued before the first use: at most 13 pieces of K of 8 bytes,
+    // each with the matching piece of every query row (those hit in L2).  The loads are
+    // unconditional (pieces past the slice re-read its last piece): a load inside a branch is
+    // waited for at the end of the branch, which would turn the 13 loads into 13 round trips.
     constexpr int kMaxIter = (kSlice * 25 + kThreads - 1) / kThreads;
     h4 kv[kMaxIter], qv[kMaxIter][T];
 #pragma unroll
     for (int it = 0; it < kMaxIter; it++) {
-        const int p = tid + it * kThreads;
-        if (p < total) {
-            const int r = p / pieces, c = p - r * pieces;
-            kv[it] = *reinterpret_cast<const h4 *>(kc + (int64_t)(j0 + r) * ldk + h * Dh + 4 * c);
+        const int p = min(tid + it * kThreads, total - 1);
+        const int r = p / pieces, c = p - r * pieces;
+        kv[it] = *reinterpret_cast<const h4 *>(kc + (int64_t)(j0 + r) * ldk + h * hsk + 4 * c);
 #pragma unroll
-            for (int t = 0; t < T; t++) qv[it][t] = *reinterpret_cast<const h4 *>(q + t * ldq + h * Dh + 4 * c);
-        }
+        for (int t = 0; t < T; t++) qv[it][t] = *reinterpret_cast<const h4 *>(q + t * ldq + h * Dh + 4 * c);
     }
 #pragma unroll
     for (int it = 0; it < kMaxIter; it++) {
@@ -95,7 +95,7 @@ constexpr int kRowIter = 4;                // 8-column pieces of a score row per
 template <int T>
 __global__ void __launch_bounds__(kThreads)
 decode_values_kernel(int C, int H, int Dh, int64_t row0, const half_t *__restrict__ s16, int64_t ld,
-                     const half_t *__restrict__ vc, int64_t ldv, float *__restrict__ partial)
+                     const half_t *__restrict__ vc, int64_t ldv, int64_t hsv, float *__restrict__ partial)
 {
     __shared__ float ps[T][kSlice];
     __shared__ float red[8][T][kMaxPieces * 4];
@@ -111,11 +111,13 @@ decode_values_kernel(int C, int H, int Dh, int64_t row0, const half_t *__restric
     constexpr int kRowsPerGroup = kSlice / G;
     const int g = tid / pieces, c = tid - g * pieces;
     h4 vv[kRowsPerGroup];
-    if (g < G) {
+    {
+        // unconditional loads (clamped to the slice's last row and to a piece of the head): see above
+        const int cc = g < G ? c : 0;
 #pragma unroll
         for (int it = 0; it < kRowsPerGroup; it++) {
-            const int r = g + it * G;
-            if (r < nrow) vv[it] = *reinterpret_cast<const h4 *>(vc + (int64_t)(j0 + r) * ldv + h * Dh + 4 * c);
+            const int r = min((g < G ? g : 0) + it * G, nrow - 1);
+            vv[it] = *reinterpret_cast<const h4 *>(vc + (int64_t)(j0 + r) * ldv + h * hsv + 4 * cc);
         }
     }
     h8 rowv[T][kRowIter];
@@ -124,12 +126,13 @@ decode_values_kernel(int C, int H, int Dh, int64_t row0, const half_t *__restric
     for (int t = 0; t < T; t++) {
         const half_t *sr = s16 + ((int64_t)t * H + h) * ld;
         const int live = (int)min((int64_t)C, (int64_t)t + row0 + 1);
+        const int last8 = ((live - 1) / 8) * 8;                        // live >= 1
 #pragma unroll
         for (int it = 0; it < kRowIter; it++) {
-            const int j8 = (tid + it * kThreads) * 8;                  // rows are 16-byte aligned, ld % 8 == 0
-            if (j8 < live) rowv[t][it] = ld8(sr + j8);
+            const int j8 = min((tid + it * kThreads) * 8, last8);      // rows are 16-byte aligned, ld % 8 == 0
+            rowv[t][it] = ld8(sr + j8);
         }
-        own[t] = (tid < nrow && j0 + tid < live) ? sr[j0 + tid] : (half_t)0.f;
+        own[t] = sr[min(j0 + tid, live - 1)];
     }
     // probabilities of the slice: every row's maximum and sum run over all its live columns
 #pragma unroll
@@ -223,8 +226,8 @@ CACTI_API size_t cacti_hip_attn_decode_workspace(int64_t T, int64_t H, int64_t D
 
 CACTI_API int cacti_hip_attn_decode_f16(int64_t T, int64_t H, int64_t Dh, int64_t C, int64_t initial_row, float alpha,
                                         const void *q, int64_t ldq, const void *k_cache, const void *v_cache,
-                                        int64_t ldkv, void *out, int64_t ldo, void *workspace, size_t workspace_bytes,
-                                        void *stream)
+                                        int64_t ldkv, int64_t head_stride, void *out, int64_t ldo, void *workspace,
+                                        size_t workspace_bytes, void *stream)
 {
     CACTI_REQUIRE(T >= 1 && T <= 4 && H > 0 && C > 0 && initial_row >= 0, CACTI_E_NOTIMPL,
                   "attn_decode: 1 to 4 rows are handled here (T=%lld)", (long long)T);
@@ -232,7 +235,7 @@ CACTI_API int cacti_hip_attn_decode_f16(int64_t T, int64_t H, int64_t Dh, int64_
     CACTI_REQUIRE(q && k_cache && v_cache && out && workspace, CACTI_E_INVALID, "attn_decode: null pointer");
     CACTI_REQUIRE(C <= (int64_t)kRowIter * kThreads * 8, CACTI_E_NOTIMPL, "attn_decode: at most %d cached positions",
                   kRowIter * kThreads * 8);
-    CACTI_REQUIRE(ldq % 4 == 0 && ldkv % 4 == 0 && aligned(q, 8) && aligned(k_cache, 8) && aligned(v_cache, 8) &&
+    CACTI_REQUIRE(ldq % 4 == 0 && ldkv % 4 == 0 && head_stride % 4 == 0 && aligned(q, 8) && aligned(k_cache, 8) && aligned(v_cache, 8) &&
                       aligned(workspace, 16),
                   CACTI_E_INVALID, "attn_decode: operands must be 8-byte aligned with row pitches that are multiples of 4");
     CACTI_REQUIRE(workspace_bytes >= cacti_hip_attn_decode_workspace(T, H, Dh, C), CACTI_E_INVALID,
@@ -247,9 +250,9 @@ CACTI_API int cacti_hip_attn_decode_f16(int64_t T, int64_t H, int64_t Dh, int64_
 #define LAUNCH(TT)                                                                                                     \
     do {                                                                                                               \
         hipLaunchKernelGGL((decode_scores_kernel<TT>), grid, block, 0, st, (int)live, (int)H, (int)Dh, alpha,          \
-                           (const half_t *)q, ldq, (const half_t *)k_cache, ldkv, s16, ld);                            \
+                           (const half_t *)q, ldq, (const half_t *)k_cache, ldkv, head_stride, s16, ld);               \
         hipLaunchKernelGGL((decode_values_kernel<TT>), grid, block, 0, st, (int)live, (int)H, (int)Dh, initial_row, s16, \
-                           ld, (const half_t *)v_cache, ldkv, partial);                                                \
+                           ld, (const half_t *)v_cache, ldkv, head_stride, partial);                                   \
         hipLaunchKernelGGL((decode_reduce_kernel<TT>), dim3((unsigned)H), dim3(128), 0, st, (int)grid.x, (int)Dh,      \
                            (const float *)partial, (half_t *)out, ldo);                                                \
     } while (0)

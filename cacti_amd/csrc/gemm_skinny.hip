@@ -121,27 +121,30 @@ gemm_skinny_nt_kernel(SkinnyArgs p)
     for (int64_t base = 0; base < chunks; base += (int64_t)kPre * kThreads) {
         half8_t b[kPre][NB][kRows];
         h8 a[kPre][M];
-        // every load of the batch is issued before the first use
+        // Every load of the batch is issued before the first use, unconditionally (pieces past the
+        // row re-read its last piece): a load inside a branch is waited for at the end of the branch.
 #pragma unroll
         for (int j = 0; j < kPre; j++) {
-            const int64_t c = base + j * kThreads + tid;
-            if (c < chunks) {
+            const int64_t cr = base + j * kThreads + tid, c = cr < chunks ? cr : chunks - 1;
 #pragma unroll
-                for (int q = 0; q < NB; q++)
+            for (int q = 0; q < NB; q++)
 #pragma unroll
-                    for (int r = 0; r < kRows; r++)
-                        b[j][q][r] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(brow[q][r]) + c);
+                for (int r = 0; r < kRows; r++)
+                    b[j][q][r] = __builtin_nontemporal_load(reinterpret_cast<const half8_t *>(brow[q][r]) + c);
 #pragma unroll
-                for (int m = 0; m < M; m++) a[j][m] = ld8(p.A + m * p.lda + c * 8);
-            }
+            for (int m = 0; m < M; m++) a[j][m] = ld8(p.A + m * p.lda + c * 8);
         }
         if (NORM) {
             // the whole row is in this one batch (K <= 8 * kPre * kThreads, seen to by the launcher)
-            h8 wv[kPre];
+            h8 wv[kPre], x2v[kPre][M];
 #pragma unroll
             for (int j = 0; j < kPre; j++) {
-                const int64_t c = base + j * kThreads + tid;
-                if (c < chunks) wv[j] = ld8(p.w + c * 8);
+                const int64_t cr = base + j * kThreads + tid, c = cr < chunks ? cr : chunks - 1;
+                wv[j] = ld8(p.w + c * 8);
+                if (p.x2) {                                       // uniform over the launch
+#pragma unroll
+                    for (int m = 0; m < M; m++) x2v[j][m] = ld8(p.x2 + m * p.lda + c * 8);
+                }
             }
 #pragma unroll
             for (int m = 0; m < M; m++) {
@@ -151,9 +154,8 @@ gemm_skinny_nt_kernel(SkinnyArgs p)
                     const int64_t c = base + j * kThreads + tid;
                     if (c < chunks) {
                         if (p.x2) {
-                            const h8 x2v = ld8(p.x2 + m * p.lda + c * 8);
 #pragma unroll
-                            for (int i = 0; i < 8; i++) a[j][m].v[i] = f2h(h2f(a[j][m].v[i]) + h2f(x2v.v[i]));
+                            for (int i = 0; i < 8; i++) a[j][m].v[i] = f2h(h2f(a[j][m].v[i]) + h2f(x2v[j][m].v[i]));
                             if (blockIdx.x == 0 && blockIdx.y == 0 && p.sum_out) st8(p.sum_out + m * p.lda + c * 8, a[j][m]);
                         }
 #pragma unroll

@@ -686,7 +686,7 @@ CACTI_API int cacti_llama_cached_apply(cacti_llama_cached *k, int64_t prev, int6
                 // q, k, v projections of the normed stream, rotation, k_cache[prev ..] += k, v_cache[prev ..] += v
                 STEP(cacti_hip_rows_qkv_rope_cache_f16(T, H, Dh, xa, xb, P(w.pre_norm), g.eps, xb ? x : nullptr, P(w.q), P(w.k),
                                                        P(w.v), cosr, sinr, qr, kc + prev * D * 2, vc + prev * D * 2, st));
-                STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, attn, D, aws, aws_bytes, st));
+                STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, Dh, attn, D, aws, aws_bytes, st));
                 STEP(cacti_hip_gemm_f16(0, 1, T, D, D, 1.f, attn, D, P(w.o), D, 0.f, o, D, st));
                 // x1 = stream + o; post = rms_norm(x1); h = silu(post gate^T) * (post up^T)
                 STEP(cacti_hip_rows_norm_matmul_f16(T, F, D, x, o, P(w.post_norm), g.eps, x1, P(w.gate), P(w.up), h, st));
@@ -711,7 +711,7 @@ CACTI_API int cacti_llama_cached_apply(cacti_llama_cached *k, int64_t prev, int6
                 // scores against the cache, row-causal mask + softmax (in place), P V.  Columns from
                 // `next` on are masked for every row, so only the first Cw of the cap columns are formed.
                 if (fused_attn) {
-                    STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, attn, D, aws, aws_bytes, st));
+                    STEP(cacti_hip_attn_decode_f16(T, H, Dh, next, prev, alpha, qr, D, kc, vc, D, Dh, attn, D, aws, aws_bytes, st));
                 } else {
                     STEP(cacti_hip_gemm_f16_strided_batched(0, 1, H, T, Cw, Dh, alpha, qr, D, Dh, kc, D, Dh, 0.f, s16, H * Cw, Cw, st));
                     STEP(cacti_hip_row_causal_softmax_fwd(T, H, Cw, Cw, prev, s16, s16, st));

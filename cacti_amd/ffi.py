@@ -80,7 +80,7 @@ SIGNATURES = {
     "cacti_hip_rows_norm_matmul_f16": (ci, [i64, i64, i64, vp, vp, vp, f32, vp, vp, vp, vp, vp]),
     "cacti_hip_rows_qkv_rope_cache_f16": (ci, [i64, i64, i64, vp, vp, vp, f32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
     "cacti_hip_attn_decode_workspace": (sz, [i64, i64, i64, i64]),
-    "cacti_hip_attn_decode_f16": (ci, [i64, i64, i64, i64, i64, f32, vp, i64, vp, vp, i64, vp, i64, vp, sz, vp]),
+    "cacti_hip_attn_decode_f16": (ci, [i64, i64, i64, i64, i64, f32, vp, i64, vp, vp, i64, i64, vp, i64, vp, sz, vp]),
     "cacti_hip_append_token_u16": (ci, [vp, i64, vp, i64, vp]),
     "cacti_hip_raw_cast_bf16_f16": (ci, [i64, vp, vp, vp]),
     "cacti_hip_raw_cast_bf16_f32": (ci, [i64, vp, vp, vp]),

@@ -240,15 +240,16 @@ int cacti_hip_rows_qkv_rope_cache_f16(int64_t M, int64_t H, int64_t Dh, const vo
  * block_matmul_scale(q, k_cache^T, alpha) -> f32 -> row-causal mask -> softmax -> f16 ->
  * block_matmul(., v_cache) of src/librarium/llama.rs:895-915 with its rounding points (f16 scores
  * and probabilities, fp32 accumulation, one rounding of the output).  q: [T, ldq] f16 with head h
- * at columns h*Dh..; k_cache, v_cache: [C, ldkv] f16 likewise (C cached positions, those beyond
+ * at columns h*Dh..; k_cache, v_cache: element (position j, head h, d) at j*ldkv + h*head_stride + d
+ * (the reference's [C, H, Dh] layout is ldkv = H*Dh, head_stride = Dh; positions beyond
  * T + initial_row - 1 are not read); out: [T, ldo] f16.  Dh % 4 == 0, Dh <= 100; pointers 8-byte
  * aligned, pitches multiples of 4; C <= 8192.  workspace: cacti_hip_attn_decode_workspace bytes,
  * 16-byte aligned, contents undefined on return. */
 size_t cacti_hip_attn_decode_workspace(int64_t T, int64_t H, int64_t Dh, int64_t C);
 int cacti_hip_attn_decode_f16(int64_t T, int64_t H, int64_t Dh, int64_t C, int64_t initial_row, float alpha,
                               const void *q, int64_t ldq, const void *k_cache, const void *v_cache,
-                              int64_t ldkv, void *out, int64_t ldo, void *workspace, size_t workspace_bytes,
-                              void *stream);
+                              int64_t ldkv, int64_t head_stride, void *out, int64_t ldo, void *workspace,
+                              size_t workspace_bytes, void *stream);
 /* in_tok[pos] += out_tok[last] (u16): the token generated for the last position appended to the
  * input sequence on the device, src/librarium/llama.rs:958-959. */
 int cacti_hip_append_token_u16(void *in_tok, int64_t pos, const void *out_tok, int64_t last, void *stream);

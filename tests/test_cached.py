@@ -128,7 +128,7 @@ def test_decoding_attention_matches_the_oracle_chain(oracle, T, H, Dh, Cc, row0)
     nb = ffi.lib().cacti_hip_attn_decode_workspace(T, H, Dh, Cc)
     ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
     for _ in range(2):
-        ffi.call("cacti_hip_attn_decode_f16", T, H, Dh, Cc, row0, alpha, dq.data_ptr(), D, dk.data_ptr(), dv.data_ptr(), D,
+        ffi.call("cacti_hip_attn_decode_f16", T, H, Dh, Cc, row0, alpha, dq.data_ptr(), D, dk.data_ptr(), dv.data_ptr(), D, Dh,
                  out.data_ptr(), D, ws.data_ptr(), nb, None)
         got = out.cpu().numpy().view(np.float16)
         assert_parity(got, want, "attn decode")
