@@ -29,17 +29,25 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
     if (n >= N) return;
     const int nchunk = D / 8;
     const half_t *xr = x + n * D;
-    h8 xv[CH];
+    // All loads of the row are issued first and unconditionally (chunks past the row re-read its
+    // last chunk): a load inside `if (ch < nchunk)` is waited for at the end of that branch, which
+    // makes the CH loads of a lane CH round trips.
+    h8 xv[CH], bv[CH], wv[CH];
+#pragma unroll
+    for (int c = 0; c < CH; c++) {
+        const int ch = min(c * 64 + lane, nchunk - 1);
+        xv[c] = ld8(xr + ch * 8);
+        if (x2) bv[c] = ld8(x2 + n * D + ch * 8);         // uniform over the launch
+        wv[c] = ld8(w + ch * 8);
+    }
     float ss = 0.f;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int ch = c * 64 + lane;
         if (ch < nchunk) {
-            xv[c] = ld8(xr + ch * 8);
             if (x2) {
-                const h8 bv = ld8(x2 + n * D + ch * 8);
 #pragma unroll
-                for (int i = 0; i < 8; i++) xv[c].v[i] = f2h(h2f(xv[c].v[i]) + h2f(bv.v[i]));
+                for (int i = 0; i < 8; i++) xv[c].v[i] = f2h(h2f(xv[c].v[i]) + h2f(bv[c].v[i]));
                 st8(sum + n * D + ch * 8, xv[c]);
             }
 #pragma unroll
@@ -57,9 +65,9 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
     for (int c = 0; c < CH; c++) {
         const int ch = c * 64 + lane;
         if (ch < nchunk) {
-            h8 wv = ld8(w + ch * 8), o;
+            h8 o;
 #pragma unroll
-            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv.v[i]) * (h2f(xv[c].v[i]) * rinv));
+            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv[c].v[i]) * (h2f(xv[c].v[i]) * rinv));
             st8(yr + ch * 8, o);
         }
     }
@@ -86,15 +94,17 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
 
     if (live) {
         const half_t *xr = x + n * D, *gr = dy + n * D;
-        h8 xv[CH], gv[CH];
+        // every load of the row up front and unconditional (see the forward kernel)
+        half_t *or_ = dx + n * D;
+        h8 xv[CH], gv[CH], wv[CH], old[CH];
         float ss = 0.f;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
-            const int ch = c * 64 + lane;
-            if (ch < nchunk) {
-                xv[c] = ld8(xr + ch * 8);
-                gv[c] = ld8(gr + ch * 8);
-            }
+            const int ch = min(c * 64 + lane, nchunk - 1);
+            xv[c] = ld8(xr + ch * 8);
+            gv[c] = ld8(gr + ch * 8);
+            wv[c] = ld8(w + ch * 8);
+            old[c] = ld8(or_ + ch * 8);                       // used only when dx accumulates
         }
 #pragma unroll
         for (int c = 0; c < CH; c++) {
@@ -115,13 +125,12 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         for (int c = 0; c < CH; c++) {
             const int ch = c * 64 + lane;
             if (ch < nchunk) {
-                h8 wv = ld8(w + ch * 8);
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     float xf = h2f(xv[c].v[i]), du = h2f(gv[c].v[i]);
                     float t = xf * rinv;
                     dwp[c][i] = rnd16(du * t);
-                    float dt = du * h2f(wv.v[i]);
+                    float dt = du * h2f(wv[c].v[i]);
                     sdx += dt * xf;
                     gv[c].v[i] = f2h(dt * rinv);        // c1, kept in place of dy
                     // dt is needed no further: c2 depends only on the row sum
@@ -132,19 +141,17 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         const float dr = -sdx / (r * r);
         const float ds = dr / (r + r);
         const float dsq = ds / (float)D;
-        half_t *or_ = dx + n * D;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int ch = c * 64 + lane;
             if (ch < nchunk) {
-                h8 o, old;
-                if (dx_acc) old = ld8(or_ + ch * 8);
+                h8 o;
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     float xf = h2f(xv[c].v[i]);
                     float c1 = h2f(gv[c].v[i]);
                     float c2 = rnd16(dsq * (xf + xf));
-                    float base = dx_acc ? rnd16(h2f(old.v[i]) + c1) : c1;
+                    float base = dx_acc ? rnd16(h2f(old[c].v[i]) + c1) : c1;
                     o.v[i] = f2h(base + c2);
                 }
                 st8(or_ + ch * 8, o);
