@@ -301,6 +301,7 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nbl
     }
     hipStream_t st = (hipStream_t)stream;
     p.win = 0;
+    p.ztab = 0;
     if (vec >= 4 && !ta && tb && K <= 128 && beta == 0.f && tri <= 1)
         return gemm_nt_smallk_launch(p, nblk, st);
     // one to four rows against a weight matrix (decoding): a stream over B
@@ -333,6 +334,51 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nbl
     if (!ta && tb) return launch_vec<false, true>(vec, p, nblk, st);
     if (ta && !tb) return launch_vec<true, false>(vec, p, nblk, st);
     return launch_vec<true, true>(vec, p, nblk, st);
+}
+
+// Pointer-array batch (cublasGemmBatchedEx shape): the products must have one shape; up to
+// kMaxPtrBatch of them share a launch when every operand is 16-byte aligned, otherwise they run
+// one after another.
+CACTI_API int cacti_hip_gemm_f16_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N, int64_t K,
+                                         float alpha, const void *const *A, int64_t lda, const void *const *B,
+                                         int64_t ldb, float beta, void *const *C, int64_t ldc, void *stream)
+{
+    CACTI_REQUIRE(nblk > 0 && A && B && C, CACTI_E_INVALID, "gemm_batched: null pointer array or empty batch");
+    for (int64_t z = 0; z < nblk; z++)
+        CACTI_REQUIRE(A[z] && B[z] && C[z], CACTI_E_INVALID, "gemm_batched: null operand in block %lld", (long long)z);
+    const int64_t ca = ta ? M : K, cb = tb ? K : N;
+    bool fast = M > 0 && N > 0 && K > 0 && (beta == 0.f || beta == 1.f) && mult(ca, 8) && mult(cb, 8) && mult(N, 8) &&
+                mult(lda, 8) && mult(ldb, 8) && mult(ldc, 8) && lda >= ca && ldb >= cb && ldc >= N && K > 128;
+    for (int64_t z = 0; z < nblk && fast; z++) fast = aligned(A[z], 16) && aligned(B[z], 16) && aligned(C[z], 16);
+    for (int64_t z0 = 0; z0 < nblk; z0 += kMaxPtrBatch) {
+        const int64_t cnt = nblk - z0 < kMaxPtrBatch ? nblk - z0 : kMaxPtrBatch;
+        if (!fast || cnt == 1) {
+            for (int64_t z = z0; z < z0 + cnt; z++) {
+                const int rc = cacti_hip_gemm_f16(ta, tb, M, N, K, alpha, A[z], lda, B[z], ldb, beta, C[z], ldc, stream);
+                if (rc) return rc;
+            }
+            continue;
+        }
+        GemmArgs p;
+        p.M = M; p.N = N; p.K = K; p.alpha = alpha; p.beta = beta;
+        p.A = (const half_t *)A[z0]; p.lda = lda; p.sa = 0;
+        p.B = (const half_t *)B[z0]; p.ldb = ldb; p.sb = 0;
+        p.C = (half_t *)C[z0]; p.ldc = ldc; p.sc = 0;
+        p.tiles_m = (int)((M + BM - 1) / BM);
+        p.tiles_n = (int)((N + BN - 1) / BN);
+        p.tri = 0;
+        p.win = 0;
+        p.ztab = 1;
+        for (int64_t z = 0; z < kMaxPtrBatch; z++) {
+            const int64_t zz = z0 + (z < cnt ? z : 0);
+            p.za[z] = (const half_t *)A[zz] - p.A;
+            p.zb[z] = (const half_t *)B[zz] - p.B;
+            p.zc[z] = (half_t *)C[zz] - p.C;
+        }
+        const int rc = gemm_mfma_launch(ta, tb, p, cnt, 8, -1, (hipStream_t)stream);
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 CACTI_API int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N,

@@ -30,7 +30,12 @@ struct GemmArgs {
     // below their first column (column window); set by the entry point when A is 16-byte
     // aligned and B, C are only 8-byte aligned because of their batch stride
     int win;
+    // 1: the blocks of the batch are separate arrays: block z starts at A + za[z], B + zb[z],
+    // C + zc[z] (element offsets) instead of z times the batch strides; at most kMaxPtrBatch blocks
+    int ztab;
+    int64_t za[4], zb[4], zc[4];
 };
+constexpr int kMaxPtrBatch = 4;
 constexpr int kTriPad = 256;
 
 // tile < 0: chosen by shape

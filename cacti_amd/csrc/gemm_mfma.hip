@@ -573,7 +573,7 @@ gemm_mfma_kernel(GemmArgs p)
     if (p.tri == 2) nk = min(nk, (int)((m0 + BM + BK - 1) / BK));
     if (p.tri == 3) kt0 = (int)(m0 / BK);
 
-    const half_t *A = p.A + bz * p.sa;
+    const half_t *A = p.A + (p.ztab ? p.za[bz] : bz * p.sa);
     // column window (p.win): the [k][n] operand B and C of block bz start 8 bytes off a 16-byte
     // boundary when bz * sb is an odd multiple of 4 (head_dim 100).  Both are then addressed
     // from the boundary before: column `shift` of this view is the block's column 0, columns
@@ -581,8 +581,8 @@ gemm_mfma_kernel(GemmArgs p)
     // and never stored.
     const int shift = p.win ? (int)((bz * p.sb) & 7) : 0;
     const int64_t nw = p.N + shift;                               // end of the window
-    const half_t *B = p.B + bz * p.sb - shift;
-    half_t *C = p.C + bz * p.sc - shift;
+    const half_t *B = p.B + (p.ztab ? p.zb[bz] : bz * p.sb) - shift;
+    half_t *C = p.C + (p.ztab ? p.zc[bz] : bz * p.sc) - shift;
     // tile origins: &op[row0][0] for a k-contiguous operand, &op[0][row0] for a strided one
     const half_t *Ao = TA ? A + m0 : A + m0 * p.lda;
     const half_t *Bo = TB ? B + n0 * p.ldb : B + n0;
@@ -1053,7 +1053,8 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             // LDS buffers (-5 us per launch against the register path with 8 waves)
             if (p.win) tile = 7;
             static const bool no_split = getenv("CACTI_GEMM_NO_SPLIT") != nullptr;
-            if (nblk == 1 && p.M >= 1024 && p.N >= 1024) {
+            // (a pointer-table batch is a handful of whole products: planned like a single one)
+            if ((nblk == 1 || p.ztab) && p.M >= 1024 && p.N >= 1024) {
                 if (no_direct) {
                     tile = ta ? 0 : 1;
                 } else if (!ta) {

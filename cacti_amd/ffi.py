@@ -41,6 +41,7 @@ SIGNATURES = {
     "cacti_hip_event_sync": (ci, [vp]),
     "cacti_hip_event_elapsed_ms": (ci, [vp, vp, C.POINTER(f32)]),
     "cacti_hip_gemm_f16": (ci, [ci, ci, i64, i64, i64, f32, vp, i64, vp, i64, f32, vp, i64, vp]),
+    "cacti_hip_gemm_f16_batched": (ci, [ci, ci, i64, i64, i64, i64, f32, vp, i64, vp, i64, f32, vp, i64, vp]),
     "cacti_hip_gemm_f16_strided_batched": (ci, [ci, ci, i64, i64, i64, i64, f32, vp, i64, i64, vp,
                                                 i64, i64, f32, vp, i64, i64, vp]),
     "cacti_hip_gemm_f16_strided_batched_tri": (ci, [ci, ci, i64, i64, i64, i64, f32, vp, i64, i64,

@@ -47,6 +47,22 @@ def gemm(a, b, ta=False, tb=False, alpha=1.0, beta=0.0, out=None):
     return out
 
 
+def gemm_batched(As, Bs, ta=False, tb=False, alpha=1.0, beta=0.0, outs=None):
+    """Pointer-array batch: outs[z] = f16(alpha op(As[z]) op(Bs[z]) + beta outs[z]), one shape."""
+    import ctypes as C
+    n = len(As)
+    a, b = As[0], Bs[0]
+    M, K = (a.shape[1], a.shape[0]) if ta else a.shape
+    N = b.shape[0] if tb else b.shape[1]
+    if outs is None:
+        assert beta == 0.0
+        outs = [torch.empty((M, N), dtype=F16, device=a.device) for _ in range(n)]
+    arr = lambda ts: C.cast((C.c_void_p * n)(*[t.data_ptr() for t in ts]), C.c_void_p)
+    ffi.call("cacti_hip_gemm_f16_batched", int(ta), int(tb), n, M, N, K, alpha, arr(As), a.stride(0), arr(Bs),
+             b.stride(0), beta, arr(outs), outs[0].stride(0), _stream())
+    return outs
+
+
 def gemm_strided_batched(ta, tb, nblk, M, N, K, alpha, a, lda, sa, b, ldb, sb, beta, c, ldc, sc,
                          tri=0):
     """tri: 0 dense; 1 only tril(C) wanted (rest unwritten); 2 A = tril; 3 A^T with A = tril."""

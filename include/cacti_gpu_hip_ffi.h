@@ -107,6 +107,15 @@ int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, 
                                        int64_t stride_b, float beta, void *C, int64_t ldc,
                                        int64_t stride_c, void *stream);
 
+/* Pointer-array batch, the shape of cublasGemmBatchedEx (cacti_gpu_cu_ffi/src/lib.rs:793-885):
+ * nblk products of one shape, block z on A[z], B[z], C[z] (host arrays of device pointers, read
+ * before the call returns).  With every operand 16-byte aligned up to four products share a launch
+ * (three projections of 200 tiles each fill the 256 CUs far better together than one after another);
+ * otherwise they run one after another.  Results equal those of nblk calls of cacti_hip_gemm_f16. */
+int cacti_hip_gemm_f16_batched(int ta, int tb, int64_t nblk, int64_t M, int64_t N, int64_t K,
+                               float alpha, const void *const *A, int64_t lda, const void *const *B,
+                               int64_t ldb, float beta, void *const *C, int64_t ldc, void *stream);
+
 /* The same with the triangular structure of causal attention made explicit, so that the
  * half of each sequence x sequence product that the causal mask discards is never computed:
  *   tri = 0  none (identical to the call above);

@@ -329,6 +329,36 @@ def test_gemm_few_rows_streams_the_weights(ops, oracle, M, N, K, pad):
         assert exact_frac(got, want) > 0.98
 
 
+@pytest.mark.parametrize("ta,tb,n,M,N,K,off", [(0, 1, 3, 1032, 1096, 192, 0), (1, 0, 2, 1096, 1032, 128, 0), (0, 0, 5, 1024, 1024, 192, 0),
+                                             (0, 1, 3, 1032, 1096, 192, 4), (0, 1, 2, 64, 72, 40, 0)])
+def test_gemm_pointer_array_batch(ops, oracle, ta, tb, n, M, N, K, off):
+    """Products of one shape on separate arrays: one launch for up to four of them (direct-load
+    tiles, ragged edges), one after another when an operand is not 16-byte aligned (off) or the
+    shape is small; every block against the oracle, with and without accumulation."""
+    say("gemm batched", ta, tb, n, M, N, K, off)
+    r = rng(300 + n + M + K + off)
+    As = [randn16(r, (K, M) if ta else (M, K)) for _ in range(n)]
+    Bs = [randn16(r, (N, K) if tb else (K, N), 0.1) for _ in range(n)]
+    C0 = [randn16(r, (M, N)) for _ in range(n)]
+    shared_a = dev(As[0])
+
+    def place(x):                        # device copy starting `off` elements past an aligned address
+        buf = torch.empty(x.size + 8, dtype=torch.float16, device="cuda")
+        v = buf[off:off + x.size].view(x.shape)
+        v.copy_(dev(x))
+        return v
+    for alpha, beta in [(1.0, 0.0), (0.5, 1.0)]:
+        dA = [shared_a if z == 0 else place(As[z]) for z in range(n)]
+        dB = [place(Bs[z]) for z in range(n)]
+        dC = [dev(C0[z]) for z in range(n)]
+        ops.gemm_batched(dA, dB, bool(ta), bool(tb), alpha, beta, dC)
+        for z in range(n):
+            want = oracle.matmul(ta, tb, As[z], Bs[z], alpha, beta, C0[z])
+            assert_parity(host(dC[z]), want, "gemm batched %d" % z)
+            single = host(ops.gemm(dA[z], dB[z], bool(ta), bool(tb), alpha, beta, dev(C0[z])))
+            assert np.array_equal(host(dC[z]).view(np.uint16), single.view(np.uint16)), z
+
+
 @pytest.mark.parametrize("case", ["fwd", "dgrad", "wgrad"])
 def test_gemm_projection_shapes(ops, oracle, case):
     """The three GEMMs of one projection at a reduced token count (oracle finishes in seconds)."""
