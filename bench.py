@@ -710,6 +710,71 @@ def run_decode(args):
     return out
 
 
+def run_cycle(args):
+    """The whole training cycle of the reference's example with one cycle per minibatch
+    (examples/open_llama_3b_train.rs:223-531): fwd + loss + bwd, the numerical-health digests of every
+    parameter and gradient, and the AdamW32 step on every parameter but the embedding; value = tokens
+    per second over complete cycles, everything on the device (the reference runs the optimiser on the
+    CPU)."""
+    import torch
+    from cacti_amd.runtime import Ctx, Llama
+    cfg = dict(LLAMA_3B)
+    if args.layers is not None:
+        cfg["L"] = args.layers
+    opt = dict(grad_scale=1024.0, lr=2.0e-5, wd=0.1, a1=0.1, a2=0.05, eps=1.0e-5)
+    ctx = Ctx(0, 0, True)
+    model = Llama(ctx, **cfg)
+    synth_params(model)
+    tok, lm_tok, scale = synth_inputs(cfg)
+    model.adamw_init()
+
+    def cycle(it):
+        model.step(tok, lm_tok, scale, want_loss=False)
+        gh, gn = model.digests(of_grads=True)
+        ph, pn = model.digests(of_grads=False)
+        model.adamw_step(it, skip_embed=True, **opt)
+        return gh, gn, ph, pn
+    it = 1
+    for _ in range(max(args.warmup, 1)):
+        cycle(it)
+        it += 1
+    ctx.sync()
+    torch.cuda.synchronize()
+    parts = {"step": 0.0, "digests": 0.0, "adamw": 0.0}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        gh, gn, ph, pn = cycle(it)
+        it += 1
+    ctx.sync()
+    dt = (time.perf_counter() - t0) / args.steps
+    assert int(gn.sum()) == 0 and int(pn.sum()) == 0 and int(gh[:, 255].sum()) == 0, "non-finite values"
+    # the three parts timed apart (each synchronised), for the breakdown only
+    for _ in range(2):
+        ta = time.perf_counter()
+        model.step(tok, lm_tok, scale, want_loss=False)
+        ctx.sync()
+        tb = time.perf_counter()
+        model.digests(of_grads=True)
+        model.digests(of_grads=False)
+        tc = time.perf_counter()
+        model.adamw_step(it, skip_embed=True, **opt)
+        it += 1
+        ctx.sync()
+        td = time.perf_counter()
+        parts = {"step": (tb - ta) * 1e3, "digests": (tc - tb) * 1e3, "adamw": (td - tc) * 1e3}
+    out = {"metric": "training-cycle tokens/sec: fwd+bwd, digests of parameters and gradients, AdamW32 step; 1 GPU",
+           "value": cfg["S"] / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 1),
+           "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+           "data": "synthetic (seeded N(0,0.02) weights, uniform token ids)",
+           "config": {"workload": "OpenLLaMA-3B-shaped training cycle: %d layers, batch 1, seq %d, one cycle per "
+                                  "minibatch, f32 master weights and moments on the device" % (cfg["L"], cfg["S"]),
+                      "parts_ms": parts},
+           "roofline": None, "cpu_baseline": None}
+    model.close()
+    ctx.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -719,7 +784,7 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest", "decode"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest", "decode", "cycle"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -737,6 +802,8 @@ def main():
         out = run_ingest(args)
     elif args.workload == "decode":
         out = run_decode(args)
+    elif args.workload == "cycle":
+        out = run_cycle(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)

@@ -214,6 +214,49 @@ def test_adamw_steps_between_cycles(oracle, capped):
     m.close(); ctx.close()
 
 
+def test_training_cycles_follow_the_oracle(oracle):
+    """The example's loop end to end (examples/open_llama_3b_train.rs:223-531 with one cycle per
+    minibatch): cycle -> AdamW32 step on every parameter but the embedding -> cycle ...; four cycles on
+    the device against four cycles of the oracle (its own gradients, its own optimiser): per-cycle
+    losses agree, the loss of the repeated batch goes down, and the parameters stay together."""
+    opt = dict(grad_scale=1024.0, lr=1.0e-3, wd=0.1, a1=0.1, a2=0.05, eps=1.0e-5)
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=9, norm_mean=1.0, grad_scale=1024.0)
+    ctx, m = _model(cfg)
+    m.put_params_flat(flat)
+    m.adamw_init()
+    names = [n for n, _ in m.params]
+    o_p = {n: v.copy() for n, v in oracle.split_params(cfg, flat).items()}
+    o_master = {n: o_p[n].astype(np.float32) for n in names}
+    o_avg = {n: np.zeros(o_p[n].shape, np.float32) for n in names}
+    o_avg2 = {n: np.zeros(o_p[n].shape, np.float32) for n in names}
+    live = scale > 0
+    g_losses, o_losses = [], []
+    for it in range(1, 5):
+        g_loss = m.step(tok, lm_tok, scale)
+        m.adamw_step(it, skip_embed=True, **opt)
+        oflat = np.concatenate([o_p[n].reshape(-1) for n in names])
+        ref = oracle.llama_step(cfg, oflat, tok, lm_tok, scale)
+        og = oracle.split_params(cfg, ref["grad"])
+        sc = oracle.adamw32_scalars(it, **opt)
+        for n in names[1:]:
+            o_avg[n], o_avg2[n], o_master[n], o_p[n] = oracle.adamw32_step(og[n], o_avg[n], o_avg2[n], o_master[n], sc)
+        g_losses.append(float(g_loss[live].mean()))
+        o_losses.append(float(ref["loss"][live].mean()))
+        assert abs(g_losses[-1] - o_losses[-1]) < 2e-3 * abs(o_losses[-1]), (it, g_losses, o_losses)
+    assert g_losses[-1] < g_losses[0] - 0.05 and o_losses[-1] < o_losses[0] - 0.05, (g_losses, o_losses)
+    for i, n in enumerate(names):
+        got, want = m.param(i), o_p[n]
+        if n == "embed":
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+            continue
+        # the step of one cycle is ~lr per element: two runs whose gradients differ in the last
+        # bits stay within a small fraction of the total movement
+        moved = np.abs(want.astype(np.float32) - oracle.split_params(cfg, flat)[n].astype(np.float32)).max()
+        diff = np.abs(got.astype(np.float32) - want.astype(np.float32)).max()
+        assert moved > 1e-3 and diff <= 0.35 * moved, (n, moved, diff)
+    m.close(); ctx.close()
+
+
 def test_adamw_step_before_init_is_a_state_error(oracle):
     from cacti_amd.ffi import CactiError
     cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=6)
