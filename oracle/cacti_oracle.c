@@ -1,5 +1,6 @@
 /*
- * cacti_oracle.c -- CPU restatement of the reference's LLaMA forward + backward path.
+ * cacti_oracle.c -- CPU restatement of the reference's LLaMA forward + backward path and of
+ * the thunks either side of it (digests, AdamW32, bf16 casts, the KV-cached forward pass).
  *
  * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE.  It is the checker that the
  * HIP kernels are compared against and the "CPU port" timed as a baseline; no
@@ -22,9 +23,18 @@
  *     (th_silu_f16, th_logistic_f16, th_bmul_f16_tab, vjp_bmul_row);
  *   - the summation order of cross-row reductions delivered in f16
  *     (vjp_bmul_row = RMSNorm dw, vjp_outer_select = embedding scatter-add);
- *   - ulp-level behaviour of exp/log/sqrt/cos/sin/pow.
+ *   - ulp-level behaviour of exp/log/sqrt/cos/sin/pow;
+ *   - whether the optimiser lambdas (th_online_*) are contracted into fused
+ *     multiply-adds by the reference's back end (<= 1 ulp of f32 per operation),
+ *     and f32::powi's exact value in oracle_adamw32_scalars;
+ *   - th_raw_cast_f16_bf16 on a signalling NaN (quieted here first).
  * Everything else is pinned in tests/ by closed forms, fp64 finite differences,
- * adjoint identities, brute force and torch.autograd on the composed model.
+ * adjoint identities, brute force and torch.autograd on the composed model;
+ * the digests by all 65536 f16 patterns against their values, the optimiser
+ * against torch.optim.AdamW in float64 and closed forms of the averages, the raw
+ * casts by all 16-bit patterns against numpy, and the cached forward pass
+ * against this file's own full forward pass (one call reproduces its logits bit
+ * for bit, any split into chunks reproduces the one-call result bit for bit).
  */
 #include <math.h>
 #include <stdint.h>
