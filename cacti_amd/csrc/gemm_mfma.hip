@@ -940,6 +940,7 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
         case 5: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1, 2, true>(p, nblk, st);
         case 6: return launch_cfg<TA, TB, 256, 192, 4, 2, 8, false, 1, 2, true>(p, nblk, st);
         case 7: return launch_cfg<TA, TB, 128, 128, 2, 4, 8, false, 1, 3, true>(p, nblk, st);
+        case 8: return launch_cfg<TA, TB, 64, 64, 2, 2, 8, false, 1, 3, true>(p, nblk, st);
         default: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
     }
 }
@@ -1006,7 +1007,10 @@ int launch_auto(int tile, int64_t cols_main, int align, const GemmArgs &p, int64
         b.B = p.B + (TB ? a.N * p.ldb : a.N);
         b.C = p.C + a.N;
         const int rc = launch_tile<TA, TB>(tile, align, a, nblk, st);
-        return rc ? rc : launch_tile<TA, TB>(3, align, b, nblk, st);
+        // the remaining columns on 64 x 64 tiles loaded straight into LDS, three buffers (the
+        // register path with two stages: 23.7 -> ~20 us for 448 columns at K = 3200)
+        static const int rem_tile = getenv("CACTI_GEMM_REM_TILE") ? atoi(getenv("CACTI_GEMM_REM_TILE")) : 8;
+        return rc ? rc : launch_tile<TA, TB>(rem_tile, align, b, nblk, st);
     }
     return launch_tile<TA, TB>(tile, align, p, nblk, st);
 }
