@@ -25,34 +25,12 @@
 
 #include "../../include/cacti_hip_runtime.h"
 #include "common.h"
+#include "ingest_internal.h"
 #include "runtime.h"
 
 using namespace cacti;
 
 namespace {
-
-struct TensorEntry {
-    std::string dtype;                  // as spelled in the file: "F16", "BF16", "F32", ...
-    std::vector<int64_t> shape;
-    int file = 0;
-    uint64_t off = 0, eoff = 0;         // absolute byte range in the file
-};
-
-struct MappedFile {
-    std::string path;
-    int fd = -1;
-    void *base = nullptr;
-    size_t size = 0;
-};
-
-size_t dtype_bytes(const std::string &d)
-{
-    if (d == "F64" || d == "I64" || d == "U64") return 8;
-    if (d == "F32" || d == "I32" || d == "U32") return 4;
-    if (d == "F16" || d == "BF16" || d == "I16" || d == "U16") return 2;
-    if (d == "I8" || d == "U8" || d == "BOOL" || d == "F8_E4M3" || d == "F8_E5M2") return 1;
-    return 0;
-}
 
 // ---- the little JSON the header needs: objects, arrays, strings, non-negative integers ----
 struct Json {
@@ -178,44 +156,14 @@ struct Json {
 
 }  // namespace
 
-struct cacti_tensors_dir {
-    std::string path;
-    std::vector<MappedFile> files;
-    std::vector<std::string> serial_key;                 // order of appearance
-    std::map<std::string, TensorEntry> tensors;          // byte-wise sorted names (BTreeMap<SmolStr, ..>)
-    std::vector<const std::string *> sorted;             // index -> name
-
-    ~cacti_tensors_dir()
-    {
-        for (MappedFile &f : files) {
-            if (f.base && f.base != MAP_FAILED) munmap(f.base, f.size);
-            if (f.fd >= 0) close(f.fd);
-        }
-    }
-};
-
 namespace {
 
 // one file: map it, parse its header, add its tensors (TensorsDir::_reopen, src/util/safetensor.rs:88-113)
 int add_file(cacti_tensors_dir *d, const std::string &path)
 {
     MappedFile mf;
-    mf.path = path;
-    mf.fd = open(path.c_str(), O_RDONLY);
-    CACTI_REQUIRE(mf.fd >= 0, CACTI_E_IO, "tensors_dir: cannot open %s", path.c_str());
-    struct stat st;
-    if (fstat(mf.fd, &st) != 0 || st.st_size < 8) {
-        close(mf.fd);
-        set_error("tensors_dir: %s is shorter than a safetensors header", path.c_str());
-        return CACTI_E_FORMAT;
-    }
-    mf.size = (size_t)st.st_size;
-    mf.base = mmap(nullptr, mf.size, PROT_READ, MAP_PRIVATE, mf.fd, 0);
-    if (mf.base == MAP_FAILED) {
-        close(mf.fd);
-        set_error("tensors_dir: cannot map %s", path.c_str());
-        return CACTI_E_IO;
-    }
+    const int rc = ingest_map_file(path, 8, "tensors_dir", &mf);
+    if (rc) return rc;
     const int file_idx = (int)d->files.size();
     d->files.push_back(mf);
     const unsigned char *b = static_cast<const unsigned char *>(mf.base);
@@ -268,7 +216,7 @@ int add_file(cacti_tensors_dir *d, const std::string &path)
                           "tensors_dir: %s: tensor %s lacks dtype, shape or data_offsets", path.c_str(), name.c_str());
             uint64_t elems = 1;
             for (int64_t v : e.shape) elems *= (uint64_t)v;
-            const size_t esz = dtype_bytes(e.dtype);
+            const size_t esz = ingest_dtype_bytes(e.dtype);
             CACTI_REQUIRE(esz != 0, CACTI_E_FORMAT, "tensors_dir: %s: tensor %s has unknown dtype %s", path.c_str(),
                           name.c_str(), e.dtype.c_str());
             // packed_span_bytes == size, src/util/safetensor.rs:127-132
@@ -436,6 +384,39 @@ CACTI_API int cacti_llama_load_tensors_dir(cacti_llama *model, cacti_tensors_dir
 
 // the pieces llama.cpp needs of a directory
 namespace cacti {
+
+size_t ingest_dtype_bytes(const std::string &d)
+{
+    if (d == "F64" || d == "I64" || d == "U64") return 8;
+    if (d == "F32" || d == "I32" || d == "U32") return 4;
+    if (d == "F16" || d == "BF16" || d == "I16" || d == "U16") return 2;
+    if (d == "I8" || d == "U8" || d == "BOOL" || d == "F8_E4M3" || d == "F8_E5M2") return 1;
+    return 0;
+}
+
+int ingest_map_file(const std::string &path, size_t min_size, const char *who, MappedFile *mf)
+{
+    mf->path = path;
+    mf->fd = open(path.c_str(), O_RDONLY);
+    CACTI_REQUIRE(mf->fd >= 0, CACTI_E_IO, "%s: cannot open %s", who, path.c_str());
+    struct stat st;
+    if (fstat(mf->fd, &st) != 0 || (size_t)st.st_size < min_size) {
+        close(mf->fd);
+        mf->fd = -1;
+        set_error("%s: %s is shorter than the %zu bytes its format needs", who, path.c_str(), min_size);
+        return CACTI_E_FORMAT;
+    }
+    mf->size = (size_t)st.st_size;
+    mf->base = mmap(nullptr, mf->size, PROT_READ, MAP_PRIVATE, mf->fd, 0);
+    if (mf->base == MAP_FAILED) {
+        close(mf->fd);
+        mf->fd = -1;
+        mf->base = nullptr;
+        set_error("%s: cannot map %s", who, path.c_str());
+        return CACTI_E_IO;
+    }
+    return 0;
+}
 
 int tensors_dir_keys(cacti_tensors_dir *dir, std::vector<const char *> *keys)
 {

@@ -121,6 +121,7 @@ SIGNATURES = {
     "cacti_llama_grad_get": (ci, [vp, ci, vp, sz]),
     "cacti_llama_digests": (ci, [vp, ci, vp, vp]),
     "cacti_tensors_dir_open": (ci, [C.c_char_p, pvp]),
+    "cacti_pickle_dir_open": (ci, [C.c_char_p, C.c_char_p, pvp]),
     "cacti_tensors_dir_close": (ci, [vp]),
     "cacti_tensors_dir_count": (ci, [vp]),
     "cacti_tensors_dir_entry": (ci, [vp, ci, C.c_char_p, sz, C.c_char_p, sz, C.POINTER(ci), C.POINTER(i64), pvp,

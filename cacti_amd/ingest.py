@@ -1,5 +1,6 @@
-"""Host side of weight ingest: TensorsDir (src/util/safetensor.rs:45-160) and CellMatcher
-(src/util/cell.rs:47-112) through the C ABI of include/cacti_hip_runtime.h."""
+"""Host side of weight ingest: TensorsDir (src/util/safetensor.rs:45-160), PickleDir
+(src/util/safepickle.rs:52-195) and CellMatcher (src/util/cell.rs:47-112) through the C ABI of
+include/cacti_hip_runtime.h."""
 import ctypes as C
 
 import numpy as np
@@ -17,13 +18,16 @@ class TensorsDir:
     def __init__(self, path):
         self._d = C.c_void_p()
         ffi.call("cacti_tensors_dir_open", str(path).encode(), C.byref(self._d))
+        self._read_entries()
+
+    def _read_entries(self):
         self.entries = {}             # name -> (dtype string, shape, address, bytes)
         name, dt = C.create_string_buffer(512), C.create_string_buffer(16)
         for i in range(ffi.lib().cacti_tensors_dir_count(self._d)):
             nd, shp, ptr, nb = C.c_int(), (C.c_int64 * 8)(), C.c_void_p(), C.c_uint64()
             ffi.call("cacti_tensors_dir_entry", self._d, i, name, 512, dt, 16, C.byref(nd), shp, C.byref(ptr),
                      C.byref(nb))
-            self.entries[name.value.decode()] = (dt.value.decode(), tuple(shp[k] for k in range(nd.value)),
+            self.entries[name.value.decode("utf-8", "surrogateescape")] = (dt.value.decode(), tuple(shp[k] for k in range(nd.value)),
                                                  ptr.value, nb.value)
 
     def keys(self):
@@ -39,6 +43,16 @@ class TensorsDir:
         if self._d:
             ffi.lib().cacti_tensors_dir_close(self._d)
             self._d = None
+
+
+class PickleDir(TensorsDir):
+    """PickleDir::open / open_with_prefix + get: the tensors of pytorch_model.bin (or its shards), found
+    by scanning the pickle without executing it; same table, same accessors as TensorsDir."""
+
+    def __init__(self, path, prefix=None):
+        self._d = C.c_void_p()
+        ffi.call("cacti_pickle_dir_open", str(path).encode(), prefix.encode() if prefix else None, C.byref(self._d))
+        self._read_entries()
 
 
 def _rule(pat):

@@ -169,7 +169,7 @@ class Llama:
         return self.ctx.cell_get(cell.value, np.float16, self.params[i][1])
 
     def load_tensors_dir(self, tensors_dir):
-        """Stores every tensor of an open ingest.TensorsDir that Llama::match_pickle_dir's rules match
+        """Stores every tensor of an open ingest.TensorsDir or ingest.PickleDir that Llama::match_pickle_dir's rules match
         into its parameter (src/librarium/llama.rs:284-302); returns how many were matched."""
         n = C.c_int(0)
         ffi.call("cacti_llama_load_tensors_dir", self._m, tensors_dir._d, C.byref(n))

@@ -138,6 +138,19 @@ int cacti_tensors_dir_count(cacti_tensors_dir *dir);
 int cacti_tensors_dir_entry(cacti_tensors_dir *dir, int i, char *name, size_t name_cap, char *dtype,
                             size_t dtype_cap, int *ndim, int64_t *shape8, const void **data,
                             uint64_t *bytes);
+/* PickleDir::open / open_with_prefix / get (src/util/safepickle.rs:52-195), the reader the training
+ * example opens its checkpoint with (examples/open_llama_3b_train.rs:91).  `path` is one torch
+ * checkpoint file, or a directory holding <prefix>.bin or the shards <prefix>-*-of-*.bin (sorted);
+ * prefix NULL or "" means "pytorch_model".  Each file is a ZIP archive (ZIP64 included) whose
+ * data.pkl is scanned without executing anything; every top-level entry of the state dictionary
+ * that is a tensor (bare or wrapped as a parameter) joins the table.  The handle is the one
+ * tensors_dir_open returns: count, entry, close and llama_load_tensors_dir apply unchanged, with
+ * dtypes spelled as in safetensors ("F16", "BF16", "F32", ...).  As in the reference, a tensor whose
+ * strides are not the packed ones is refused (CACTI_E_NOTIMPL), as is a storage type outside
+ * src/cell/mod.rs:1553-1574; a first byte that is not 64-byte aligned, a tensor that does not fit
+ * its storage, a duplicate name, a legacy (non-ZIP) file or an unknown pickle opcode is
+ * CACTI_E_FORMAT. */
+int cacti_pickle_dir_open(const char *path, const char *prefix, cacti_tensors_dir **dir);
 /* CellMatcher::match_: rule r (components separated by '/', "#12" = the integer 12, anything else
  * a string) takes the first key, in sorted order and not taken by an earlier rule, whose
  * '.'-separated tokens consume the rule left to right: an integer needs a token equal to its
