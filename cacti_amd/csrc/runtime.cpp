@@ -190,8 +190,9 @@ static void host_quiesce(Cell &c)
 }
 static void host_mark_busy(Cell &c, hipStream_t st)
 {
-    if (!c.h_busy) hipEventCreateWithFlags(&c.h_busy, hipEventDisableTiming);
-    hipEventRecord(c.h_busy, st);
+    // without an event to wait on later, wait now: the host buffer must never be handed out mid-copy
+    if (!c.h_busy && hipEventCreateWithFlags(&c.h_busy, hipEventDisableTiming) != hipSuccess) c.h_busy = nullptr;
+    if (!c.h_busy || hipEventRecord(c.h_busy, st) != hipSuccess) (void)hipStreamSynchronize(st);
 }
 
 void Ctx::host_free(Cell &c)
@@ -845,14 +846,19 @@ int Ctx::run_entry(const Entry &e)
         }
         if (timing == 2) {
             if (ev_keys_.size() == ev_pool_.size()) {
-                hipEvent_t a, b;
-                hipEventCreate(&a);
-                hipEventCreate(&b);
-                ev_pool_.emplace_back(a, b);
+                hipEvent_t a = nullptr, b = nullptr;
+                if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) {
+                    if (a) hipEventDestroy(a);
+                    timing = 0;                          // this launch goes unsampled
+                } else {
+                    ev_pool_.emplace_back(a, b);
+                }
             }
-            e0 = ev_pool_[ev_keys_.size()].first;
-            e1 = ev_pool_[ev_keys_.size()].second;
-            ev_keys_.push_back(key);
+            if (timing) {
+                e0 = ev_pool_[ev_keys_.size()].first;
+                e1 = ev_pool_[ev_keys_.size()].second;
+                ev_keys_.push_back(key);
+            }
         }
         if (timing) hipEventRecord(e0, stream_);
         rc = sp.run(*this, aty, ap.data(), oty, op.data(), e.acc_mask,
