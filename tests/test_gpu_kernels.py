@@ -391,6 +391,37 @@ def test_gemm_linearity_full_size(ops):
     assert (got.float() - ref).norm() / ref.norm() < 5e-4
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_gemm_random_shapes_through_the_tile_choice(ops, seed):
+    """Seeded random shapes, transpositions and alpha / beta through the automatic choice of kernel and
+    tile (direct-load and register tiles, the two-launch column split, the short-K and few-row kernels,
+    the element-wise fallback for unaligned operands) against fp32 torch: rel-L2 <= 6e-4 and largest
+    error <= 4e-3 of the largest value (f16 rounding of the result is 4.9e-4 relative)."""
+    import random
+    rnd = random.Random(seed)
+    torch.manual_seed(seed)
+    for it in range(24):
+        ta, tb = rnd.random() < 0.5, rnd.random() < 0.5
+        step = rnd.choice([8, 8, 8, 4, 1])                     # alignment class of the leading dimensions
+        M = rnd.randrange(1024, 4300, step)
+        N = rnd.randrange(1024, 9000, step)
+        K = rnd.choice([rnd.randrange(64, 1100, 64), rnd.randrange(8, 600, step), 100])
+        if rnd.random() < 0.2:
+            N = rnd.choice([3200, 8640, 8192 + 8, 8448])
+        if rnd.random() < 0.2:
+            M = rnd.choice([2048, 3200, 2056, 1, 3, 4])
+        alpha, beta = rnd.choice([1.0, 0.5]), rnd.choice([0.0, 1.0])
+        say("gemm random", seed, it, ta, tb, M, N, K, alpha, beta)
+        A = torch.randn((K, M) if ta else (M, K), device="cuda").half()
+        B = (torch.randn((N, K) if tb else (K, N), device="cuda") * 0.1).half()
+        C0 = torch.randn(M, N, device="cuda").half()
+        got = ops.gemm(A, B, ta, tb, alpha, beta, C0.clone()).float()
+        ref = alpha * ((A.float().T if ta else A.float()) @ (B.float().T if tb else B.float())) + beta * C0.float()
+        err = ((got - ref).norm() / ref.norm()).item()
+        mx = ((got - ref).abs().max() / ref.abs().max()).item()
+        assert err < 6e-4 and mx < 4e-3, (ta, tb, M, N, K, alpha, beta, err, mx)
+
+
 def test_gemm_colmajor_entry(ops, oracle):
     """The cuBLAS-shaped entry: row-major callers pass operands swapped (thunk/op.rs:4469-4491)."""
     import ctypes as C
