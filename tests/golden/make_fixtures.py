@@ -1,12 +1,15 @@
 """Writes tests/golden/*.npz: small seeded inputs and the CPU oracle's outputs for every unit of
-the path (fused adjoint kernels, the four GEMM layouts, the attention block, one tiny model step).
+the path (fused adjoint kernels, the four GEMM layouts, the attention block, one tiny model step)
+and of the rows around it (digests, optimiser thunks and one AdamW32 step, the bf16 raw casts, the
+key / value-cached forward pass).
 
 The reference holds no golden vectors for this path and cannot be run here, so these vectors
 are the oracle's own output, frozen: what pins the oracle is the mathematics in
 tests/test_oracle_thunks.py and tests/test_oracle_model.py.  The fixtures guard against the
 oracle drifting (tests/test_golden.py, CPU) and give the HIP path fixed vectors to hit (GPU).
 
-f16 tensors are stored as their uint16 bit patterns.  Run from the repository root:
+f16 tensors are stored as their uint16 bit patterns (bf16 patterns and token ids are genuine uint16:
+tests/test_golden.py lists those names).  Run from the repository root:
     python tests/golden/make_fixtures.py
 """
 import os
@@ -102,6 +105,56 @@ def units():
     out["llama_tiny"] = dict(in_param=flat, in_tok=tok, in_lm_tok=lm_tok, in_scale=scale,
                              out_loss=ref["loss"], out_logit=ref["logit"], out_amax=ref["amax"],
                              out_grad=ref["grad"])
+    out.update(next_rows(r, cfg, flat, tok))
+    return out
+
+
+def next_rows(r, cfg, flat, tok):
+    """digests, optimiser thunks, raw casts, cached forward pass"""
+    out = {}
+    # every exponent class, both signs, zeros, denormals, infinities, quiet and signalling NaNs
+    pat = np.concatenate([r.integers(0, 65536, 3000), np.arange(0, 65536, 1024), [0, 0x8000, 1, 0x8001, 0x03ff, 0x0400,
+                          0x7c00, 0xfc00, 0x7c01, 0x7e00, 0xfe00, 0x7fff, 0xffff, 0x7bff]]).astype(np.uint16)
+    x = pat.view(np.float16)
+    out["digests"] = dict(in_x=x, out_nan=np.int64(oracle.nan_count(x)), out_hist=oracle.abs_log2_hist8(x))
+
+    n = 777
+    grad = randn16(r, (n,), 300.0)
+    grad[:3] = [0.0, 65504.0, -65504.0]
+    avg, avg2 = (r.standard_normal(n) * 0.1).astype(np.float32), (r.random(n) * 0.1).astype(np.float32)
+    avg2[3:6] = [0.0, 1e-30, 4.0]
+    master = (r.standard_normal(n) * 0.02).astype(np.float32)
+    hyper = dict(iter_nr=3, grad_scale=1024.0, lr=2e-5, wd=0.1, a1=0.1, a2=0.05, eps=1e-5)
+    sc = oracle.adamw32_scalars(**hyper)
+    navg, navg2, nmaster, nparam = oracle.adamw32_step(grad, avg, avg2, master, sc)
+    out["optimizer"] = dict(
+        in_grad=grad, in_avg=avg, in_avg2=avg2, in_master=master,
+        in_hyper=np.array([hyper[k] for k in ("iter_nr", "grad_scale", "lr", "wd", "a1", "a2", "eps")], np.float64),
+        out_scalars=sc, out_avg=navg, out_avg2=navg2, out_master=nmaster, out_param=nparam,
+        out_thunk_avg=oracle.online_average_scale(grad, avg, sc[0], sc[1]),
+        out_thunk_avg2=oracle.online_average_square_scale(grad, avg2, sc[0], sc[2]),
+        out_thunk_update=oracle.online_adamw_update(avg, avg2, master, sc[3], sc[4], sc[5], sc[6]),
+        out_thunk_cast=oracle.cast_f32_f16(master * 3000.0))
+
+    bf = np.concatenate([r.integers(0, 65536, 2000), np.arange(0, 65536, 512)]).astype(np.uint16)
+    f32 = np.concatenate([r.standard_normal(1000) * 10.0 ** r.integers(-42, 39, 1000),
+                          [0.0, -0.0, np.inf, -np.inf, np.nan, 65504.0, 1e-45, 3.4e38]]).astype(np.float32)
+    h16 = np.concatenate([r.integers(0, 65536, 2000), np.arange(0, 65536, 512)]).astype(np.uint16).view(np.float16)
+    out["raw_casts"] = dict(in_bf16=bf, in_f32=f32, in_f16=h16,
+                            out_bf16_f16=oracle.raw_cast("bf16_f16", bf), out_bf16_f32=oracle.raw_cast("bf16_f32", bf),
+                            out_f32_bf16=oracle.raw_cast("f32_bf16", f32), out_f16_bf16=oracle.raw_cast("f16_bf16", h16))
+
+    # the cached pass on the tiny model's parameters: a prompt of 5, one position, the other 10
+    kc, vc = oracle.llama_cached_state(cfg)
+    logits, toks = [], []
+    cuts = [0, 5, 6, cfg.S]
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        got = oracle.llama_cached_apply(cfg, flat, kc, vc, tok.copy(), a, b)
+        logits.append(got["logit"])
+        toks.append(got["tok"])
+    out["llama_cached_tiny"] = dict(in_param=flat, in_tok=tok, in_cuts=np.array(cuts, np.int64),
+                                    out_logit=np.concatenate(logits), out_tok=np.concatenate(toks),
+                                    out_k_cache=kc, out_v_cache=vc)
     return out
 
 

@@ -13,9 +13,11 @@ import pytest
 from tests.util import assert_parity
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-INTS = {"in_tok", "in_idx", "in_lm_tok", "out_amax"}        # genuine uint16; other uint16 = f16 bits
+# genuine uint16 (token ids, bf16 bit patterns); any other uint16 array holds f16 bits
+INTS = {"in_tok", "in_idx", "in_lm_tok", "out_amax", "out_tok", "in_bf16", "out_f32_bf16", "out_f16_bf16"}
 UNITS = ["rmsnorm", "rope_dh12", "rope_dh100", "silu_gate", "causal_softmax", "softmax_ce", "embed",
-         "matmul", "attention", "llama_tiny"]
+         "matmul", "attention", "llama_tiny", "digests", "optimizer", "raw_casts", "llama_cached_tiny"]
+EXACT = {"digests", "optimizer", "raw_casts"}               # integer, byte and f32 element-wise work: every bit
 
 
 def load(name):
@@ -53,6 +55,9 @@ def test_oracle_reproduces_fixtures(oracle):
         assert sorted(want) == sorted(fresh[u]), u
         for k, w in want.items():
             g = np.asarray(fresh[u][k])
+            if u in EXACT:
+                assert np.ascontiguousarray(g).tobytes() == np.ascontiguousarray(w).tobytes(), (u, k)
+                continue
             close_enough(g, w, u + "." + k)
             if w.dtype == np.float16 and w.size >= 64:
                 same = np.mean(np.ascontiguousarray(g).view(np.uint16) == np.ascontiguousarray(w).view(np.uint16))
@@ -171,6 +176,73 @@ def test_gpu_gemm_and_attention_hit_fixtures(ops):
     close_enough(_host(dv), d["out_dv"], "attn.dv")
     close_enough(_host(dq), d["out_dq"], "attn.dq")
     close_enough(_host(dk), d["out_dk"], "attn.dk")
+
+
+def _same_bits(got, want, name):
+    got = np.ascontiguousarray(got)
+    assert got.dtype.itemsize == want.dtype.itemsize and got.size == want.size, name
+    assert got.tobytes() == np.ascontiguousarray(want).tobytes(), name
+
+
+@pytest.mark.gpu
+def test_gpu_digests_optimizer_and_raw_casts_hit_fixtures_bit_for_bit(ops):
+    import torch
+    d = load("digests")
+    x = _dev(d["in_x"])
+    assert int(ops.nan_count(x)) == int(d["out_nan"].ravel()[0])
+    _same_bits(_host(ops.abs_log2_hist8(x)), d["out_hist"], "hist")
+    hist, nan = ops.digests([x, x[:100]])
+    _same_bits(_host(hist[0]), d["out_hist"], "batched hist")
+    assert int(nan[0]) == int(d["out_nan"].ravel()[0])
+
+    d = load("optimizer")
+    hy = d["in_hyper"]
+    sc = ops.adamw32_scalars(int(hy[0]), *[float(v) for v in hy[1:]])
+    _same_bits(np.array(sc, np.float32), d["out_scalars"], "scalars")
+    grad = _dev(d["in_grad"])
+    f = lambda k: torch.from_numpy(d[k].copy()).cuda()
+    _same_bits(_host(ops.online_average_scale_(grad, f("in_avg"), sc[0], sc[1])), d["out_thunk_avg"], "avg thunk")
+    _same_bits(_host(ops.online_average_square_scale_(grad, f("in_avg2"), sc[0], sc[2])), d["out_thunk_avg2"], "avg2 thunk")
+    _same_bits(_host(ops.online_adamw_update_(f("in_avg"), f("in_avg2"), f("in_master"), sc[3], sc[4], sc[5], sc[6])),
+               d["out_thunk_update"], "update thunk")
+    _same_bits(_host(ops.cast_f32_f16(f("in_master") * 3000.0)), d["out_thunk_cast"], "cast thunk")
+    avg, avg2, master = f("in_avg"), f("in_avg2"), f("in_master")
+    param = torch.empty_like(grad)
+    ops.adamw32_step_([grad], [avg], [avg2], [master], [param], sc)
+    for got, key in ((avg, "out_avg"), (avg2, "out_avg2"), (master, "out_master"), (param, "out_param")):
+        _same_bits(_host(got), d[key], key)
+
+    d = load("raw_casts")
+    bf = torch.from_numpy(d["in_bf16"].view(np.int16).copy()).cuda()
+    _same_bits(_host(ops.raw_cast_bf16_f16(bf)), d["out_bf16_f16"], "bf16_f16")
+    _same_bits(_host(ops.raw_cast_bf16_f32(bf)), d["out_bf16_f32"], "bf16_f32")
+    _same_bits(_host(ops.raw_cast_f32_bf16(torch.from_numpy(d["in_f32"].copy()).cuda())), d["out_f32_bf16"], "f32_bf16")
+    _same_bits(_host(ops.raw_cast_f16_bf16(_dev(d["in_f16"]))), d["out_f16_bf16"], "f16_bf16")
+
+
+@pytest.mark.gpu
+def test_gpu_cached_pass_hits_fixture():
+    from cacti_amd.runtime import Ctx, Llama, LlamaCached
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(GOLDEN, "make_fixtures.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    c = mod.TINY
+    d = load("llama_cached_tiny")
+    ctx = Ctx(0, 1 << 28, True)
+    m = Llama(ctx, c["S"], c["D"], c["H"], c["Dh"], c["F"], c["V"], c["L"], c["eps"])
+    m.put_params_flat(d["in_param"])
+    k = LlamaCached(m, c["S"])
+    cuts = [int(v) for v in d["in_cuts"]]
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        k.set_tokens(d["in_tok"])
+        k.apply(a, b)
+        got = k.outputs()
+        assert_parity(got["logit"], d["out_logit"][a:b], "cached logit %d:%d" % (a, b))
+        want = d["out_logit"][a:b].astype(np.float32)
+        top2 = np.sort(want, axis=1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 0.02
+        assert np.array_equal(got["tok"][clear], d["out_tok"][a:b][clear])
+    k.close(); m.close(); ctx.close()
 
 
 @pytest.mark.gpu
