@@ -790,6 +790,8 @@ def main():
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
             "has no collective); --gpus %d is not supported" % args.gpus)
         sys.exit(2)
+    from cacti_amd import build
+    build.ensure()                        # loads what is built; compiles only if nothing is
     if args.workload == "step":
         out = run_step(args)
     elif args.workload == "adjoints":

@@ -48,5 +48,11 @@ def build(jobs=4):
     return LIB
 
 
+def ensure():
+    """The library's path, built first if no built library is there (tests, the smoke run and the
+    benchmark call this; the loader itself never builds and never falls back)."""
+    return LIB if os.path.exists(LIB) else build()
+
+
 if __name__ == "__main__":
     print(build())

@@ -12,6 +12,12 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    # a fresh checkout holds no built library: compile it once (hipcc cross-compiles without a GPU)
+    from cacti_amd import build
+    build.ensure()
+
+
 @pytest.fixture(scope="session")
 def oracle():
     from oracle import oracle as o
