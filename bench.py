@@ -569,15 +569,26 @@ def run_ingest(args):
             blobs.append(bits.astype(np.uint16))
             hdr[key] = {"dtype": "BF16", "shape": list(shp), "data_offsets": [off, off + 2 * n]}
             off += 2 * n
-        h = json.dumps(hdr).encode()
-        with open(os.path.join(d, "model.safetensors"), "wb") as f:
-            f.write(struct.pack("<Q", len(h)) + h)
-            for b in blobs:
-                f.write(b.tobytes())
+        pickled = args.ckpt_format == "pickle"
+        if pickled:
+            # pytorch_model.bin as torch.save writes it (the file PickleDir::open reads,
+            # src/util/safepickle.rs:52-119); the bytes of each tensor are the same bf16 patterns
+            import collections
+            sd = collections.OrderedDict(
+                (key, torch.from_numpy(b.view(np.int16)).view(torch.bfloat16).reshape(shp))
+                for key, b, (_, shp) in zip(keys, blobs, model.params))
+            torch.save(sd, os.path.join(d, "pytorch_model.bin"))
+            del sd
+        else:
+            h = json.dumps(hdr).encode()
+            with open(os.path.join(d, "model.safetensors"), "wb") as f:
+                f.write(struct.pack("<Q", len(h)) + h)
+                for b in blobs:
+                    f.write(b.tobytes())
         nbytes = off
 
         def load():
-            td = ingest.TensorsDir(d)
+            td = ingest.PickleDir(d) if pickled else ingest.TensorsDir(d)
             n = model.load_tensors_dir(td)
             ctx.sync()
             td.close()
@@ -593,7 +604,8 @@ def run_ingest(args):
         got = model.param(len(keys) - 1)
         nan = np.isnan(want)
         assert np.array_equal(got[~nan].view(np.uint16), want[~nan].view(np.uint16))
-        out = {"metric": "weight ingest: bf16 safetensors checkpoint -> f16 parameter cells on the device",
+        out = {"metric": "weight ingest: bf16 %s checkpoint -> f16 parameter cells on the device"
+                         % ("torch (pickle)" if pickled else "safetensors"),
                "value": nbytes / dt / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": max(args.warmup, 1),
                "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                "dtype": "u16", "data": "synthetic (N(0, 0.02) bf16 weights, file in the page cache)",
@@ -603,7 +615,7 @@ def run_ingest(args):
                             "frac": 3 * nbytes / dt / 1e9 / PEAK_HBM_GBS, "traffic": None,
                             "note": "device bytes per checkpoint byte: staging write + cast read + cast write; the "
                                     "path is bound by the host copy and PCIe, not by HBM"}}
-        if not args.no_cpu_baseline:
+        if not args.no_cpu_baseline and not pickled:
             t0 = time.time()
             hd = o.read_safetensors_header(os.path.join(d, "model.safetensors"))
             mm = np.memmap(os.path.join(d, "model.safetensors"), dtype=np.uint8, mode="r")
@@ -784,6 +796,8 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ckpt-format", choices=["safetensors", "pickle"], default="safetensors",
+                    help="file format of the ingest workload's checkpoint")
     ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest", "decode", "cycle"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
