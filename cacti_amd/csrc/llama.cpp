@@ -24,6 +24,7 @@ struct cacti_llama {
     cacti_ctx *ctx;
     cacti_llama_cfg cfg;
     std::vector<CellPtr> params, grads;
+    bool grads_written = false;                                 // a gradient cycle has been staged
     std::vector<CellPtr> master, grad_avg, grad2_avg;           // f32 optimiser state (adamw_init)
     std::vector<std::string> names;
     CellPtr embed, head_norm, lm_head;
@@ -477,9 +478,14 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
 
     if (want_grad) {
         // sink.add(out_lm_loss, in_lm_loss_scale); grad_map.add(p, g); vadd_vjp(src, sink)
+        // want_grad = 2: g.cache() on every gradient before the cycle, the micro-batch accumulation of
+        // examples/open_llama_3b_train.rs:334-345 -- this cycle's gradients add to the held ones
+        CACTI_REQUIRE(want_grad != 2 || m->grads_written, CACTI_E_STATE,
+                      "llama_stage: gradients cached before any cycle has written them");
         c.adj_seed(m->out_loss, m->in_loss_scale);
-        for (size_t i = 0; i < m->params.size(); i++) c.adj_bind(m->params[i], m->grads[i]);
+        for (size_t i = 0; i < m->params.size(); i++) c.adj_bind(m->params[i], m->grads[i], want_grad == 2);
         TRY(c.vadd_vjp());
+        m->grads_written = true;
     }
     return 0;
 }

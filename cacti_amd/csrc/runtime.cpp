@@ -675,10 +675,12 @@ void Ctx::adj_seed(CellPtr primal, CellPtr adj)
     adj_wr_[adj] = true;
 }
 
-void Ctx::adj_bind(CellPtr primal, CellPtr adj)
+void Ctx::adj_bind(CellPtr primal, CellPtr adj, bool cached)
 {
     adj_[primal] = adj;
-    adj_wr_[adj] = false;
+    // a cached adjoint counts as written: the cycle's first write into it accumulates
+    // (SpineEntry::Cache gives the cell this cycle's init_once clock, src/spine.rs:786-805)
+    adj_wr_[adj] = cached;
 }
 
 CellPtr Ctx::adj_of(CellPtr primal)

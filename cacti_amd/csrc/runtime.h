@@ -169,7 +169,7 @@ class Ctx {
     void keep(CellPtr c) { kept_.push_back(c); }
     // reverse-mode AD: src/spine.rs:447-690 (CellMap::vadd_vjp, src/op.rs:2386-2393)
     void adj_seed(CellPtr primal, CellPtr adj);                  // sink.add(y, dy)
-    void adj_bind(CellPtr primal, CellPtr adj);                  // grad_map.add(p, g)
+    void adj_bind(CellPtr primal, CellPtr adj, bool cached = false);   // grad_map.add(p, g) [+ g.cache()]
     CellPtr adj_of(CellPtr primal);                              // 0 for const cells
     bool adj_written(CellPtr primal);
     // arg_adj[..] += thunk(args): Apply on first write, Accumulate afterwards (src/op.rs:20-188)

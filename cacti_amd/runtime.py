@@ -201,8 +201,10 @@ class Llama:
     def stage(self, want_prob=False, want_grad=True):
         ffi.call("cacti_llama_stage", self._m, int(want_prob), int(want_grad))
 
-    def step(self, tok, lm_tok, loss_scale, want_prob=False, want_grad=True, want_loss=True):
-        """One fwd + loss + bwd cycle; returns the per-position loss (f32 [S]) or None."""
+    def step(self, tok, lm_tok, loss_scale, want_prob=False, want_grad=True, want_loss=True, accumulate=False):
+        """One fwd + loss + bwd cycle; returns the per-position loss (f32 [S]) or None.  accumulate:
+        the gradients are cached first (g.cache(), examples/open_llama_3b_train.rs:334-345), so this
+        cycle's gradients add to the ones held."""
         tok = np.ascontiguousarray(tok, dtype=np.uint16)
         lm_tok = np.ascontiguousarray(lm_tok, dtype=np.uint16)
         loss_scale = np.ascontiguousarray(loss_scale, dtype=np.float32)
@@ -210,7 +212,7 @@ class Llama:
         assert tok.size == S and lm_tok.size == S and loss_scale.size == S
         loss = np.empty(S, np.float32) if want_loss else None
         ffi.call("cacti_llama_step", self._m, tok.ctypes.data, lm_tok.ctypes.data,
-                 loss_scale.ctypes.data, int(want_prob), int(want_grad),
+                 loss_scale.ctypes.data, int(want_prob), 2 if (want_grad and accumulate) else int(want_grad),
                  loss.ctypes.data if want_loss else None)
         return loss
 

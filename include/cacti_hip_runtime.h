@@ -191,7 +191,10 @@ int cacti_llama_io_cells(cacti_llama *model, int *tok, int *lm_tok, int *loss_sc
                          int *loss, int *amax, int *prob);
 /* Stages one cycle on a freshly reset spine: mem_set_yield_ of the three inputs,
  * Llama::apply, and (want_grad) sink.add(loss, loss_scale) + vadd_vjp over all parameters
- * (examples/open_llama_3b_train.rs:350-389). */
+ * (examples/open_llama_3b_train.rs:350-389).  want_grad = 1 overwrites the gradients; want_grad = 2
+ * is g.cache() on every gradient first (the micro-batch accumulation of :334-345; SpineEntry::Cache,
+ * src/spine.rs:786-805): this cycle's gradients are added, in f16 as every accumulation of the
+ * path, to the values the cells hold.  CACTI_E_STATE if no cycle has written them yet. */
 int cacti_llama_stage(cacti_llama *model, int want_prob, int want_grad);
 /* reset + stage + compile + resume/resume_put.  With loss_out [S] f32 the call syncs, checks
  * the token-range status and copies the loss back; with loss_out = NULL it returns while the

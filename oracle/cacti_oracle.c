@@ -839,14 +839,18 @@ static h16 *halloc(i64 n) { return (h16 *)xmalloc((size_t)n * 2); }
 static float *falloc(i64 n) { return (float *)xmalloc((size_t)n * 4); }
 
 /* Returns 0 on success, 1+row when a token id is out of range.
- * loss [S] f32; logit16 [S,V] (may be NULL); grad has the layout of param. */
+ * loss [S] f32; logit16 [S,V] (may be NULL); grad has the layout of param and, with grad_cached,
+ * holds the gradients this cycle adds to. */
 ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const uint16_t *tok,
                                  const uint16_t *lm_tok, const float *loss_scale, float *loss,
-                                 h16 *logit_out, uint16_t *amax_out, h16 *grad, int n_layers_bwd)
+                                 h16 *logit_out, uint16_t *amax_out, h16 *grad, int grad_cached)
 {
     const i64 S = c->S, D = c->D, H = c->H, Dh = c->Dh, F = c->F, V = c->V, L = c->L;
     const float alpha = 1.0f / sqrtf((float)Dh);
-    (void)n_layers_bwd;
+    /* grad_cached: the gradients were cached before the cycle (g.cache(),
+     * examples/open_llama_3b_train.rs:334-345; SpineEntry::Cache, src/spine.rs:786-805), so every
+     * first write into one accumulates: beta = 1 for the products, y = oy + y for the others */
+    const float gb = grad_cached ? 1.0f : 0.0f;
     if (H * Dh != D) return -1;
     const h16 *embed = param;
     const h16 *layers = param + V * D;
@@ -911,11 +915,11 @@ ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const ui
         h16 *dlogit = halloc(S * V);
         oracle_softmax_ce_bwd(S, V, logit, lm_tok, loss_scale, dlogit);
         /* lm_head matmul (ft): dW += dY^T x A ; dA += dY x W */
-        th_matmul_f16(1, 0, V, D, S, 1.0f, dlogit, V, hn, D, 0.0f, g_lm_head, D);
+        th_matmul_f16(1, 0, V, D, S, 1.0f, dlogit, V, hn, D, gb, g_lm_head, D);
         h16 *dhn = halloc(S * D);
         th_matmul_f16(0, 0, S, D, V, 1.0f, dlogit, V, lm_head, D, 0.0f, dhn, D);
         h16 *dstream = halloc(S * D);
-        oracle_rmsnorm_bwd(S, D, stream, head_norm, t3, s3, dhn, dstream, 0, g_head_norm, 0);
+        oracle_rmsnorm_bwd(S, D, stream, head_norm, t3, s3, dhn, dstream, 0, g_head_norm, grad_cached);
         free(dlogit); free(dhn);
 
         for (i64 l = L - 1; l >= 0; l--) {
@@ -932,25 +936,25 @@ ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const ui
             memcpy(dx1, dstream, (size_t)(S * D) * 2);
             h16 *ddown = dstream;
             /* down matmul */
-            th_matmul_f16(1, 0, D, F, S, 1.0f, ddown, D, s->h, F, 0.0f, gd, F);
+            th_matmul_f16(1, 0, D, F, S, 1.0f, ddown, D, s->h, F, gb, gd, F);
             h16 *dh = halloc(S * F);
             th_matmul_f16(0, 0, S, F, D, 1.0f, ddown, D, wd, F, 0.0f, dh, F);
             h16 *dgate = halloc(S * F), *dup = halloc(S * F);
             oracle_silu_gate_bwd(S * F, s->gate, s->up, s->y, dh, dgate, 0, dup, 0);
             /* gate matmul was staged after up: its adjoint comes first */
             h16 *dpost = halloc(S * D);
-            th_matmul_f16(1, 0, F, D, S, 1.0f, dgate, F, s->post, D, 0.0f, gg, D);
+            th_matmul_f16(1, 0, F, D, S, 1.0f, dgate, F, s->post, D, gb, gg, D);
             th_matmul_f16(0, 0, S, D, F, 1.0f, dgate, F, wg, D, 0.0f, dpost, D);
-            th_matmul_f16(1, 0, F, D, S, 1.0f, dup, F, s->post, D, 0.0f, gu, D);
+            th_matmul_f16(1, 0, F, D, S, 1.0f, dup, F, s->post, D, gb, gu, D);
             th_matmul_f16(0, 0, S, D, F, 1.0f, dup, F, wu, D, 1.0f, dpost, D);
-            oracle_rmsnorm_bwd(S, D, s->x1, w_post, s->t2, s->s2, dpost, dx1, 1, g_post, 0);
+            oracle_rmsnorm_bwd(S, D, s->x1, w_post, s->t2, s->s2, dpost, dx1, 1, g_post, grad_cached);
             free(dh); free(dgate); free(dup); free(dpost); free(ddown);
 
             /* x1 = x0 + o */
             h16 *dx0 = halloc(S * D);
             memcpy(dx0, dx1, (size_t)(S * D) * 2);
             h16 *d_o = dx1;
-            th_matmul_f16(1, 0, D, D, S, 1.0f, d_o, D, s->attn, D, 0.0f, go, D);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, d_o, D, s->attn, D, gb, go, D);
             h16 *dattn = halloc(S * D);
             th_matmul_f16(0, 0, S, D, D, 1.0f, d_o, D, wo, D, 0.0f, dattn, D);
             h16 *dqr = halloc(S * D), *dkr = halloc(S * D), *dv = halloc(S * D);
@@ -958,20 +962,27 @@ ORACLE_API i64 oracle_llama_step(const oracle_cfg *c, const h16 *param, const ui
                                  dkr, dv);
             /* reverse log order of the q, k, v branches: v, k, q */
             h16 *dpre = halloc(S * D);
-            th_matmul_f16(1, 0, D, D, S, 1.0f, dv, D, s->pre, D, 0.0f, gv, D);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, dv, D, s->pre, D, gb, gv, D);
             th_matmul_f16(0, 0, S, D, D, 1.0f, dv, D, wv, D, 0.0f, dpre, D);
             h16 *dk = halloc(S * D), *dq = halloc(S * D);
             oracle_rope_bwd(S, H, Dh, dkr, cos16, sin16, dk, 0);
-            th_matmul_f16(1, 0, D, D, S, 1.0f, dk, D, s->pre, D, 0.0f, gk, D);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, dk, D, s->pre, D, gb, gk, D);
             th_matmul_f16(0, 0, S, D, D, 1.0f, dk, D, wk, D, 1.0f, dpre, D);
             oracle_rope_bwd(S, H, Dh, dqr, cos16, sin16, dq, 0);
-            th_matmul_f16(1, 0, D, D, S, 1.0f, dq, D, s->pre, D, 0.0f, gq, D);
+            th_matmul_f16(1, 0, D, D, S, 1.0f, dq, D, s->pre, D, gb, gq, D);
             th_matmul_f16(0, 0, S, D, D, 1.0f, dq, D, wq, D, 1.0f, dpre, D);
-            oracle_rmsnorm_bwd(S, D, s->x0, w_pre, s->t1, s->s1, dpre, dx0, 1, g_pre, 0);
+            oracle_rmsnorm_bwd(S, D, s->x0, w_pre, s->t1, s->s1, dpre, dx0, 1, g_pre, grad_cached);
             free(d_o); free(dattn); free(dqr); free(dkr); free(dv); free(dpre); free(dk); free(dq);
             dstream = dx0;
         }
-        vjp_outer_select_f16(V, D, S, tok, dstream, g_embed);
+        if (grad_cached) {
+            h16 *ge = halloc(V * D);
+            vjp_outer_select_f16(V, D, S, tok, dstream, ge);
+            th_add_f16(V * D, g_embed, ge, g_embed);
+            free(ge);
+        } else {
+            vjp_outer_select_f16(V, D, S, tok, dstream, g_embed);
+        }
         free(dstream);
     }
 

@@ -275,16 +275,21 @@ def split_params(cfg, flat):
     return out
 
 
-def llama_step(cfg, param, tok, lm_tok, loss_scale, want_grad=True):
-    """Returns dict(loss [S] f32, logit [S,V] f16, amax [S] u16, grad flat f16 or None)."""
+def llama_step(cfg, param, tok, lm_tok, loss_scale, want_grad=True, grad_cached=None):
+    """Returns dict(loss [S] f32, logit [S,V] f16, amax [S] u16, grad flat f16 or None).  grad_cached:
+    the gradients held from earlier micro-batches, cached before this cycle
+    (examples/open_llama_3b_train.rs:334-345): the returned gradients are theirs plus this cycle's."""
     n = lib().oracle_param_elems(C.byref(cfg))
     assert param.size == n and param.dtype == np.float16
     loss = np.empty((cfg.S,), np.float32)
     logit = np.empty((cfg.S, cfg.V), np.float16)
     amax = np.empty((cfg.S,), np.uint16)
     grad = np.zeros((n,), np.float16) if want_grad else None
+    if grad_cached is not None:
+        assert want_grad and grad_cached.dtype == np.float16 and grad_cached.size == n
+        grad = np.array(grad_cached, dtype=np.float16, copy=True, order="C").reshape(n)
     rc = lib().oracle_llama_step(C.byref(cfg), P(param), P(tok), P(lm_tok), P(loss_scale), P(loss),
-                                 P(logit), P(amax), P(grad), C.c_int(0))
+                                 P(logit), P(amax), P(grad), C.c_int(0 if grad_cached is None else 1))
     if rc:
         raise IndexError("oracle_llama_step failed rc=%d" % rc)
     return dict(loss=loss, logit=logit, amax=amax, grad=grad)

@@ -325,3 +325,38 @@ def test_full_size_step_properties():
               flush=True)
         assert err < 5e-3, (n, same, err)
     m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_cached_gradients_accumulate_micro_batches(oracle):
+    """Two micro-batches with the gradients cached in between (g.cache(),
+    examples/open_llama_3b_train.rs:334-345) against the oracle doing the same; caching before any cycle
+    has written the gradients is an error; a plain cycle afterwards overwrites again."""
+    from cacti_amd.ffi import CactiError
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=0, norm_mean=1.0, grad_scale=1024.0)
+    _, _, tok2, lm_tok2, _ = make_inputs(TINY, seed=17, norm_mean=1.0, grad_scale=1024.0)
+    ctx, m = _model(cfg)
+    m.put_params_flat(flat)
+    with pytest.raises(CactiError) as e:
+        m.step(tok, lm_tok, scale, accumulate=True)
+    assert e.value.code == -5
+    m.step(tok, lm_tok, scale)
+    first = m.grads()
+    loss2 = m.step(tok2, lm_tok2, scale, accumulate=True)
+    a = oracle.llama_step(cfg, flat, tok, lm_tok, scale)
+    ab = oracle.llama_step(cfg, flat, tok2, lm_tok2, scale, grad_cached=a["grad"])
+    assert_parity(loss2, ab["loss"], "loss", l2=1e-4, mx=1e-3)
+    want = oracle.split_params(cfg, ab["grad"])
+    got = m.grads()
+    for name, g in got.items():
+        assert_parity(g, want[name], "accumulated grad " + name, l2=2e-3, mx=4e-2)
+        assert not np.array_equal(g, first[name]), name
+    # from the device's own first gradients the accumulation adds exactly one micro-batch: got - first ~ b
+    b = oracle.split_params(cfg, oracle.llama_step(cfg, flat, tok2, lm_tok2, scale)["grad"])
+    for name, g in got.items():
+        d = g.astype(np.float32) - first[name].astype(np.float32)
+        assert rel_l2(d, b[name]) < 5e-3, name
+    m.step(tok2, lm_tok2, scale)
+    for name, g in m.grads().items():
+        assert_parity(g, b[name], "overwritten grad " + name, l2=2e-3, mx=4e-2)
+    m.close(); ctx.close()

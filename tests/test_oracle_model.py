@@ -55,3 +55,29 @@ def test_summation_order_floor_of_the_f16_chain(oracle):
     print("order floor: min %.2e max %.2e" % (min(floors), max(floors)))
     assert 2e-4 < min(floors) and max(floors) < 3e-3
     assert rel_l2(b["loss"], a["loss"]) < 1e-4
+
+
+def test_cached_gradients_accumulate_micro_batches(oracle):
+    """g.cache() before a cycle (examples/open_llama_3b_train.rs:334-345) makes the cycle's first write into
+    every gradient an accumulation.  Pins: cached zeros change nothing, bit for bit (f16(x + 0) = x for the
+    beta = 1 products and for the y = oy + y thunks alike); two micro-batches give, within f16 rounding of
+    the sum, the fp64 autograd gradient of the two-batch loss."""
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=0, norm_mean=1.0, grad_scale=1024.0)
+    _, _, tok2, lm_tok2, _ = make_inputs(TINY, seed=17, norm_mean=1.0, grad_scale=1024.0)
+    a = oracle.llama_step(cfg, flat, tok, lm_tok, scale)
+    z = oracle.llama_step(cfg, flat, tok, lm_tok, scale, grad_cached=np.zeros_like(a["grad"]))
+    assert np.array_equal(z["grad"].view(np.uint16), a["grad"].view(np.uint16))
+    assert np.array_equal(z["loss"], a["loss"])
+    ab = oracle.llama_step(cfg, flat, tok2, lm_tok2, scale, grad_cached=a["grad"])
+    b = oracle.llama_step(cfg, flat, tok2, lm_tok2, scale)
+    assert np.array_equal(ab["loss"], b["loss"])                       # the forward pass does not see the cache
+    params = oracle.split_params(cfg, flat)
+    _, ga64, _ = torch_step(cfg, params, tok, lm_tok, scale)
+    _, gb64, _ = torch_step(cfg, params, tok2, lm_tok2, scale)
+    got = oracle.split_params(cfg, ab["grad"])
+    ga, gb = oracle.split_params(cfg, a["grad"]), oracle.split_params(cfg, b["grad"])
+    for name, g in got.items():
+        assert rel_l2(g, ga64[name] + gb64[name]) < 3e-3, name
+        # against the sum of the two separately rounded gradients: one more f16 rounding at most
+        want = ga[name].astype(np.float32) + gb[name].astype(np.float32)
+        assert rel_l2(g, want) < 6e-4 and max_rel(g, want) < 2e-3, name
