@@ -341,8 +341,11 @@ def run_adjoints(args):
     R = 8
     xs, dys, dxs = [rn(N, D) for _ in range(R)], [rn(N, D) for _ in range(R)], [rn(N, D) for _ in range(R)]
     w = rn(D)
-    add("rms_norm_bwd", time_launches(lambda i: ops.rms_norm_bwd(xs[i % R], w, 1e-6, dys[i % R], dxs[i % R], None), None),
+    add("rms_norm_bwd", time_launches(lambda i: ops.rms_norm_bwd(xs[i % R], w, 1e-6, dys[i % R]), None),
         3 * 2 * N * D + 2 * 2 * D)
+    # the form every layer norm of the step runs: dx accumulates (one more read of [N, D])
+    add("rms_norm_bwd(dx+=)", time_launches(lambda i: ops.rms_norm_bwd(xs[i % R], w, 1e-6, dys[i % R], dxs[i % R], None), None),
+        4 * 2 * N * D + 2 * 2 * D)
     add("rms_norm_fwd", time_launches(lambda i: ops.rms_norm_fwd(xs[i % R], w, 1e-6), None), 2 * 2 * N * D + 2 * D)
     cos, sin = ops.rope_tables(N, Dh)
     q = [rn(N, H, Dh) for _ in range(12)]
@@ -358,7 +361,17 @@ def run_adjoints(args):
     tok = torch.randint(0, V, (N,), device="cuda").to(torch.int16)
     sc = torch.full((N,), 1.0 / N, device="cuda")
     add("softmax_ce_bwd", time_launches(lambda i: ops.softmax_ce_bwd(lg[i % 3], tok, sc), None), 2 * 2 * N * V)
-    add("softmax_ce_fwd(loss)", time_launches(lambda i: ops.softmax_ce_fwd(lg[i % 3], tok, want_prob=False), None), 2 * N * V)
+    # through the C entry point with outputs allocated once: the Python wrapper reads the token-range
+    # status back after every call, which would time a host synchronisation instead of the kernel
+    from cacti_amd import ffi
+    ce_loss = torch.empty(N, device="cuda")
+    ce_amax = torch.empty(N, dtype=torch.int16, device="cuda")
+    ce_stat = torch.zeros(1, dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    add("softmax_ce_fwd(loss)",
+        time_launches(lambda i: ffi.call("cacti_hip_softmax_ce_fwd", N, V, lg[i % 3].data_ptr(), tok.data_ptr(), None,
+                                         ce_loss.data_ptr(), ce_amax.data_ptr(), ce_stat.data_ptr(), st), None), 2 * N * V)
+    assert int(ce_stat.item()) == 0
     del lg
     s16 = [rn(N, H, N) for _ in range(2)]
     dp = rn(N, H, N)

@@ -96,6 +96,8 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         const half_t *xr = x + n * D, *gr = dy + n * D;
         // every load of the row up front and unconditional (see the forward kernel)
         half_t *or_ = dx + n * D;
+        // without accumulation the fourth stream re-reads dy (a cache hit) instead of dx
+        const half_t *oldr = dx_acc ? or_ : gr;
         h8 xv[CH], gv[CH], wv[CH], old[CH];
         float ss = 0.f;
 #pragma unroll
@@ -104,7 +106,7 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
             xv[c] = ld8(xr + ch * 8);
             gv[c] = ld8(gr + ch * 8);
             wv[c] = ld8(w + ch * 8);
-            old[c] = ld8(or_ + ch * 8);                       // used only when dx accumulates
+            old[c] = ld8(oldr + ch * 8);                      // used only when dx accumulates
         }
 #pragma unroll
         for (int c = 0; c < CH; c++) {

@@ -145,6 +145,48 @@ causal_softmax_kernel(int64_t S, int H, const half_t *__restrict__ s16,
 // LM-head softmax / cross-entropy on [N,V], one block of 1024 lanes per row.
 constexpr int kCeThreads = 1024;
 
+// The row lives in registers as fp32 (CH x 8 values per lane); chunks past the row hold -inf, and
+// differences from the maximum below -100 contribute nothing to an fp32 sum that is at least 1.
+// The kernels are bound by their arithmetic as much as by HBM (per element: convert, maximum,
+// exponential, sum, quotient, one-hot, scale, round), hence exp_nonpos and RowDivide.
+template <int CH>
+struct CeRow {
+    float e[CH][8];
+    __device__ float load_max(const half_t *row, int nchunk)
+    {
+        // every load first and unconditional (a chunk past the row re-reads the last one): a load
+        // inside `if (ch < nchunk)` is waited for at the end of that branch, one round trip per chunk
+        h8 raw[CH];
+#pragma unroll
+        for (int c = 0; c < CH; c++) raw[c] = ld8(row + min(c * kCeThreads + (int)threadIdx.x, nchunk - 1) * 8);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < CH; c++) {
+            const bool valid = c * kCeThreads + (int)threadIdx.x < nchunk;
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                e[c][k] = valid ? h2f(raw[c].v[k]) : -INFINITY;
+                mx = fmaxf(mx, e[c][k]);
+            }
+        }
+        return mx;
+    }
+    // e := exp(e - mx); returns the lane's partial sum
+    __device__ float exp_sum(float mx)
+    {
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < CH; c++)
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float x = e[c][k] - mx;
+                e[c][k] = x >= -100.f ? exp_nonpos(x) : 0.f;
+                s += e[c][k];
+            }
+        return s;
+    }
+};
+
 template <int CH>
 __global__ void __launch_bounds__(kCeThreads)
 softmax_ce_fwd_kernel(int64_t N, int V, const half_t *__restrict__ logit,
@@ -155,30 +197,13 @@ softmax_ce_fwd_kernel(int64_t N, int V, const half_t *__restrict__ logit,
     __shared__ float xt_s;
     const int64_t n = blockIdx.x;
     const int nchunk = V / 8;
-    const half_t *lr = logit + n * V;
     const int t = tok ? (int)tok[n] : 0;
     if (tok && t >= V) {
         if (threadIdx.x == 0 && status) atomicMax(status, (int)n + 1);
         return;                                    // uniform for the block
     }
-    float e[CH][8];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int c = 0; c < CH; c++) {
-        const int ch = c * kCeThreads + threadIdx.x;
-        if (ch < nchunk) {
-            h8 v = ld8(lr + ch * 8);
-#pragma unroll
-            for (int k = 0; k < 8; k++) {
-                e[c][k] = h2f(v.v[k]);
-                mx = fmaxf(mx, e[c][k]);
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < 8; k++) e[c][k] = -INFINITY;
-        }
-    }
-    mx = block_reduce(mx, OpMax(), -INFINITY, red);
+    CeRow<CH> row;
+    const float mx = block_reduce(row.load_max(logit + n * V, nchunk), OpMax(), -INFINITY, red);
     if (amax) {
         // first index holding the maximum
         float best = 3.0e38f;
@@ -187,32 +212,36 @@ softmax_ce_fwd_kernel(int64_t N, int V, const half_t *__restrict__ logit,
             const int ch = c * kCeThreads + threadIdx.x;
 #pragma unroll
             for (int k = 0; k < 8; k++)
-                if (e[c][k] == mx) best = fminf(best, (float)(ch * 8 + k));
+                if (row.e[c][k] == mx) best = fminf(best, (float)(ch * 8 + k));
         }
         best = -block_reduce(-best, OpMax(), -3.0e38f, red);
         if (threadIdx.x == 0) amax[n] = (uint16_t)best;
     }
-    float sum = 0.f;
+    if (loss) {
+        // the label's logit: selected in a register, stored by the one lane that holds it
+        float xt = 0.f;
+        bool mine = false;
 #pragma unroll
-    for (int c = 0; c < CH; c++) {
-        const int ch = c * kCeThreads + threadIdx.x;
+        for (int c = 0; c < CH; c++) {
+            const int ch = c * kCeThreads + threadIdx.x;
+            mine = mine || ch == (t >> 3);
 #pragma unroll
-        for (int k = 0; k < 8; k++) {
-            if (loss && ch * 8 + k == t) xt_s = e[c][k];
-            e[c][k] = expf(e[c][k] - mx);
-            sum += e[c][k];
+            for (int k = 0; k < 8; k++) xt = (ch * 8 + k == t) ? row.e[c][k] : xt;
         }
+        if (mine) xt_s = xt;
     }
-    sum = block_reduce(sum, OpSum(), 0.f, red);     // barriers inside publish xt_s
+    const float sum = block_reduce(row.exp_sum(mx), OpSum(), 0.f, red);     // barriers inside publish xt_s
     if (loss && threadIdx.x == 0) loss[n] = -logf(expf(xt_s - mx) / sum);
     if (prob) {
         float *pr = prob + n * V;
+        const RowDivide div(sum);
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int ch = c * kCeThreads + threadIdx.x;
             if (ch < nchunk) {
-                float4 a = make_float4(e[c][0] / sum, e[c][1] / sum, e[c][2] / sum, e[c][3] / sum);
-                float4 b = make_float4(e[c][4] / sum, e[c][5] / sum, e[c][6] / sum, e[c][7] / sum);
+                const float *e = row.e[c];
+                float4 a = make_float4(div(e[0]), div(e[1]), div(e[2]), div(e[3]));
+                float4 b = make_float4(div(e[4]), div(e[5]), div(e[6]), div(e[7]));
                 *reinterpret_cast<float4 *>(pr + ch * 8) = a;
                 *reinterpret_cast<float4 *>(pr + ch * 8 + 4) = b;
             }
@@ -230,46 +259,24 @@ softmax_ce_bwd_kernel(int64_t N, int V, const half_t *__restrict__ logit,
     __shared__ float red[16];
     const int64_t n = blockIdx.x;
     const int nchunk = V / 8;
-    const half_t *lr = logit + n * V;
     const int t = (int)tok[n];
     const float sc = scale[n];
-    float e[CH][8];
-    float mx = -INFINITY;
-#pragma unroll
-    for (int c = 0; c < CH; c++) {
-        const int ch = c * kCeThreads + threadIdx.x;
-        if (ch < nchunk) {
-            h8 v = ld8(lr + ch * 8);
-#pragma unroll
-            for (int k = 0; k < 8; k++) {
-                e[c][k] = h2f(v.v[k]);
-                mx = fmaxf(mx, e[c][k]);
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < 8; k++) e[c][k] = -INFINITY;
-        }
-    }
-    mx = block_reduce(mx, OpMax(), -INFINITY, red);
-    float sum = 0.f;
-#pragma unroll
-    for (int c = 0; c < CH; c++)
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            e[c][k] = expf(e[c][k] - mx);
-            sum += e[c][k];
-        }
-    sum = block_reduce(sum, OpSum(), 0.f, red);
     half_t *dr = dlogit + n * V;
+    CeRow<CH> row;
+    const float mx = block_reduce(row.load_max(logit + n * V, nchunk), OpMax(), -INFINITY, red);
+    const float sum = block_reduce(row.exp_sum(mx), OpSum(), 0.f, red);
+    const RowDivide div(sum);
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int ch = c * kCeThreads + threadIdx.x;
         if (ch < nchunk) {
             h8 o, old;
+            // loaded here, not with the row: the accumulating form runs once per cycle at most (the
+            // first write of dlogit overwrites)
             if (acc) old = ld8(dr + ch * 8);
 #pragma unroll
             for (int k = 0; k < 8; k++) {
-                float p = e[c][k] / sum;
+                float p = div(row.e[c][k]);
                 float z = p - ((ch * 8 + k == t) ? 1.0f : 0.0f);
                 float d = sc * z;
                 o.v[k] = acc ? f2h(h2f(old.v[k]) + rnd16(d)) : f2h(d);
