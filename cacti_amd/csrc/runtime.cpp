@@ -749,6 +749,38 @@ int Ctx::vadd_vjp()
 // there (Spine::_compile splices Live/Unlive, src/spine.rs:1435-1478).
 int Ctx::compile()
 {
+    // Copy forwarding.  y := copy(x) (the adjoint of an add hands the same gradient to both operands)
+    // where x is still read later: if nothing writes x any more and nothing writes y before the last
+    // of those reads, the readers may as well read y, which holds the same bytes until then.  x then
+    // dies at the copy, and the copy becomes the storage move below instead of a launch.
+    static const bool no_forward = getenv("CACTI_NO_COPY_FORWARD") != nullptr;
+    for (size_t i = 0; i < log_.size() && !no_forward; i++) {
+        const Entry &e = log_[i];
+        if (!(e.kind == E_APPLY && thunks_[e.thunk]->is_copy() && e.acc_mask == 0)) continue;
+        const CellPtr x = e.args[0], y = e.outs[0];
+        if (x == y || cells_[x].stable || cells_[y].stable || cells_[x].ty.bytes() != cells_[y].ty.bytes() ||
+            std::find(kept_.begin(), kept_.end(), x) != kept_.end())
+            continue;
+        size_t last_read = i, first_write_y = log_.size();
+        bool ok = true;
+        for (size_t j = i + 1; j < log_.size() && ok; j++) {
+            const Entry &f = log_[j];
+            if (f.kind == E_APPLY) {
+                if (std::find(f.outs.begin(), f.outs.end(), x) != f.outs.end()) ok = false;
+                if (std::find(f.args.begin(), f.args.end(), x) != f.args.end()) last_read = j;
+                if (first_write_y == log_.size() && std::find(f.outs.begin(), f.outs.end(), y) != f.outs.end())
+                    first_write_y = j;
+            } else if (f.kind == E_YIELD_SET) {
+                if (f.cell == x) ok = false;
+                if (f.cell == y && first_write_y == log_.size()) first_write_y = j;
+            }
+        }
+        if (!ok || last_read == i || last_read >= first_write_y) continue;
+        for (size_t j = i + 1; j <= last_read; j++)
+            if (log_[j].kind == E_APPLY)
+                for (CellPtr &a : log_[j].args)
+                    if (a == x) a = y;
+    }
     std::unordered_map<CellPtr, size_t> last;
     for (size_t i = 0; i < log_.size(); i++) {
         const Entry &e = log_[i];
