@@ -360,3 +360,37 @@ def test_cached_gradients_accumulate_micro_batches(oracle):
     for name, g in m.grads().items():
         assert_parity(g, b[name], "overwritten grad " + name, l2=2e-3, mx=4e-2)
     m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_copy_forwarding_changes_no_bit(tmp_path):
+    """The compile pass that turns the adjoint copies of a residual add into storage moves must not change
+    any result: one cycle in a child process with the pass, one with CACTI_NO_COPY_FORWARD=1 (the switch is
+    read once per process), gradients and loss compared byte for byte."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, numpy as np\n"
+        "sys.path.insert(0, %r)\n"
+        "from tests.llama_ref import make_inputs\n"
+        "from tests.test_gpu_llama import TINY, _model\n"
+        "cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=4, norm_mean=1.0, grad_scale=1024.0)\n"
+        "ctx, m = _model(cfg)\n"
+        "m.put_params_flat(flat)\n"
+        "loss = m.step(tok, lm_tok, scale)\n"
+        "g = m.grads()\n"
+        "np.savez(sys.argv[1], loss=loss, **{k: v.view(np.uint16) for k, v in g.items()})\n"
+        "print(ctx.stats())\n" % root)
+    outs = []
+    for tag, extra in (("fwd", {}), ("plain", {"CACTI_NO_COPY_FORWARD": "1"})):
+        path = str(tmp_path / (tag + ".npz"))
+        env = dict(os.environ, **extra)
+        r = subprocess.run([sys.executable, "-c", code, path], env=env, capture_output=True, text=True, timeout=110)
+        assert r.returncode == 0, r.stderr[-2000:]
+        outs.append(np.load(path))
+    a, b = outs
+    assert sorted(a.files) == sorted(b.files) and len(a.files) == 3 + 9 * TINY["L"] + 1
+    for k in a.files:
+        assert a[k].tobytes() == b[k].tobytes(), k
