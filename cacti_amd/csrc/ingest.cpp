@@ -333,8 +333,12 @@ CACTI_API int cacti_tensors_dir_entry(cacti_tensors_dir *dir, int i, char *name,
     const std::string &key = *dir->sorted[(size_t)i];
     const TensorEntry &e = dir->tensors.at(key);
     CACTI_REQUIRE(e.shape.size() <= 8, CACTI_E_NOTIMPL, "tensors_dir_entry: %s has more than 8 dimensions", key.c_str());
-    if (name && name_cap) snprintf(name, name_cap, "%s", key.c_str());
-    if (dtype && dtype_cap) snprintf(dtype, dtype_cap, "%s", e.dtype.c_str());
+    // a name or dtype that does not fit is an error, not a silently shortened string
+    CACTI_REQUIRE(!name || name_cap > key.size(), CACTI_E_INVALID, "tensors_dir_entry: name of %zu bytes needs a larger buffer",
+                  key.size());
+    CACTI_REQUIRE(!dtype || dtype_cap > e.dtype.size(), CACTI_E_INVALID, "tensors_dir_entry: dtype buffer too small");
+    if (name) snprintf(name, name_cap, "%s", key.c_str());
+    if (dtype) snprintf(dtype, dtype_cap, "%s", e.dtype.c_str());
     if (ndim) *ndim = (int)e.shape.size();
     if (shape8)
         for (size_t k = 0; k < e.shape.size(); k++) shape8[k] = e.shape[k];

@@ -22,10 +22,10 @@ class TensorsDir:
 
     def _read_entries(self):
         self.entries = {}             # name -> (dtype string, shape, address, bytes)
-        name, dt = C.create_string_buffer(512), C.create_string_buffer(16)
+        name, dt = C.create_string_buffer(4096), C.create_string_buffer(16)
         for i in range(ffi.lib().cacti_tensors_dir_count(self._d)):
             nd, shp, ptr, nb = C.c_int(), (C.c_int64 * 8)(), C.c_void_p(), C.c_uint64()
-            ffi.call("cacti_tensors_dir_entry", self._d, i, name, 512, dt, 16, C.byref(nd), shp, C.byref(ptr),
+            ffi.call("cacti_tensors_dir_entry", self._d, i, name, 4096, dt, 16, C.byref(nd), shp, C.byref(ptr),
                      C.byref(nb))
             self.entries[name.value.decode("utf-8", "surrogateescape")] = (dt.value.decode(), tuple(shp[k] for k in range(nd.value)),
                                                  ptr.value, nb.value)

@@ -130,7 +130,8 @@ int cacti_llama_adamw_state_get(cacti_llama *model, int i, int which, void *host
  * tensor's type, or a malformed header is CACTI_E_FORMAT, a missing file CACTI_E_IO.
  * tensors_dir_entry: entry i in byte-wise sorted name order (the order CellMatcher scans): name,
  * dtype as spelled in the file ("F16", "BF16", "F32", ...), shape (at most 8 dims), a pointer into
- * the mapping (valid until close) and its length. */
+ * the mapping (valid until close) and its length; a name or dtype longer than its buffer is
+ * CACTI_E_INVALID. */
 typedef struct cacti_tensors_dir cacti_tensors_dir;
 int cacti_tensors_dir_open(const char *path, cacti_tensors_dir **dir);
 int cacti_tensors_dir_close(cacti_tensors_dir *dir);
