@@ -313,3 +313,20 @@ def test_load_rejects_a_shape_mismatch_and_an_unsupported_dtype(oracle, ingest, 
     td.close()
     assert np.array_equal(m.param(len(m.params) - 2).view(np.uint16), x.view(np.uint16))
     m.close(); ctx.close()
+
+
+def test_tensors_dir_entry_refuses_a_buffer_that_is_too_small(ingest, tmp_path):
+    import ctypes as C
+    from cacti_amd import ffi
+    from cacti_amd.ffi import CactiError
+    _write_raw(str(tmp_path / "one.safetensors"),
+               {"a.rather.long.tensor.name": {"dtype": "F16", "shape": [2], "data_offsets": [0, 4]}}, b"\0" * 4)
+    td = ingest.TensorsDir(tmp_path / "one.safetensors")
+    name, dt = C.create_string_buffer(8), C.create_string_buffer(16)
+    nd, shp, ptr, nb = C.c_int(), (C.c_int64 * 8)(), C.c_void_p(), C.c_uint64()
+    with pytest.raises(CactiError) as e:
+        ffi.call("cacti_tensors_dir_entry", td._d, 0, name, 8, dt, 16, C.byref(nd), shp, C.byref(ptr), C.byref(nb))
+    assert e.value.code == -1
+    ffi.call("cacti_tensors_dir_entry", td._d, 0, None, 0, dt, 16, C.byref(nd), shp, C.byref(ptr), C.byref(nb))
+    assert dt.value == b"F16" and nd.value == 1 and nb.value == 4
+    td.close()
