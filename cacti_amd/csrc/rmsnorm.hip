@@ -334,3 +334,40 @@ CACTI_API int cacti_hip_rms_norm_bwd(int64_t N, int64_t D, const void *x, const 
                        (half_t *)dw, dw_acc);
     return launch_status("rms_norm_dw_finalize");
 }
+
+// ---- the same adjoint for callers that cannot allocate ----------------------------------------
+// The fp32 dw partial rows go to a file-scope device array instead of a caller workspace.  The
+// array's name is only a host-side stand-in: its device address is looked up once per device and
+// that pointer, never the name, is what reaches the kernels.
+namespace {
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];          // per device, nullptr until first use on that device
+}  // namespace
+
+CACTI_API size_t cacti_hip_rms_norm_bwd_static_max_bytes(void) { return kStaticScratchBytes; }
+
+CACTI_API int cacti_hip_rms_norm_bwd_static(int64_t N, int64_t D, const void *x, const void *w, float eps,
+                                            const void *dy, void *dx, int dx_acc, void *dw, int dw_acc,
+                                            void *stream)
+{
+    const size_t need = cacti_hip_rms_norm_bwd_workspace(N, D);
+    CACTI_REQUIRE(N > 0 && D > 0 && need <= kStaticScratchBytes, CACTI_E_INVALID,
+                  "rms_norm_bwd_static: N=%lld, D=%lld needs %zu bytes of scratch, the built-in buffer "
+                  "holds %zu; use cacti_hip_rms_norm_bwd with a workspace",
+                  (long long)N, (long long)D, need, kStaticScratchBytes);
+    int dev = -1;
+    CACTI_HIP(hipGetDevice(&dev));
+    CACTI_REQUIRE(dev >= 0 && dev < kMaxDevices, CACTI_E_NOTIMPL,
+                  "rms_norm_bwd_static: device %d is beyond the %d this entry point keeps a buffer for",
+                  dev, kMaxDevices);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        CACTI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        CACTI_REQUIRE(p != nullptr, CACTI_E_STATE, "rms_norm_bwd_static: no device address for the scratch array");
+        g_scratch_ptr[dev] = p;
+    }
+    return cacti_hip_rms_norm_bwd(N, D, x, w, eps, dy, dx, dx_acc, dw, dw_acc, g_scratch_ptr[dev],
+                                  kStaticScratchBytes, stream);
+}

@@ -55,6 +55,8 @@ SIGNATURES = {
     "cacti_hip_add_rms_norm_fwd": (ci, [i64, i64, vp, vp, vp, f32, vp, vp, vp]),
     "cacti_hip_rms_norm_bwd_workspace": (sz, [i64, i64]),
     "cacti_hip_rms_norm_bwd": (ci, [i64, i64, vp, vp, f32, vp, vp, ci, vp, ci, vp, sz, vp]),
+    "cacti_hip_rms_norm_bwd_static_max_bytes": (sz, []),
+    "cacti_hip_rms_norm_bwd_static": (ci, [i64, i64, vp, vp, f32, vp, vp, ci, vp, ci, vp]),
     "cacti_hip_rope_tables": (ci, [i64, i64, vp, vp, vp]),
     "cacti_hip_rope_fwd": (ci, [i64, i64, i64, vp, vp, vp, vp, vp]),
     "cacti_hip_rope_bwd": (ci, [i64, i64, i64, vp, vp, vp, vp, ci, vp]),

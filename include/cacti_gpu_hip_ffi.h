@@ -177,6 +177,19 @@ int cacti_hip_rms_norm_bwd(int64_t N, int64_t D, const void *x, const void *w, f
                            const void *dy, void *dx, int dx_acc, void *dw, int dw_acc,
                            void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same adjoint for callers that cannot allocate device memory or carry a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  The fp32 partial rows of dw go to a buffer built into the library, of
+ * cacti_hip_rms_norm_bwd_static_max_bytes() = 8 MiB per device, held until the process ends; shapes
+ * with cacti_hip_rms_norm_bwd_workspace(N, D) above that are CACTI_E_INVALID.  The call allocates
+ * nothing and frees nothing.  All calls on one device share the one buffer: calls that overlap on a
+ * device (two streams, two threads) race; calls on one stream are ordered and safe.  Results are
+ * bit-identical to cacti_hip_rms_norm_bwd. */
+size_t cacti_hip_rms_norm_bwd_static_max_bytes(void);
+int cacti_hip_rms_norm_bwd_static(int64_t N, int64_t D, const void *x, const void *w, float eps,
+                                  const void *dy, void *dx, int dx_acc, void *dw, int dw_acc,
+                                  void *stream);
+
 /* RoPE tables, Llama::init_constants src/librarium/llama.rs:389-411.
  * cos16, sin16: [S,Dh] f16 (two identical halves of width Dh/2). */
 int cacti_hip_rope_tables(int64_t S, int64_t Dh, void *cos16, void *sin16, void *stream);
