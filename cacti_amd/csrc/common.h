@@ -92,6 +92,14 @@ __device__ __forceinline__ float wave_reduce(float v, Op op)
 __device__ __forceinline__ float wave_sum(float v) { return wave_reduce(v, OpSum()); }
 __device__ __forceinline__ float wave_max(float v) { return wave_reduce(v, OpMax()); }
 
+// fp64 sum over the 64 lanes (two 32-bit exchanges per step); every lane ends with the result
+__device__ __forceinline__ double wave_sum_f64(double v)
+{
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
 // Block reduction through LDS: `red` holds one float per wave (<= 16 waves).
 template <class Op>
 __device__ __forceinline__ float block_reduce(float v, Op op, float ident, float *red)

@@ -8,6 +8,7 @@
 //   c2 = f16(dsq (x+x)); dx = f16(f16(dx_old + c1) + c2)   (or f16(c1 + c2))
 // (rms_norm closure src/librarium/llama.rs:442-451 and its adjoint chain).
 #include "common.h"
+#include "softmax_math.h"
 
 using namespace cacti;
 
@@ -40,7 +41,9 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         if (x2) bv[c] = ld8(x2 + n * D + ch * 8);         // uniform over the launch
         wv[c] = ld8(w + ch * 8);
     }
-    float ss = 0.f;
+    // the squares of f16 values are exact in fp32; summed in fp64 the row sum is the exactly rounded
+    // one, whatever the order, so r is the reference's r and not one of its neighbours
+    double ss = 0.0;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
         const int ch = c * 64 + lane;
@@ -53,13 +56,15 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
 #pragma unroll
             for (int i = 0; i < 8; i++) {
                 float f = h2f(xv[c].v[i]);
-                ss += f * f;
+                ss += (double)(f * f);
             }
         }
     }
-    ss = wave_sum(ss);
-    // one exact division per row; x * (1/r) differs from x / r by at most one fp32 ulp
-    const float rinv = 1.0f / sqrtf(ss / (float)D + eps);
+    ss = wave_sum_f64(ss);
+    // t = x / r as the reference divides: a reciprocal and one residual correction give the
+    // correctly rounded quotient (x * (1/r) alone is an ulp off for a quarter of the elements, and
+    // in a chain of f16-rounded products that ulp grows like any other change of rounding)
+    const RowDivide div(sqrtf((float)ss / (float)D + eps));
     half_t *yr = y + n * D;
 #pragma unroll
     for (int c = 0; c < CH; c++) {
@@ -67,7 +72,7 @@ rms_norm_fwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         if (ch < nchunk) {
             h8 o;
 #pragma unroll
-            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv[c].v[i]) * (h2f(xv[c].v[i]) * rinv));
+            for (int i = 0; i < 8; i++) o.v[i] = f2h(h2f(wv[c].v[i]) * div(h2f(xv[c].v[i])));
             st8(yr + ch * 8, o);
         }
     }
@@ -99,7 +104,7 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
         // without accumulation the fourth stream re-reads dy (a cache hit) instead of dx
         const half_t *oldr = dx_acc ? or_ : gr;
         h8 xv[CH], gv[CH], wv[CH], old[CH];
-        float ss = 0.f;
+        double ss = 0.0;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int ch = min(c * 64 + lane, nchunk - 1);
@@ -115,14 +120,14 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     float f = h2f(xv[c].v[i]);
-                    ss += f * f;
+                    ss += (double)(f * f);
                 }
             }
         }
-        ss = wave_sum(ss);
-        const float r = sqrtf(ss / (float)D + eps);
-        const float rinv = 1.0f / r;              // x * rinv: within one fp32 ulp of x / r
-        float sdx = 0.f;
+        ss = wave_sum_f64(ss);                    // as in the forward kernel: the same r, bit for bit
+        const float r = sqrtf((float)ss / (float)D + eps);
+        const RowDivide div(r), div2(r * r);      // correctly rounded x / r, dt / r and (dt x) / r^2
+        double sdx = 0.0;
 #pragma unroll
         for (int c = 0; c < CH; c++) {
             const int ch = c * 64 + lane;
@@ -130,17 +135,17 @@ rms_norm_bwd_kernel(int64_t N, int D, const half_t *__restrict__ x, const half_t
 #pragma unroll
                 for (int i = 0; i < 8; i++) {
                     float xf = h2f(xv[c].v[i]), du = h2f(gv[c].v[i]);
-                    float t = xf * rinv;
+                    float t = div(xf);
                     dwp[c][i] = rnd16(du * t);
                     float dt = du * h2f(wv[c].v[i]);
-                    sdx += dt * xf;
-                    gv[c].v[i] = f2h(dt * rinv);        // c1, kept in place of dy
+                    sdx += (double)div2(dt * xf);       // the reference's per-element term of dr
+                    gv[c].v[i] = f2h(div(dt));          // c1, kept in place of dy
                     // dt is needed no further: c2 depends only on the row sum
                 }
             }
         }
-        sdx = wave_sum(sdx);
-        const float dr = -sdx / (r * r);
+        sdx = wave_sum_f64(sdx);
+        const float dr = -(float)sdx;
         const float ds = dr / (r + r);
         const float dsq = ds / (float)D;
 #pragma unroll

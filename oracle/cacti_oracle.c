@@ -113,6 +113,25 @@ ORACLE_API h16 oracle_f2h(float f) { return f2h(f); }
 /* ------------------------------------------------------------------------- */
 /* elementwise thunks                                                         */
 
+/* A switch for the one division the norm performs per element:
+ * 0  t = f32(x) / r (as written in the reference's lambda), 1  t = f32(x) * (1 / r), which differs
+ * by at most one fp32 ulp.  Like the GEMM summation order below it is only used to measure how far such a change moves a composed result. */
+static int g_norm_recip = 0;
+/* Two more of the same kind, for what the reference leaves to Futhark and libm:
+ * g_reduce_f32: row and column reductions accumulate in f32, ascending (the reference's f32 `reduce (+)`
+ *   in one of its possible association orders), instead of f64-then-round;
+ * g_exp_exact: exp and log are the correctly rounded ones ((float)exp((double)x)) instead of libm's
+ *   expf / logf (which may be an ulp away). */
+static int g_reduce_f32 = 0, g_exp_exact = 0;
+ORACLE_API void oracle_set_reduce_f32(int on) { g_reduce_f32 = on ? 1 : 0; }
+ORACLE_API void oracle_set_exp_exact(int on) { g_exp_exact = on ? 1 : 0; }
+typedef struct { double d; float f; } racc;          /* a running sum in either precision */
+static inline void racc_add(racc *a, float v) { if (g_reduce_f32) a->f += v; else a->d += (double)v; }
+static inline float racc_get(const racc *a) { return g_reduce_f32 ? a->f : (float)a->d; }
+static inline float o_expf(float x) { return g_exp_exact ? (float)exp((double)x) : expf(x); }
+static inline float o_logf(float x) { return g_exp_exact ? (float)log((double)x) : logf(x); }
+ORACLE_API void oracle_set_norm_reciprocal(int on) { g_norm_recip = on ? 1 : 0; }
+
 /* CastFutThunkSpec, src/thunk/op.rs:621-663 */
 ORACLE_API void th_cast_f16_f32(i64 n, const h16 *x, float *y)
 {
@@ -137,9 +156,9 @@ ORACLE_API void th_inner_mean_f32(i64 rows, i64 len, const float *x, float *y)
 {
 #pragma omp parallel for schedule(static)
     for (i64 r = 0; r < rows; r++) {
-        double acc = 0.0;
-        for (i64 j = 0; j < len; j++) acc += (double)x[r * len + j];
-        y[r] = (float)acc / (float)len;
+        racc acc = {0.0, 0.0f};
+        for (i64 j = 0; j < len; j++) racc_add(&acc, x[r * len + j]);
+        y[r] = racc_get(&acc) / (float)len;
     }
 }
 
@@ -161,7 +180,14 @@ ORACLE_API void th_bdiv_f16_col(i64 N, i64 D, const h16 *x, const float *r, floa
 {
 #pragma omp parallel for schedule(static)
     for (i64 n = 0; n < N; n++)
-        for (i64 d = 0; d < D; d++) y[n * D + d] = h2f(x[n * D + d]) / r[n];
+    {
+        if (g_norm_recip) {
+            const float ri = 1.0f / r[n];
+            for (i64 d = 0; d < D; d++) y[n * D + d] = h2f(x[n * D + d]) * ri;
+        } else {
+            for (i64 d = 0; d < D; d++) y[n * D + d] = h2f(x[n * D + d]) / r[n];
+        }
+    }
 }
 
 /* BroadcastMulFutThunkSpec, src/thunk/op.rs:2058-2134: (f32.f16 u) * (f32.f32 v),
@@ -249,7 +275,7 @@ ORACLE_API void th_silu_f16(i64 n, const h16 *x, h16 *y)
 #pragma omp parallel for schedule(static)
     for (i64 i = 0; i < n; i++) {
         float u = h2f(x[i]);
-        y[i] = f2h(u / (1.0f + expf(-u)));
+        y[i] = f2h(u / (1.0f + o_expf(-u)));
     }
 }
 
@@ -259,7 +285,7 @@ ORACLE_API void th_logistic_f16(i64 n, const h16 *x, h16 *y)
 #pragma omp parallel for schedule(static)
     for (i64 i = 0; i < n; i++) {
         float u = h2f(x[i]);
-        y[i] = f2h(1.0f / (1.0f + expf(-u)));
+        y[i] = f2h(1.0f / (1.0f + o_expf(-u)));
     }
 }
 
@@ -322,13 +348,13 @@ ORACLE_API void th_softmax_f32(i64 rows, i64 len, const float *x, float *y)
         float *yr = y + r * len;
         float mx = -INFINITY;
         for (i64 j = 0; j < len; j++) mx = fmaxf(mx, xr[j]);
-        double sum = 0.0;
+        racc sum = {0.0, 0.0f};
         for (i64 j = 0; j < len; j++) {
-            float e = expf(xr[j] - mx);
+            float e = o_expf(xr[j] - mx);
             yr[j] = e;
-            sum += (double)e;
+            racc_add(&sum, e);
         }
-        float s = (float)sum;
+        float s = racc_get(&sum);
         for (i64 j = 0; j < len; j++) yr[j] = yr[j] / s;
     }
 }
@@ -343,13 +369,13 @@ ORACLE_API void th_softmax_post_adj_f32(i64 rows, i64 len, const float *y, const
         const float *yr = y + r * len;
         const float *gr = dy + r * len;
         float *o = out + r * len;
-        double sum = 0.0;
+        racc sum = {0.0, 0.0f};
         for (i64 j = 0; j < len; j++) {
             float t = yr[j] * gr[j];
             o[j] = t;
-            sum += (double)t;
+            racc_add(&sum, t);
         }
-        float s = (float)sum;
+        float s = racc_get(&sum);
         for (i64 j = 0; j < len; j++) o[j] = o[j] - s * yr[j];
     }
 }
@@ -367,10 +393,10 @@ ORACLE_API i64 th_softmax_nll_f32(i64 rows, i64 len, const float *x, const uint1
         const float *xr = x + r * len;
         float mx = -INFINITY;
         for (i64 j = 0; j < len; j++) mx = fmaxf(mx, xr[j]);
-        double sum = 0.0;
-        for (i64 j = 0; j < len; j++) sum += (double)expf(xr[j] - mx);
-        float v = expf(xr[key[r]] - mx) / (float)sum;
-        out[r] = -logf(v);
+        racc sum = {0.0, 0.0f};
+        for (i64 j = 0; j < len; j++) racc_add(&sum, o_expf(xr[j] - mx));
+        float v = o_expf(xr[key[r]] - mx) / racc_get(&sum);
+        out[r] = -o_logf(v);
     }
     return 0;
 }
@@ -431,9 +457,9 @@ ORACLE_API void vjp_bmul_row(i64 N, i64 D, const float *dy, const float *t, h16 
 {
 #pragma omp parallel for schedule(static)
     for (i64 d = 0; d < D; d++) {
-        double acc = 0.0;
-        for (i64 n = 0; n < N; n++) acc += (double)h2f(f2h(dy[n * D + d] * t[n * D + d]));
-        dw[d] = f2h((float)acc);
+        racc acc = {0.0, 0.0f};
+        for (i64 n = 0; n < N; n++) racc_add(&acc, h2f(f2h(dy[n * D + d] * t[n * D + d])));
+        dw[d] = f2h(racc_get(&acc));
     }
 }
 
@@ -450,7 +476,14 @@ ORACLE_API void vjp_bdiv_x(i64 N, i64 D, const float *dt, const float *r, h16 *d
 {
 #pragma omp parallel for schedule(static)
     for (i64 n = 0; n < N; n++)
-        for (i64 d = 0; d < D; d++) dx[n * D + d] = f2h(dt[n * D + d] / r[n]);
+    {
+        if (g_norm_recip) {
+            const float ri = 1.0f / r[n];
+            for (i64 d = 0; d < D; d++) dx[n * D + d] = f2h(dt[n * D + d] * ri);
+        } else {
+            for (i64 d = 0; d < D; d++) dx[n * D + d] = f2h(dt[n * D + d] / r[n]);
+        }
+    }
 }
 
 /* vjp of (f32.f16 x) / r wrt r: sum_d (-dt * x / r^2) */
@@ -458,10 +491,10 @@ ORACLE_API void vjp_bdiv_r(i64 N, i64 D, const float *dt, const h16 *x, const fl
 {
 #pragma omp parallel for schedule(static)
     for (i64 n = 0; n < N; n++) {
-        double acc = 0.0;
+        racc acc = {0.0, 0.0f};
         float rr = r[n] * r[n];
-        for (i64 d = 0; d < D; d++) acc += (double)(-(dt[n * D + d] * h2f(x[n * D + d])) / rr);
-        dr[n] = (float)acc;
+        for (i64 d = 0; d < D; d++) racc_add(&acc, -(dt[n * D + d] * h2f(x[n * D + d])) / rr);
+        dr[n] = racc_get(&acc);
     }
 }
 
@@ -487,11 +520,82 @@ ORACLE_API void vjp_inner_mean(i64 N, i64 D, const float *dm, float *dsq)
 
 typedef float v8f __attribute__((vector_size(32)));
 
-/* The fp32 summation order of a GEMM is not fixed by the reference (cuBLAS picks it).
- * 0 = ascending k, 1 = descending k: two equally valid restatements whose difference
- * is the floor below which no parity tolerance on a chain of f16 GEMMs can go. */
-static int g_gemm_reverse_k = 0;
-ORACLE_API void oracle_set_gemm_reverse_k(int on) { g_gemm_reverse_k = on; }
+/* The fp32 summation order of a GEMM is not fixed by the reference (cuBLAS picks it).  Equally valid
+ * restatements of "f16 products, fp32 accumulate" are described by three numbers:
+ *   run      k is cut into runs of `run` consecutive values (0 = one run over all of k), each summed
+ *            on its own from zero;
+ *   rev      inside a run the sum goes in descending instead of ascending k;
+ *   combine  0: the run sums are added in ascending order onto one total (what a k-tiled kernel with
+ *            a per-tile partial does), 1: as a balanced binary tree (pairwise summation).
+ * The named modes of oracle_set_gemm_order: 0 ascending (run 0), 1 descending (run 0, rev),
+ * 2 blocked (run 64), 3 pairwise (run 32, tree).  Their mutual distances on a chain of f16-rounded
+ * GEMMs are the envelope inside which any other correct implementation (cuBLAS, an MFMA kernel) must
+ * be expected to land. */
+static int g_gemm_run = 0, g_gemm_rev = 0, g_gemm_tree = 0;
+ORACLE_API void oracle_set_gemm_order_ex(int run, int rev, int tree)
+{
+    g_gemm_run = run > 0 ? run : 0;
+    g_gemm_rev = rev ? 1 : 0;
+    g_gemm_tree = (tree && run > 0) ? 1 : 0;
+}
+ORACLE_API void oracle_set_gemm_order(int mode)
+{
+    switch (mode) {
+    case 1: oracle_set_gemm_order_ex(0, 1, 0); break;
+    case 2: oracle_set_gemm_order_ex(64, 0, 0); break;
+    case 3: oracle_set_gemm_order_ex(32, 0, 1); break;
+    default: oracle_set_gemm_order_ex(0, 0, 0); break;
+    }
+}
+ORACLE_API void oracle_set_gemm_reverse_k(int on) { oracle_set_gemm_order(on ? 1 : 0); }
+
+typedef struct { v8f v[4][2]; } gemm_acc;
+
+static inline void acc_zero(gemm_acc *a)
+{
+    for (int i = 0; i < 4; i++) {
+        a->v[i][0] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
+        a->v[i][1] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
+    }
+}
+static inline void acc_add(gemm_acc *a, const gemm_acc *b)
+{
+    for (int i = 0; i < 4; i++) {
+        a->v[i][0] += b->v[i][0];
+        a->v[i][1] += b->v[i][1];
+    }
+}
+/* running sum over k0 <= k < k1 (descending when rev) added onto *a */
+static inline void acc_run(gemm_acc *a, const float *ap, const float *bp, i64 k0, i64 k1, int rev)
+{
+    for (i64 kk = k0; kk < k1; kk++) {
+        const i64 k = rev ? k1 - 1 - (kk - k0) : kk;
+        v8f b0, b1;
+        memcpy(&b0, bp + k * 16, 32);
+        memcpy(&b1, bp + k * 16 + 8, 32);
+        for (int i = 0; i < 4; i++) {
+            const float av = ap[k * 4 + i];
+            const v8f avv = {av, av, av, av, av, av, av, av};
+            a->v[i][0] += avv * b0;
+            a->v[i][1] += avv * b1;
+        }
+    }
+}
+/* balanced tree over runs [r0, r1) of `run` k each */
+static void acc_tree(gemm_acc *out, const float *ap, const float *bp, i64 r0, i64 r1, i64 K, i64 run, int rev)
+{
+    if (r1 - r0 == 1) {
+        acc_zero(out);
+        const i64 k0 = r0 * run, k1 = (k0 + run < K) ? k0 + run : K;
+        acc_run(out, ap, bp, k0, k1, rev);
+        return;
+    }
+    const i64 mid = r0 + (r1 - r0) / 2;
+    gemm_acc right;
+    acc_tree(out, ap, bp, r0, mid, K, run, rev);
+    acc_tree(&right, ap, bp, mid, r1, K, run, rev);
+    acc_add(out, &right);
+}
 
 static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h16 *A, i64 lda,
                        const h16 *B, i64 ldb, float beta, h16 *C, i64 ldc)
@@ -516,7 +620,8 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
                 b[(np * K + k) * 16 + j] = (n < N) ? h2f(tb ? B[n * ldb + k] : B[k * ldb + n]) : 0.0f;
             }
 
-    const int rev = g_gemm_reverse_k;
+    const i64 run = g_gemm_run;
+    const int rev = g_gemm_rev, tree = g_gemm_tree;
 #pragma omp parallel for schedule(dynamic, 1)
     for (i64 np = 0; np < Np / 16; np++) {
         const float *bp = b + np * K * 16;
@@ -524,24 +629,22 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
         for (i64 mp = 0; mp < Mp / 4; mp++) {
             const float *ap = a + mp * K * 4;
             const i64 m0 = mp * 4;
-            v8f acc[4][2];
-            for (int i = 0; i < 4; i++) {
-                acc[i][0] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
-                acc[i][1] = (v8f){0, 0, 0, 0, 0, 0, 0, 0};
-            }
-            for (i64 kk = 0; kk < K; kk++) {
-                const i64 k = rev ? K - 1 - kk : kk;
-                v8f b0, b1;
-                memcpy(&b0, bp + k * 16, 32);
-                memcpy(&b1, bp + k * 16 + 8, 32);
-                for (int i = 0; i < 4; i++) {
-                    const float av = ap[k * 4 + i];
-                    const v8f avv = {av, av, av, av, av, av, av, av};
-                    acc[i][0] += avv * b0;
-                    acc[i][1] += avv * b1;
+            gemm_acc A4;
+            acc_zero(&A4);
+            if (run == 0) {
+                acc_run(&A4, ap, bp, 0, K, rev);
+            } else if (tree) {
+                if (K > 0) acc_tree(&A4, ap, bp, 0, (K + run - 1) / run, K, run, rev);
+            } else {
+                for (i64 k0 = 0; k0 < K; k0 += run) {
+                    gemm_acc blk;
+                    acc_zero(&blk);
+                    acc_run(&blk, ap, bp, k0, (k0 + run < K) ? k0 + run : K, rev);
+                    acc_add(&A4, &blk);
                 }
             }
-            for (int i = 0; i < 4; i++) {
+#define acc A4.v
+    for (int i = 0; i < 4; i++) {
                 const i64 m = m0 + i;
                 if (m >= M) break;
                 for (int j = 0; j < 16; j++) {
@@ -552,6 +655,7 @@ static void gemm_block(int ta, int tb, i64 M, i64 N, i64 K, float alpha, const h
                     C[m * ldc + n] = f2h(v);
                 }
             }
+#undef acc
         }
     }
     free(a);

@@ -91,6 +91,59 @@ def set_gemm_reverse_k(on):
     lib().oracle_set_gemm_reverse_k(C.c_int(int(on)))
 
 
+# fp32 summation orders of the oracle's GEMMs as (run, rev, tree): k cut into runs of `run` values
+# (0 = one run), each summed ascending (rev: descending) from zero; run sums added in order or as a tree
+GEMM_ORDERS = {"ascending": (0, 0, 0), "descending": (0, 1, 0), "blocked64": (64, 0, 0), "pairwise": (32, 0, 1),
+               "blocked16": (16, 0, 0), "blocked64rev": (64, 1, 0), "pairwise8": (8, 0, 1), "blocked256": (256, 0, 0)}
+
+
+def set_gemm_order(mode):
+    """fp32 summation order of every oracle GEMM: a key of GEMM_ORDERS or a (run, rev, tree) tuple."""
+    run, rev, tree = GEMM_ORDERS.get(mode, mode)
+    lib().oracle_set_gemm_order_ex(C.c_int(run), C.c_int(rev), C.c_int(tree))
+
+
+def set_norm_reciprocal(on):
+    """RMSNorm divides (0, the reference's lambda) or multiplies by the reciprocal (1, <= 1 fp32 ulp away)."""
+    lib().oracle_set_norm_reciprocal(C.c_int(int(on)))
+
+
+def set_reduce_f32(on):
+    """Row / column reductions accumulate in f32, ascending (1), instead of f64 then one rounding (0)."""
+    lib().oracle_set_reduce_f32(C.c_int(int(on)))
+
+
+def set_exp_exact(on):
+    """exp / log correctly rounded through double (1) instead of libm's expf / logf (0)."""
+    lib().oracle_set_exp_exact(C.c_int(int(on)))
+
+
+# Restatements of the cycle that differ only in what the reference leaves open: the fp32 summation
+# order of its GEMMs (cuBLAS), the association order of its f32 reductions (Futhark) and the last ulp
+# of exp / log (libm).  (gemm order, reduce_f32, exp_exact); the first one is the default oracle.
+RESTATEMENTS = {
+    "ascending": ("ascending", 0, 0),
+    "descending": ("descending", 0, 0),
+    "blocked64": ("blocked64", 0, 0),
+    "pairwise": ("pairwise", 0, 0),
+    "ascending+f32sums": ("ascending", 1, 0),
+    "blocked64+f32sums+exp": ("blocked64", 1, 1),
+    "pairwise+exp": ("pairwise", 0, 1),
+    "descending+f32sums+exp": ("descending", 1, 1),
+    "blocked16": ("blocked16", 0, 0),
+    "blocked64rev+f32sums": ("blocked64rev", 1, 0),
+    "pairwise8+exp": ("pairwise8", 0, 1),
+    "blocked256+f32sums+exp": ("blocked256", 1, 1),
+}
+
+
+def set_restatement(name):
+    order, red, ex = RESTATEMENTS[name]
+    set_gemm_order(order)
+    set_reduce_f32(red)
+    set_exp_exact(ex)
+
+
 def set_num_threads(n):
     lib().oracle_set_num_threads(C.c_int(n))
 

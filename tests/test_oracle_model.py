@@ -81,3 +81,47 @@ def test_cached_gradients_accumulate_micro_batches(oracle):
         # against the sum of the two separately rounded gradients: one more f16 rounding at most
         want = ga[name].astype(np.float32) + gb[name].astype(np.float32)
         assert rel_l2(g, want) < 6e-4 and max_rel(g, want) < 2e-3, name
+
+
+def test_python_trace_reproduces_the_c_composition(oracle):
+    """tests/teacher.py composes the cycle from the oracle's per-thunk functions and records every
+    call; its loss and 21 gradients must be those of oracle_llama_step bit for bit, which is what
+    lets a device test replay the recorded calls one thunk at a time."""
+    from tests.teacher import trace_step
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=0, norm_mean=1.0, grad_scale=1024.0)
+    ref = oracle.llama_step(cfg, flat, tok, lm_tok, scale)
+    calls, loss, grads = trace_step(cfg, flat, tok, lm_tok, scale)
+    assert np.array_equal(loss, ref["loss"])
+    want = oracle.split_params(cfg, ref["grad"])
+    assert sorted(grads) == sorted(want)
+    for name, g in grads.items():
+        assert np.array_equal(g.view(np.uint16), want[name].view(np.uint16)), name
+    kinds = {c.kind for c in calls}
+    assert kinds >= {"matmul", "block_matmul", "rms_norm_fwd", "rms_norm_bwd", "rope_fwd", "rope_bwd",
+                     "silu_gate_fwd", "silu_gate_bwd", "causal_softmax_fwd", "causal_softmax_bwd",
+                     "softmax_ce_fwd", "softmax_ce_bwd", "embed_fwd", "embed_bwd", "add"}
+    # 7 forward + 14 backward products per layer, 1 + 2 for the head
+    assert sum(c.kind == "matmul" for c in calls) == 21 * cfg.L + 3
+
+
+def test_summation_order_envelope(oracle):
+    """Twelve restatements of the cycle that differ only in what the reference leaves open (eight fp32
+    summation orders of the GEMMs: ascending, descending, in blocks, pairwise; f32 instead of f64
+    reductions; correctly rounded exp / log): every pair of them lands 0.6-1.3e-3 apart per gradient
+    tensor after two layers, none of them is special.  The largest pairwise distance per tensor is the envelope the device
+    result is held to.  A one-ulp change elsewhere (the norm's x / r as x * (1 / r)) moves the result
+    just as far, which is why the device kernels keep the reference's operations where they can."""
+    from tests.envelope import order_envelope
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=0, norm_mean=1.0, grad_scale=1024.0)
+    runs, env = order_envelope(oracle, cfg, flat, tok, lm_tok, scale)
+    assert len(runs) == 12
+    l2s = [e[0] for e in env.values()]
+    print("envelope rel_l2: min %.2e max %.2e" % (min(l2s), max(l2s)))
+    assert 4e-4 < min(l2s) and max(l2s) < 2e-3
+    oracle.set_norm_reciprocal(1)
+    try:
+        alt = oracle.split_params(cfg, oracle.llama_step(cfg, flat, tok, lm_tok, scale)["grad"])
+    finally:
+        oracle.set_norm_reciprocal(0)
+    moved = max(rel_l2(alt[n], runs["ascending"][n]) for n in alt)
+    assert 5e-4 < moved < 3e-3
