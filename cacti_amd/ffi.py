@@ -64,6 +64,11 @@ SIGNATURES = {
     "cacti_hip_silu_gate_bwd": (ci, [i64, vp, vp, vp, vp, ci, vp, ci, vp]),
     "cacti_hip_causal_softmax_fwd": (ci, [i64, i64, vp, vp, vp]),
     "cacti_hip_causal_softmax_bwd": (ci, [i64, i64, vp, vp, vp, vp]),
+    "cacti_hip_attention_stats_bytes": (sz, [i64, i64]),
+    "cacti_hip_attention_fwd": (ci, [i64, i64, i64, f32, vp, vp, vp, i64, vp, vp, vp]),
+    "cacti_hip_attention_bwd_workspace": (sz, [i64, i64]),
+    "cacti_hip_attention_bwd": (ci, [i64, i64, i64, f32, vp, vp, vp, vp, i64, vp, vp, ci, vp, ci, vp, ci,
+                                     vp, sz, vp]),
     "cacti_hip_softmax_ce_fwd": (ci, [i64, i64, vp, vp, vp, vp, vp, vp, vp]),
     "cacti_hip_softmax_ce_bwd": (ci, [i64, i64, vp, vp, vp, vp, ci, vp]),
     "cacti_hip_embed_fwd": (ci, [i64, i64, vp, i64, vp, vp, vp, vp]),

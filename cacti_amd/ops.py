@@ -91,6 +91,31 @@ def block_matmul_pv(p16, v, causal=False):
                                 H * Dh, Dh, tri=2 if causal else 0)
 
 
+def attention_fwd(q, k, v, alpha):
+    """Fused causal attention on [S,H,Dh] tensors: returns (o, stats); stats feeds attention_bwd."""
+    _chk(q), _chk(k), _chk(v)
+    S, H, Dh = q.shape
+    o = torch.empty_like(q)
+    stats = torch.empty(ffi.lib().cacti_hip_attention_stats_bytes(S, H) // 4, dtype=torch.float32, device=q.device)
+    ffi.call("cacti_hip_attention_fwd", S, H, Dh, alpha, q.data_ptr(), k.data_ptr(), v.data_ptr(), H * Dh,
+             o.data_ptr(), stats.data_ptr(), _stream())
+    return o, stats
+
+
+def attention_bwd(q, k, v, dO, stats, alpha, acc=None):
+    """Adjoint of attention_fwd: returns (dq, dk, dv); acc = (dq, dk, dv) to accumulate into."""
+    _chk(q), _chk(k), _chk(v), _chk(dO)
+    S, H, Dh = q.shape
+    dq, dk, dv = acc if acc is not None else (torch.empty_like(q), torch.empty_like(q), torch.empty_like(q))
+    a = int(acc is not None)
+    nbytes = ffi.lib().cacti_hip_attention_bwd_workspace(S, H)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    ffi.call("cacti_hip_attention_bwd", S, H, Dh, alpha, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+             dO.data_ptr(), H * Dh, stats.data_ptr(), dq.data_ptr(), a, dk.data_ptr(), a, dv.data_ptr(), a,
+             ws.data_ptr(), nbytes, _stream())
+    return dq, dk, dv
+
+
 # ---------------------------------------------------------------- fused thunks
 def rms_norm_fwd(x, w, eps):
     _chk(x), _chk(w)

@@ -223,6 +223,31 @@ int cacti_hip_causal_softmax_fwd(int64_t S, int64_t H, const void *s16, void *p1
 int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const void *dp16,
                                  void *ds16, void *stream);
 
+/* Causal attention of one layer, fused: O = f16(P16 V), P16 = f16(softmax_j(mask(f32(S16)))),
+ * S16 = f16(alpha Q K^T) -- the chain block_matmul_scale -> cast -> BlockTriElemAffine -> InnerSoftmax ->
+ * cast -> block_matmul of src/librarium/llama.rs:501-507 (src/thunk/op.rs:4719-5471, 4189-4278,
+ * 3257-3383) with every rounding point of the chain kept -- and its adjoint
+ * (pop_adj src/thunk/op.rs:4882-4912, InnerSoftmaxPostAdj :3386-3457):
+ *   dV (+)= f16(P16^T dO), dQ (+)= f16(alpha dS16 K), dK (+)= f16(alpha dS16^T Q),
+ *   dS16 = f16(tril(T - (sum_j T) P')), T = P' f32(f16(dO V^T)).
+ * The sequence x sequence tensors S16, P16, dP16, dS16 never reach memory (the reference, and the
+ * separate entry points above, keep them: 4 x H S^2 f16); the adjoint recomputes S16, P' and dP16
+ * tile by tile and forms the row sums sum_j T from the rounded dP16 as the reference does.
+ * q, k, v, o, dO, dq, dk, dv: [S, H, Dh] f16 with row stride ld (elements), 8-byte aligned;
+ * Dh % 4 == 0, Dh <= 128, ld % 4 == 0.  stats: cacti_hip_attention_stats_bytes(S, H) bytes of device
+ * memory, written by the forward call (row maximum and sum per head and row, f32) and read by the
+ * adjoint; workspace: cacti_hip_attention_bwd_workspace(S, H) bytes, contents undefined on return.
+ * *_acc: 0 first write, 1 the product is added to the tensor in fp32 before the one rounding (the
+ * GEMMs' beta = 1). */
+size_t cacti_hip_attention_stats_bytes(int64_t S, int64_t H);
+int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float alpha, const void *q, const void *k,
+                            const void *v, int64_t ld, void *o, void *stats, void *stream);
+size_t cacti_hip_attention_bwd_workspace(int64_t S, int64_t H);
+int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float alpha, const void *q, const void *k,
+                            const void *v, const void *dO, int64_t ld, const void *stats,
+                            void *dq, int dq_acc, void *dk, int dk_acc, void *dv, int dv_acc,
+                            void *workspace, size_t workspace_bytes, void *stream);
+
 /* Row-causal softmax of the cached forward pass, src/librarium/llama.rs:905-907:
  * P16 = f16(softmax_j(mask(f32(S16)))) with mask j > t + initial_row -> -inf
  * (Cast, RowCausalAttentionMaskFutThunkSpec src/librarium/llama.rs:1052-1112, InnerSoftmax, Cast).

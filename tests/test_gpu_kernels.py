@@ -492,3 +492,43 @@ def test_attention_block_via_thunks(ops, oracle, S, H, Dh, tri):
     assert_parity(host(dv), dv_, "dv")
     assert_parity(host(dq), dq_, "dq")
     assert_parity(host(dk), dk_, "dk")
+
+
+@pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100), (200, 2, 100), (72, 2, 128), (1024, 2, 100),
+                                    (384, 6, 100), (8, 1, 4)])
+def test_fused_attention(ops, oracle, S, H, Dh):
+    """The fused forward and adjoint kernels against the oracle's chain of separate thunks: O, the row
+    statistics they keep (maximum and sum of exp of the f16 scores), dQ, dK, dV; ragged sequence lengths
+    (rows and keys beyond S are masked) and head dims 4 .. 128; accumulation into existing gradients."""
+    say("fused attention", S, H, Dh)
+    r = rng(1200 + S + Dh)
+    alpha = float(np.float32(1.0) / np.sqrt(np.float32(Dh)))
+    q, k, v, dO = (randn16(r, (S, H, Dh)) for _ in range(4))
+    ws16, wp16, wo = oracle.attention_fwd(q, k, v, alpha)
+    dq_, dk_, dv_ = oracle.attention_bwd(q, k, v, dO, alpha)
+    Q, K_, V_, DO = dev(q), dev(k), dev(v), dev(dO)
+    o, stats = ops.attention_fwd(Q, K_, V_, alpha)
+    assert_parity(host(o), wo, "o")
+    st = host(stats).reshape(2, H, S)
+    low = np.arange(S)[:, None, None] >= np.arange(S)[None, None, :]
+    sm = np.where(low, ws16.astype(np.float32), -np.inf)                      # [S, H, S]
+    want_m = sm.max(2).T
+    want_l = np.exp(sm.astype(np.float64) - sm.max(2, keepdims=True)).sum(2).T
+    # up to the few scores whose f16 rounding falls the other way with another fp32 summation order
+    assert np.abs(st[0] - want_m).max() <= 2e-3 * max(1.0, np.abs(want_m).max()), "row maxima of the f16 scores"
+    assert np.mean(st[0] == want_m) > 0.95
+    assert np.abs(st[1] / want_l - 1).max() < 2e-3
+    dq, dk, dv = ops.attention_bwd(Q, K_, V_, DO, stats, alpha)
+    for name, got, want in (("dv", dv, dv_), ("dq", dq, dq_), ("dk", dk, dk_)):
+        assert_parity(host(got), want, name)
+    # accumulate mode: the product is added to what the tensors hold, one rounding
+    base = [randn16(r, (S, H, Dh)) for _ in range(3)]
+    acc = tuple(dev(b) for b in base)
+    ops.attention_bwd(Q, K_, V_, DO, stats, alpha, acc=acc)
+    for name, got, b, plain in zip(("dq", "dk", "dv"), acc, base, (dq, dk, dv)):
+        want = b.astype(np.float32) + host(plain).astype(np.float32)
+        assert_parity(host(got), want, name + " accumulated", l2=6e-4, mx=2e-3)
+    # a second call gives the same bits (no atomics, no order dependence)
+    dq2, dk2, dv2 = ops.attention_bwd(Q, K_, V_, DO, stats, alpha)
+    for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert_bits(host(a), host(b), "repeat")
