@@ -25,6 +25,7 @@ struct cacti_llama {
     cacti_llama_cfg cfg;
     std::vector<CellPtr> params, grads;
     bool grads_written = false;                                 // a gradient cycle has been staged
+    int attention_mode = 0;                                     // 0 fused thunk, 1 the chain of separate thunks
     std::vector<CellPtr> master, grad_avg, grad2_avg;           // f32 optimiser state (adamw_init)
     std::vector<std::string> names;
     CellPtr embed, head_norm, lm_head;
@@ -414,6 +415,13 @@ CACTI_API int cacti_llama_io_cells(cacti_llama *m, int *tok, int *lm_tok, int *l
     return 0;
 }
 
+CACTI_API int cacti_llama_set_attention(cacti_llama *m, int mode)
+{
+    CACTI_REQUIRE(m && (mode == 0 || mode == 1), CACTI_E_INVALID, "llama_set_attention: mode must be 0 or 1");
+    m->attention_mode = mode;
+    return 0;
+}
+
 CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
 {
     Ctx &c = m->ctx->c;
@@ -448,9 +456,17 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
         TRY(ap(c, make_rope(g.H), {k, m->cos, m->sin}, &kr));
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.v}, &v));
-        TRY(ap(c, make_causal_scores(alpha, g.H), {qr, kr}, &s16));
-        TRY(ap(c, make_causal_softmax(g.H), {s16}, &p16));
-        TRY(ap(c, make_causal_pv(g.H), {p16, v}, &attn));
+        if (m->attention_mode == 0) {
+            // scores, mask, softmax and the product with v as one thunk: the [S, H, S] cells of
+            // llama.rs:501-505 exist only tile by tile in registers
+            std::vector<CellPtr> ao;
+            TRY(c.stage_apply(c.add_thunk(make_attention(alpha, g.H)), {qr, kr, v}, &ao));
+            attn = ao[0];
+        } else {
+            TRY(ap(c, make_causal_scores(alpha, g.H), {qr, kr}, &s16));
+            TRY(ap(c, make_causal_softmax(g.H), {s16}, &p16));
+            TRY(ap(c, make_causal_pv(g.H), {p16, v}, &attn));
+        }
         TRY(ap(c, make_matmul(false, true, 1.f), {attn, w.o}, &o));
         add_a = stream;                                       // x1 = stream + o
         add_b = o;

@@ -404,6 +404,68 @@ struct CausalSoftmaxSpec : ThunkSpec {
 };
 
 // ---------------------------------------------------------------------------
+// The attention block of a layer as one thunk: scores, cast, mask, softmax, cast and the product with
+// v (src/librarium/llama.rs:501-507) with the rounding points of the separate thunks; the adjoint thunk
+// stands for the adjoints of all of them.  q, k, v, o: [S, H*Dh]; stats: f32 [2*H*S].
+struct AttentionBwdSpec : ThunkSpec {
+    int64_t H;
+    float alpha;
+    AttentionBwdSpec(int64_t h, float a) : H(h), alpha(a) {}
+    const char *name() const override { return "attention_bwd"; }
+    int arity() const override { return 5; }                       // (q, k, v, dO, stats) -> dq, dk, dv
+    int nout() const override { return 3; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0] == a[1] && a[0] == a[2] && a[0] == a[3] && a[0].shape.size() == 2 && a[4].dtype == F32,
+                   "attention_bwd: (q, k, v, dO f16 [S,H*Dh], stats f32) expected");
+        o = {a[0], a[0], a[0]};
+        return 0;
+    }
+    size_t workspace(const std::vector<CellType> &a) const override
+    {
+        return cacti_hip_attention_bwd_workspace(a[0].shape[0], H);
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *ws, size_t wsb) const override
+    {
+        const auto &s = aty[0].shape;
+        return cacti_hip_attention_bwd(s[0], H, s[1] / H, alpha, a[0], a[1], a[2], a[3], s[1], a[4], o[0],
+                                       acc & 1, o[1], (acc >> 1) & 1, o[2], (acc >> 2) & 1, ws, wsb, S(c));
+    }
+};
+
+struct AttentionSpec : ThunkSpec {
+    int64_t H;
+    float alpha;
+    AttentionSpec(int64_t h, float a) : H(h), alpha(a) {}
+    const char *name() const override { return "attention"; }
+    int arity() const override { return 3; }                       // (q, k, v) -> o, stats
+    int nout() const override { return 2; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0] == a[1] && a[0] == a[2] && a[0].shape.size() == 2 &&
+                       a[0].shape[1] % H == 0,
+                   "attention: (q, k, v f16 [S,H*Dh]) expected");
+        o = {a[0], CellType({(int64_t)(cacti_hip_attention_stats_bytes(a[0].shape[0], H) / sizeof(float))}, F32)};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        TY_REQUIRE(acc == 0, "attention: accumulate mode not staged on this path");
+        const auto &s = aty[0].shape;
+        return cacti_hip_attention_fwd(s[0], H, s[1] / H, alpha, a[0], a[1], a[2], s[1], o[0], o[1], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        if (!dy[0]) return 0;
+        return c.adj_add({e.args[0], e.args[1], e.args[2]},
+                         std::unique_ptr<ThunkSpec>(new AttentionBwdSpec(H, alpha)),
+                         {e.args[0], e.args[1], e.args[2], dy[0], e.outs[1]});
+    }
+};
+
+// ---------------------------------------------------------------------------
 // SiLU gate (src/librarium/llama.rs:526-527)
 struct SiluGateBwdSpec : ThunkSpec {
     const char *name() const override { return "silu_gate_bwd"; }
@@ -520,6 +582,10 @@ std::unique_ptr<ThunkSpec> make_rope(int64_t H) { return std::unique_ptr<ThunkSp
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H)
 {
     return std::unique_ptr<ThunkSpec>(new CausalSoftmaxSpec(H));
+}
+std::unique_ptr<ThunkSpec> make_attention(float alpha, int64_t H)
+{
+    return std::unique_ptr<ThunkSpec>(new AttentionSpec(H, alpha));
 }
 std::unique_ptr<ThunkSpec> make_add() { return std::unique_ptr<ThunkSpec>(new AddSpec()); }
 std::unique_ptr<ThunkSpec> make_add_rms_norm(float eps)

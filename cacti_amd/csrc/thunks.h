@@ -14,6 +14,8 @@ std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int6
 // the two block products of causal attention, computed on the lower triangle only
 std::unique_ptr<ThunkSpec> make_causal_scores(float alpha, int64_t H);   // (q, k) -> a q k^T
 std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H);                    // (p16, v) -> p16 v
+// the whole block (scores, mask, softmax, product with v) as one thunk: (q, k, v) -> o, row statistics
+std::unique_ptr<ThunkSpec> make_attention(float alpha, int64_t H);
 std::unique_ptr<ThunkSpec> make_rope(int64_t H);                      // (x [S,H*Dh], cos, sin) -> y
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H);            // (s16 [S,H*S]) -> p16
 std::unique_ptr<ThunkSpec> make_add();                                // (a, b) -> y

@@ -132,6 +132,11 @@ class Llama:
             ffi.lib().cacti_llama_destroy(self._m)
             self._m = None
 
+    def set_attention(self, mode):
+        """"fused" (default): one thunk per layer, nothing of size S x S stored; "thunks": the reference's
+        chain of separate thunks."""
+        ffi.call("cacti_llama_set_attention", self._m, {"fused": 0, "thunks": 1}[mode])
+
     def put_param(self, i, arr):
         arr = np.ascontiguousarray(arr, dtype=np.float16)
         assert arr.shape == self.params[i][1], (arr.shape, self.params[i])

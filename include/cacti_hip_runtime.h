@@ -190,6 +190,11 @@ int cacti_llama_cached_outputs(cacti_llama_cached *cached, void *logit_f16, floa
  * prob f32 [S,V] or 0) */
 int cacti_llama_io_cells(cacti_llama *model, int *tok, int *lm_tok, int *loss_scale, int *logit,
                          int *loss, int *amax, int *prob);
+/* How the attention block of a layer (src/librarium/llama.rs:501-507) is staged from the next cycle on:
+ * 0 (default) one fused thunk, cacti_hip_attention_fwd / _bwd, which keeps the [S, H, S] scores and
+ * probabilities in registers; 1 the reference's chain of separate thunks (block product, causal softmax,
+ * block product and their adjoints), which materialises them.  Same rounding points either way. */
+int cacti_llama_set_attention(cacti_llama *model, int mode);
 /* Stages one cycle on a freshly reset spine: mem_set_yield_ of the three inputs,
  * Llama::apply, and (want_grad) sink.add(loss, loss_scale) + vadd_vjp over all parameters
  * (examples/open_llama_3b_train.rs:350-389).  want_grad = 1 overwrites the gradients; want_grad = 2

@@ -126,28 +126,43 @@ def test_lm_head_and_cross_entropy_full_shape(oracle):
         say("  %s rel_l2 %.2e max_rel %.2e" % (name, e2, em))
 
 
-def test_one_layer_cycle_full_shape(oracle):
-    """One decoder layer + head at the 3B shapes, staged on the spine: loss and all 12 gradient tensors
-    against the oracle, each held to the envelope of the oracle's own fp32 summation orders
-    (tests/envelope.py) and reported against the literal 1e-3 / 2e-2 as well."""
-    from cacti_amd.runtime import Ctx, Llama
-    from tests.envelope import assert_inside_envelope, order_envelope
+@pytest.fixture(scope="module")
+def one_layer_case(oracle):
+    """One decoder layer + head at the 3B shapes: inputs, the oracle's step and the envelope of its
+    restatements (8 of them: each takes about 4 s of host time)."""
+    from tests.envelope import order_envelope
     from tests.llama_ref import make_inputs
-    say("one-layer cycle, full shape")
     cfgd = dict(S=S, D=D, H=H, Dh=DH, F=F, V=V, L=1, eps=1e-6)
     cfg, flat, tok, lm_tok, scale = make_inputs(cfgd, seed=7, norm_mean=1.0, grad_scale=1024.0)
     ref = oracle.llama_step(cfg, flat, tok, lm_tok, scale)
+    _, env = order_envelope(oracle, cfg, flat, tok, lm_tok, scale, count=8)
+    return dict(cfgd=cfgd, cfg=cfg, flat=flat, tok=tok, lm_tok=lm_tok, scale=scale, ref=ref, env=env)
+
+
+@pytest.mark.parametrize("attention", ["fused", "thunks"])
+def test_one_layer_cycle_full_shape(oracle, one_layer_case, attention):
+    """One decoder layer + head at the 3B shapes, staged on the spine: loss and all 12 gradient tensors
+    against the oracle, each held to the envelope of the oracle's own restatements (tests/envelope.py) and
+    reported against the literal 1e-3 / 2e-2 as well; with the attention block as the fused thunk and as
+    the chain of separate thunks."""
+    from cacti_amd.runtime import Ctx, Llama
+    from tests.envelope import assert_inside_envelope
+    say("one-layer cycle, full shape, attention:", attention)
+    k = one_layer_case
+    cfg, ref = k["cfg"], k["ref"]
     ctx = Ctx(0, 8 << 30, True)
-    m = Llama(ctx, **cfgd)
-    m.put_params_flat(flat)
-    loss = m.step(tok, lm_tok, scale)
+    m = Llama(ctx, **k["cfgd"])
+    m.set_attention(attention)
+    m.put_params_flat(k["flat"])
+    loss = m.step(k["tok"], k["lm_tok"], k["scale"])
     assert_parity(loss, ref["loss"], "loss", l2=1e-4, mx=1e-3)
     grads = m.grads()
+    peak = ctx.stats()["pool_peak"]
     m.close(); ctx.close()
     assert len(grads) == 12
     want = oracle.split_params(cfg, ref["grad"])
-    literal = {n: (rel_l2(g, want[n]), max_rel(g, want[n])) for n, g in grads.items()}
-    for n, (e2, em) in literal.items():
+    for n, g in grads.items():
+        e2, em = rel_l2(g, want[n]), max_rel(g, want[n])
         say("  %-12s rel_l2 %.2e max_rel %.2e%s" % (n, e2, em, "" if e2 <= 1e-3 and em <= 2e-2 else "   (outside 1e-3 / 2e-2)"))
-    _, env = order_envelope(oracle, cfg, flat, tok, lm_tok, scale, count=8)      # ~4 s of host time each
-    assert_inside_envelope(grads, want, env, "one layer, full shape")
+    say("  pool peak %.2f GB" % (peak / 1e9))
+    assert_inside_envelope(grads, want, k["env"], "one layer, full shape, " + attention)

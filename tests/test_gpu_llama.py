@@ -28,11 +28,14 @@ def _compare(oracle, cfg, m, ref, env, tag):
     return assert_inside_envelope(grads, oracle.split_params(cfg, ref["grad"]), env, tag)
 
 
-def test_tiny_llama_step_all_gradients(oracle):
-    """Healthy-range variant: norm weights ~N(1, 0.02), grad_scale 1024 (the example's)."""
+@pytest.mark.parametrize("attention", ["fused", "thunks"])
+def test_tiny_llama_step_all_gradients(oracle, attention):
+    """Healthy-range variant: norm weights ~N(1, 0.02), grad_scale 1024 (the example's); the attention
+    block staged as the fused thunk and as the reference's chain of separate thunks."""
     cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=0, norm_mean=1.0, grad_scale=1024.0)
     ref = oracle.llama_step(cfg, flat, tok, lm_tok, scale)
     ctx, m = _model(cfg)
+    m.set_attention(attention)
     m.put_params_flat(flat)
     out = m.step_explicit(tok, lm_tok, scale, want_prob=True)
     assert_parity(out["loss"], ref["loss"], "loss", l2=1e-4, mx=1e-3)
@@ -50,6 +53,8 @@ def test_tiny_llama_step_all_gradients(oracle):
         assert rel_l2(g, g64[name]) <= 1.15 * rel_l2(want[name], g64[name]) + 1e-4, name
     names = ctx.log_names()
     assert names.count("yield_set") == 3 and "unlive" in names and "rms_norm_bwd" in names
+    assert ("attention_bwd" in names) == (attention == "fused")
+    assert ("causal_softmax_bwd" in names) == (attention == "thunks")
     # a second cycle on the same context (reset GCs the first one's cells) gives the same result
     g1 = m.grads()
     loss2 = m.step(tok, lm_tok, scale)
