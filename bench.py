@@ -289,7 +289,8 @@ def run_step(args):
                                "fwd + softmax-CE loss + bwd" % cfg["L"],
                    "pool_cap_bytes": st1["pool_cap"], "pool_peak_bytes": st1["pool_peak"],
                    "spill_evictions_per_step": (st1["n_evict"] - st0["n_evict"]) / args.steps,
-                   "spill_d2h_bytes_per_step": (st1["bytes_d2h"] - st0["bytes_d2h"]) / args.steps},
+                   "spill_d2h_bytes_per_step": (st1["bytes_d2h"] - st0["bytes_d2h"]) / args.steps,
+                   "spill_h2d_bytes_per_step": (st1["bytes_h2d"] - st0["bytes_h2d"]) / args.steps},
         "survey_device_ms_per_step": dev_ms,
         "roofline": roofline,
         "kernels": kernels[:24],

@@ -187,6 +187,11 @@ CACTI_API uint64_t cacti_mempool_alloc(cacti_mempool *pool, uint64_t bytes)
     size_t o = pool->p.alloc((size_t)bytes);
     return o == kNoOffset ? UINT64_MAX : (uint64_t)o;
 }
+CACTI_API uint64_t cacti_mempool_alloc_high(cacti_mempool *pool, uint64_t bytes)
+{
+    size_t o = pool->p.alloc((size_t)bytes, true);
+    return o == kNoOffset ? UINT64_MAX : (uint64_t)o;
+}
 CACTI_API int cacti_mempool_free(cacti_mempool *pool, uint64_t offset)
 {
     CACTI_REQUIRE(pool->p.size_of((size_t)offset) != 0, CACTI_E_INVALID,

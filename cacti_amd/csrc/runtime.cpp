@@ -18,31 +18,55 @@ namespace cacti {
 
 void MemPool::reset(size_t cap)
 {
-    cap_ = cap;
+    cap_ = back_ = cap;
     front_ = used_ = peak_ = 0;
     free_.clear();
+    free_hi_.clear();
     alloc_.clear();
 }
 
-size_t MemPool::alloc(size_t bytes)
+// first fit from the lowest offset, the low end of the hole
+size_t MemPool::take_low(size_t req, std::map<size_t, size_t> &holes)
+{
+    for (auto it = holes.begin(); it != holes.end(); ++it) {
+        if (it->second < req) continue;
+        const size_t off = it->first, rest = it->second - req;
+        holes.erase(it);
+        if (rest) holes[off + req] = rest;
+        return off;
+    }
+    return kNoOffset;
+}
+
+// first fit from the highest offset, the high end of the hole
+size_t MemPool::take_high(size_t req, std::map<size_t, size_t> &holes)
+{
+    for (auto it = holes.rbegin(); it != holes.rend(); ++it) {
+        if (it->second < req) continue;
+        it->second -= req;
+        const size_t off = it->first + it->second;
+        if (it->second == 0) holes.erase(it->first);
+        return off;
+    }
+    return kNoOffset;
+}
+
+size_t MemPool::alloc(size_t bytes, bool high)
 {
     if (bytes == 0) bytes = 1;
     const size_t req = (bytes + kAllocAlign - 1) / kAllocAlign * kAllocAlign;
-    size_t off = kNoOffset;
-    for (auto it = free_.begin(); it != free_.end(); ++it) {      // first fit, lowest offset
-        if (it->second >= req) {
-            off = it->first;
-            const size_t rest = it->second - req;
-            free_.erase(it);
-            if (rest) free_[off + req] = rest;
-            break;
+    size_t off = high ? take_high(req, free_hi_) : take_low(req, free_);
+    if (off == kNoOffset && req <= back_ - front_) {              // move the cursor of that end
+        if (high) {
+            back_ -= req;
+            off = back_;
+        } else {
+            off = front_;
+            front_ += req;
         }
     }
-    if (off == kNoOffset) {
-        if (front_ + req > cap_) return kNoOffset;
-        off = front_;
-        front_ += req;
-    }
+    if (off == kNoOffset) off = high ? take_high(req, free_) : take_low(req, free_hi_);
+    if (off == kNoOffset) return kNoOffset;
     alloc_[off] = req;
     used_ += req;
     if (used_ > peak_) peak_ = used_;
@@ -56,23 +80,27 @@ void MemPool::free(size_t off)
     size_t sz = it->second;
     alloc_.erase(it);
     used_ -= sz;
-    auto next = free_.lower_bound(off);
-    if (next != free_.end() && off + sz == next->first) {         // merge with the next region
+    const bool hi = off >= back_;
+    std::map<size_t, size_t> &holes = hi ? free_hi_ : free_;
+    auto next = holes.lower_bound(off);
+    if (next != holes.end() && off + sz == next->first) {         // merge with the next region
         sz += next->second;
-        next = free_.erase(next);
+        next = holes.erase(next);
     }
-    if (next != free_.begin()) {                                  // merge with the previous one
+    if (next != holes.begin()) {                                  // merge with the previous one
         auto prev = std::prev(next);
         if (prev->first + prev->second == off) {
             off = prev->first;
             sz += prev->second;
-            free_.erase(prev);
+            holes.erase(prev);
         }
     }
-    if (off + sz == front_)
-        front_ = off;                                             // retract the bump cursor
+    if (!hi && off + sz == front_)
+        front_ = off;                                             // retract the cursor of that end
+    else if (hi && off == back_)
+        back_ = off + sz;
     else
-        free_[off] = sz;
+        holes[off] = sz;
 }
 
 size_t MemPool::size_of(size_t off) const
@@ -83,8 +111,9 @@ size_t MemPool::size_of(size_t off) const
 
 size_t MemPool::largest_free() const
 {
-    size_t best = cap_ - front_;
+    size_t best = back_ - front_;
     for (auto &kv : free_) best = std::max(best, kv.second);
+    for (auto &kv : free_hi_) best = std::max(best, kv.second);
     return best;
 }
 
@@ -96,7 +125,20 @@ Ctx::Ctx() { cells_.emplace_back(); cells_[0].alive = false; }   // cell 0 = nil
 Ctx::~Ctx()
 {
     if (stream_) hipStreamSynchronize(stream_);
-    for (auto &c : cells_) host_free(c);
+    if (down_stream_) hipStreamSynchronize(down_stream_);
+    if (up_stream_) hipStreamSynchronize(up_stream_);
+    for (auto &c : cells_) {
+        host_free(c);
+        if (c.v_ready) hipEventDestroy(c.v_ready);
+    }
+    for (auto &kv : host_pool_) {
+        if (kv.second.busy) hipEventDestroy(kv.second.busy);
+        hipHostFree(kv.second.ptr);
+    }
+    for (auto &pf : pending_) hipEventDestroy(pf.done);
+    for (hipEvent_t e : ev_spare_) hipEventDestroy(e);
+    if (down_stream_) hipStreamDestroy(down_stream_);
+    if (up_stream_) hipStreamDestroy(up_stream_);
     for (auto &e : ev_pool_) {
         hipEventDestroy(e.first);
         hipEventDestroy(e.second);
@@ -135,6 +177,13 @@ int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
     CACTI_HIP(hipMemset(base_ + status_off_, 0, kAllocAlign));
     CACTI_HIP(hipStreamCreateWithFlags(&stream_, hipStreamNonBlocking));
     own_stream_ = true;
+    // spill copies overlap compute only from page-locked memory (a copy from pageable memory is staged
+    // synchronously by the runtime); default priority, like the compute stream
+    async_spill_ = host_pagelocked != 0;
+    if (async_spill_) {
+        CACTI_HIP(hipStreamCreateWithFlags(&down_stream_, hipStreamNonBlocking));
+        CACTI_HIP(hipStreamCreateWithFlags(&up_stream_, hipStreamNonBlocking));
+    }
     CACTI_HIP(hipEventCreate(&ev0_));
     CACTI_HIP(hipEventCreate(&ev1_));
     return 0;
@@ -143,6 +192,31 @@ int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
 int Ctx::sync()
 {
     CACTI_HIP(hipStreamSynchronize(stream_));
+    if (down_stream_) CACTI_HIP(hipStreamSynchronize(down_stream_));
+    if (up_stream_) CACTI_HIP(hipStreamSynchronize(up_stream_));
+    return 0;
+}
+
+hipEvent_t Ctx::ev_get()
+{
+    // an event goes back into use long after the waits that name it were queued
+    if (ev_spare_.size() > 256) {
+        hipEvent_t e = ev_spare_.front();
+        ev_spare_.pop_front();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) return nullptr;
+    return e;
+}
+
+int Ctx::order_after_compute(hipStream_t st)
+{
+    hipEvent_t e = ev_get();
+    CACTI_REQUIRE(e, CACTI_E_STATE, "ctx: cannot create an event");
+    CACTI_HIP(hipEventRecord(e, stream_));
+    CACTI_HIP(hipStreamWaitEvent(st, e, 0));
+    ev_put(e);                         // the wait is queued; the event may be recorded again
     return 0;
 }
 
@@ -174,6 +248,15 @@ int Ctx::host_alloc(Cell &c)
     if (c.hptr) return 0;
     const size_t n = std::max<size_t>(c.ty.bytes(), 1);
     if (host_pagelocked_) {
+        // a buffer of a dead cell of the same size, if there is one (page-locking memory costs
+        // milliseconds; the cells of a cycle have the sizes of the cycle before)
+        auto it = host_pool_.find(n);
+        if (it != host_pool_.end()) {
+            c.hptr = it->second.ptr;
+            c.h_busy = it->second.busy;        // copies of the previous owner may still be in flight
+            host_pool_.erase(it);
+            return 0;
+        }
         CACTI_HIP(hipHostMalloc(&c.hptr, n, hipHostMallocDefault));
     } else {
         c.hptr = malloc(n);
@@ -197,13 +280,21 @@ static void host_mark_busy(Cell &c, hipStream_t st)
 
 void Ctx::host_free(Cell &c)
 {
+    if (c.hptr && host_pagelocked_) {
+        // back to the pool together with the event of its last copy
+        host_pool_.emplace(std::max<size_t>(c.ty.bytes(), 1), HostBuf{c.hptr, c.h_busy});
+        c.hptr = nullptr;
+        c.h_busy = nullptr;
+        c.h_valid = false;
+        return;
+    }
     if (c.h_busy) {
         hipEventSynchronize(c.h_busy);
         hipEventDestroy(c.h_busy);
         c.h_busy = nullptr;
     }
     if (!c.hptr) return;
-    if (host_pagelocked_) hipHostFree(c.hptr); else free(c.hptr);
+    free(c.hptr);
     host_bytes_ -= std::max<size_t>(c.ty.bytes(), 1);
     c.hptr = nullptr;
     c.h_valid = false;
@@ -217,6 +308,11 @@ int Ctx::cell_free_all(CellPtr ci)
         c.voff = kNoOffset;
     }
     c.v_valid = false;
+    if (c.v_ready) {                          // a prefetch nobody consumed: the region is free once it has landed
+        hipStreamWaitEvent(stream_, c.v_ready, 0);
+        ev_put(c.v_ready);
+        c.v_ready = nullptr;
+    }
     if (c.hptr || c.h_busy) host_free(c);     // waits for in-flight copies of this cell only
     return 0;
 }
@@ -505,9 +601,35 @@ int Ctx::evict(CellPtr ci)
 {
     Cell &c = cells_[ci];
     if (c.voff == kNoOffset) return 0;
+    if (c.v_ready) {                           // never picked as a victim; a direct call waits for the upload
+        CACTI_HIP(hipStreamWaitEvent(stream_, c.v_ready, 0));
+        ev_put(c.v_ready);
+        c.v_ready = nullptr;
+    }
     if (c.v_valid && !c.h_valid) {
         int rc = host_alloc(c);
         if (rc) return rc;
+        if (async_spill_) {
+            // download on the copy stream, after the compute work queued so far (the cell's producer);
+            // the region goes back to the pool when the download is done (reclaim)
+            if ((rc = order_after_compute(down_stream_))) return rc;
+            if (c.h_busy) CACTI_HIP(hipStreamWaitEvent(down_stream_, c.h_busy, 0));   // earlier users of the buffer
+            CACTI_HIP(hipMemcpyAsync(c.hptr, dev_ptr(c.voff), c.ty.bytes(), hipMemcpyDeviceToHost, down_stream_));
+            host_mark_busy(c, down_stream_);
+            hipEvent_t done = ev_get();
+            CACTI_REQUIRE(done, CACTI_E_STATE, "ctx: cannot create an event");
+            CACTI_HIP(hipEventRecord(done, down_stream_));
+            sum_downloaded_ += c.ty.bytes();
+            (in_eager_ ? cyc_eager_ : cyc_demand_down_) += c.ty.bytes();
+            pending_.push_back(PendingFree{c.voff, pool_.size_of(c.voff), done});
+            pending_bytes_ += pending_.back().bytes;
+            c.h_valid = true;
+            bytes_d2h_ += c.ty.bytes();
+            c.voff = kNoOffset;
+            c.v_valid = false;
+            n_evict_++;
+            return 0;
+        }
         CACTI_HIP(hipMemcpyAsync(c.hptr, dev_ptr(c.voff), c.ty.bytes(), hipMemcpyDeviceToHost,
                                  stream_));
         if (!host_pagelocked_) CACTI_HIP(hipStreamSynchronize(stream_));
@@ -515,11 +637,81 @@ int Ctx::evict(CellPtr ci)
         c.h_valid = true;
         bytes_d2h_ += c.ty.bytes();
     }
+    if (async_spill_) {
+        sum_dropped_ += c.ty.bytes();
+        cyc_dropped_ += c.ty.bytes();
+    }
     pool_.free(c.voff);          // later users of the region are ordered after the copy
     c.voff = kNoOffset;
     c.v_valid = false;
     n_evict_++;
     return 0;
+}
+
+// Regions of evicted cells whose download has finished go back to the pool; with a request that
+// does not fit yet, the streams that may reuse a region are made to wait for the unfinished downloads,
+// oldest first, and those regions go back too until the request fits (no host wait either way).
+void Ctx::reclaim(size_t need)
+{
+    size_t kept = 0;
+    bool busy = false;          // the downloads finish in the order they were queued: one query finds the first unfinished
+    for (size_t i = 0; i < pending_.size(); i++) {
+        PendingFree &pf = pending_[i];
+        bool done = !busy && hipEventQuery(pf.done) == hipSuccess;
+        busy = !done;
+        if (!done && need && pool_.largest_free() < need) {
+            hipStreamWaitEvent(stream_, pf.done, 0);        // whoever gets the region next: a thunk ...
+            hipStreamWaitEvent(up_stream_, pf.done, 0);     // ... or an upload
+            done = true;
+        }
+        if (done) {
+            pool_.free(pf.off);
+            pending_bytes_ -= pf.bytes;
+            ev_put(pf.done);
+        } else {
+            pending_[kept++] = pf;
+        }
+    }
+    pending_.resize(kept);
+}
+
+// Entry index of the next use of a cell in the compiled log, from the entry being run on; a cell that
+// this cycle does not touch again is needed by the next cycle, where its first use says how soon.
+// (uses_ holds 2 * entry + 1 where the entry overwrites the cell without reading it.)
+size_t Ctx::next_use(CellPtr c, bool *overwrite) const
+{
+    if (overwrite) *overwrite = false;
+    auto it = uses_.find(c);
+    if (it == uses_.end() || it->second.empty()) return 2 * log_.size() + (size_t)c;
+    const std::vector<uint32_t> &u = it->second;
+    auto p = std::lower_bound(u.begin(), u.end(), (uint32_t)(2 * pc_));
+    if (p == u.end()) p = u.begin();
+    if (overwrite) *overwrite = (*p & 1) != 0;
+    return (p == u.begin() && (*p >> 1) < pc_ ? log_.size() : 0) + (*p >> 1);
+}
+
+// The resident, unpinned cell whose next use lies farthest ahead (among those of at least min_bytes);
+// without a compiled log, the oldest cell (the reference's creation order, src/pctx/nvgpu.rs:2004-2283).
+int Ctx::pick_victim(size_t min_bytes, bool allow_prefetched, int cls) const
+{
+    int best = 0;
+    size_t best_use = 0;
+    for (size_t i = 1; i < cells_.size(); i++) {
+        const Cell &c = cells_[i];
+        if (!c.alive || c.voff == kNoOffset || c.pin > 0 || (c.v_ready && !allow_prefetched)) continue;
+        if (pool_.size_of(c.voff) < min_bytes) continue;
+        if (!compiled_) return (int)i;
+        bool ow = false;
+        const size_t u = next_use((CellPtr)i, &ow);
+        const bool drop = !c.v_valid || c.h_valid;               // nothing to download
+        if (cls == V_DROP && !drop) continue;
+        if (cls == V_DOWN_ONLY && (drop || !ow)) continue;
+        if (!best || u > best_use) {
+            best = (int)i;
+            best_use = u;
+        }
+    }
+    return best;
 }
 
 // NvGpuMemPool::_try_soft_oom, src/pctx/nvgpu.rs:2004-2283: dead cells are already freed
@@ -529,25 +721,144 @@ int Ctx::try_soft_oom(size_t need)
 {
     n_soft_oom_++;
     const size_t req = (need + kAllocAlign - 1) / kAllocAlign * kAllocAlign;
-    for (int pass = 0; pass < 2; pass++) {
-        for (size_t i = 1; i < cells_.size(); i++) {
-            Cell &c = cells_[i];
-            if (!c.alive || c.voff == kNoOffset || c.pin > 0) continue;
-            if (pass == 0 && pool_.size_of(c.voff) < req) continue;
-            int rc = evict((CellPtr)i);
+    // regions whose download is under way first: finished ones cost nothing, the others a stream wait
+    reclaim(0);
+    if (pool_.largest_free() >= req) return 0;
+    reclaim(req);
+    if (pool_.largest_free() >= req) return 0;
+    // then victims: those that free their memory at once (nothing to download) and are not needed
+    // soon, then by next use alone, first only cells at least as large as the request, then any
+    // (a last pass also takes cells that were uploaded ahead of their use)
+    for (int pass = -1; pass < 3; pass++) {
+        for (;;) {
+            const int v = pick_victim(pass <= 0 ? req : 0, pass == 2, pass < 0 ? V_DROP : V_ANY);
+            if (!v || (pass <= 0 && compiled_ && next_use((CellPtr)v) < pc_ + 48)) break;
+            int rc = evict((CellPtr)v);
             if (rc) return rc;
+            reclaim(req);
             if (pool_.largest_free() >= req) return 0;
         }
     }
     return CACTI_E_OOM;
 }
 
-int Ctx::pool_alloc(size_t bytes, size_t *off)
+// Before a thunk runs on a pool that has already run out once: evict ahead of need, so that the
+// downloads overlap the thunks in between and allocations find free memory instead of waiting.
+int Ctx::keep_reserve()
 {
-    size_t o = pool_.alloc(bytes);
+    if (!async_spill_ || n_soft_oom_ == 0 || !compiled_) return 0;
+    reclaim(0);
+    const size_t reserve = reserve_bytes();
+    while (pool_.cap() - pool_.used() + pending_bytes_ < reserve) {
+        // the class that has carried less so far first, then the other, then any cell
+        const int first = sum_dropped_ <= sum_downloaded_ ? V_DROP : V_DOWN_ONLY;
+        int v = pick_victim(0, false, first);
+        if (!v || next_use((CellPtr)v) < pc_ + 48) v = pick_victim(0, false, first == V_DROP ? V_DOWN_ONLY : V_DROP);
+        if (!v || next_use((CellPtr)v) < pc_ + 48) v = pick_victim(0);
+        if (!v) break;
+        // nothing is gained by evicting what the next thunks use
+        if (next_use((CellPtr)v) < pc_ + 24) break;
+        int rc = evict((CellPtr)v);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+// One spilled cell back into memory that is free now, on the upload stream; 1 when there is no room.
+int Ctx::upload_ahead(Cell &c, bool *ordered)
+{
+    const size_t off = pool_.alloc(c.ty.bytes(), c.stable);
+    if (off == kNoOffset) return 1;
+    n_alloc_++;
+    if (!*ordered) {
+        // the region may have belonged to a cell that queued compute work still reads
+        int rc = order_after_compute(up_stream_);
+        if (rc) {
+            pool_.free(off);
+            return rc;
+        }
+        *ordered = true;
+    }
+    c.voff = off;
+    if (c.h_busy) CACTI_HIP(hipStreamWaitEvent(up_stream_, c.h_busy, 0));
+    CACTI_HIP(hipMemcpyAsync(dev_ptr(off), c.hptr, c.ty.bytes(), hipMemcpyHostToDevice, up_stream_));
+    host_mark_busy(c, up_stream_);
+    c.v_ready = ev_get();
+    CACTI_REQUIRE(c.v_ready, CACTI_E_STATE, "ctx: cannot create an event");
+    CACTI_HIP(hipEventRecord(c.v_ready, up_stream_));
+    c.v_valid = true;
+    n_upload_++;
+    bytes_h2d_ += c.ty.bytes();
+    return 0;
+}
+
+// Upload, on the upload stream, the spilled cells that coming thunks read, into memory that is free
+// now (never by evicting: a prefetch must not push out what is needed sooner).  The next 16 thunks
+// are looked at before every thunk, past the end of the log into the start of the next cycle (which
+// replays this one); entries farther ahead are gone through once, by a cursor that stops where an
+// upload would leave less than the reserve free: the backward pass frees memory as it goes, and an
+// upload takes longer than the thunks that wait for it, so it has to start that early.
+int Ctx::prefetch_ahead()
+{
+    if (!async_spill_ || n_soft_oom_ == 0 || !compiled_) return 0;
+    bool ordered = false;
+    auto reads = [&](const Entry &f, bool far) -> int {
+        for (size_t k = 0; k < f.args.size() + f.outs.size(); k++) {
+            const bool is_out = k >= f.args.size();
+            const CellPtr ci = is_out ? f.outs[k - f.args.size()] : f.args[k];
+            if (is_out && !((f.acc_mask >> (k - f.args.size())) & 1)) continue;      // written, not read
+            Cell &c = cells_[ci];
+            if (!c.alive || c.voff != kNoOffset || !c.h_valid) continue;
+            if (far && pool_.cap() - pool_.used() < c.ty.bytes() + reserve_bytes()) return 1;
+            int rc = upload_ahead(c, &ordered);
+            if (rc) return rc;
+        }
+        return 0;
+    };
+    int thunks = 0;
+    const size_t n = log_.size();
+    for (size_t j = pc_ + 1; j < pc_ + n && thunks < 16; j++) {
+        const Entry &f = log_[j < n ? j : j - n];
+        if (f.kind != E_APPLY) continue;
+        thunks++;
+        int rc = reads(f, false);
+        if (rc) return rc < 0 ? rc : 0;                                              // no room now: later
+    }
+    if (pf_cursor_ < pc_ + 1) pf_cursor_ = pc_ + 1;
+    for (const size_t end = std::min(n, pc_ + 1 + 640); pf_cursor_ < end; pf_cursor_++) {
+        const Entry &f = log_[pf_cursor_];
+        if (f.kind != E_APPLY) continue;
+        int rc = reads(f, true);
+        if (rc) return rc < 0 ? rc : 0;
+    }
+    return 0;
+}
+
+int Ctx::spill_eagerly(const Entry &e)
+{
+    if (!async_spill_ || eager_left_ == 0 || e.kind != E_APPLY) return 0;
+    for (CellPtr o : e.outs) {
+        Cell &c = cells_[o];
+        if (!c.alive || !c.stable || c.voff == kNoOffset || c.pin > 0 || c.v_ready || !c.v_valid || c.h_valid)
+            continue;
+        if (c.ty.bytes() > eager_left_) continue;
+        bool ow = false;
+        if (next_use(o, &ow) < log_.size() || !ow) continue;
+        eager_left_ -= c.ty.bytes();
+        in_eager_ = true;
+        int rc = evict(o);
+        in_eager_ = false;
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+int Ctx::pool_alloc(size_t bytes, size_t *off, bool high)
+{
+    size_t o = pool_.alloc(bytes, high);
     if (o == kNoOffset) {
         int rc = try_soft_oom(bytes);
-        if (rc == 0) o = pool_.alloc(bytes);
+        if (rc == 0) o = pool_.alloc(bytes, high);
         if (o == kNoOffset) {
             set_error("device pool exhausted: request %zu bytes, cap %zu, used %zu, front %zu, "
                       "largest free %zu (every other cell is pinned by the running thunk)",
@@ -566,15 +877,23 @@ int Ctx::ensure_vmem(CellPtr ci, bool need_value)
     CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "use of dead cell %d (%s)", ci, c.name.c_str());
     if (c.voff == kNoOffset) {
         size_t off;
-        int rc = pool_alloc(c.ty.bytes(), &off);
+        int rc = pool_alloc(c.ty.bytes(), &off, c.stable);
         if (rc) return rc;
         cells_[ci].voff = off;
         cells_[ci].v_valid = false;
     }
     Cell &d = cells_[ci];
+    if (d.v_ready) {                           // prefetched: the compute stream waits for the upload here
+        CACTI_HIP(hipStreamWaitEvent(stream_, d.v_ready, 0));
+        ev_put(d.v_ready);
+        d.v_ready = nullptr;
+    }
     if (need_value && !d.v_valid) {
         CACTI_REQUIRE(d.h_valid, CACTI_E_STATE, "cell %d (%s) is read before it holds a value", ci,
                       d.name.c_str());
+        // an upload the prefetch did not get to: on the compute stream, which needs it now (a download
+        // of this cell that is still under way on the copy stream comes first)
+        if (d.h_busy) CACTI_HIP(hipStreamWaitEvent(stream_, d.h_busy, 0));
         CACTI_HIP(hipMemcpyAsync(dev_ptr(d.voff), d.hptr, d.ty.bytes(), hipMemcpyHostToDevice,
                                  stream_));
         host_mark_busy(d, stream_);
@@ -600,6 +919,10 @@ void Ctx::reset()
     // compact trailing dead cells so ids do not grow without bound across cycles
     while (cells_.size() > 1 && !cells_.back().alive) cells_.pop_back();
     log_.clear();
+    uses_.clear();
+    if (pc_ > 0) eager_left_ = (cyc_eager_ + cyc_demand_down_ + cyc_dropped_) / 2;
+    cyc_eager_ = cyc_demand_down_ = cyc_dropped_ = 0;
+    pf_cursor_ = 0;
     thunks_.clear();
     kept_.clear();
     adj_.clear();
@@ -816,6 +1139,18 @@ int Ctx::compile()
         }
     }
     log_.swap(out);
+    uses_.clear();
+    for (size_t i = 0; i < log_.size(); i++) {
+        const Entry &e = log_[i];
+        if (e.kind != E_APPLY) continue;
+        for (CellPtr a : e.args)
+            if (uses_[a].empty() || (uses_[a].back() >> 1) != (uint32_t)i) uses_[a].push_back((uint32_t)(2 * i));
+        for (size_t k = 0; k < e.outs.size(); k++) {
+            const CellPtr o = e.outs[k];
+            if (!uses_[o].empty() && (uses_[o].back() >> 1) == (uint32_t)i) continue;     // also read here
+            uses_[o].push_back((uint32_t)(2 * i + (((e.acc_mask >> k) & 1) || e.move ? 0 : 1)));
+        }
+    }
     compiled_ = true;
     pc_ = 0;
     return 0;
@@ -946,8 +1281,13 @@ int Ctx::resume(CellPtr *yield_cell)
             cell_free_all(e.cell);
             cells_[e.cell].alive = false;
         } else {
-            int rc = run_entry(e);
+            int rc = keep_reserve();
+            if (!rc) rc = prefetch_ahead();
+            if (!rc) rc = run_entry(e);
             if (rc) return rc < 0 ? rc : -1000 - rc;  // keep 0/1 for DONE/YIELD
+            pc_++;
+            if ((rc = spill_eagerly(e))) return rc;
+            continue;
         }
         pc_++;
     }

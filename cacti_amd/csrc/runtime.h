@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <deque>
 #include <map>
 #include <memory>
 #include <string>
@@ -48,7 +49,11 @@ class MemPool {
    public:
     explicit MemPool(size_t cap = 0) : cap_(cap) {}
     void reset(size_t cap);
-    size_t alloc(size_t bytes);          // offset, or kNoOffset when it does not fit
+    // offset, or kNoOffset when it does not fit.  `high` allocations (cells that live across cycles:
+    // parameters, gradients) are packed downwards from the top of the pool, the others upwards from
+    // the bottom, so that the short-lived regions of a cycle do not end up scattered between the
+    // long-lived ones; each kind falls back to the other's holes before it gives up.
+    size_t alloc(size_t bytes, bool high = false);
     void free(size_t off);
     size_t size_of(size_t off) const;
     size_t cap() const { return cap_; }
@@ -59,8 +64,11 @@ class MemPool {
     size_t num_allocs() const { return alloc_.size(); }
 
    private:
-    size_t cap_ = 0, front_ = 0, used_ = 0, peak_ = 0;
-    std::map<size_t, size_t> free_;                  // offset -> size, coalesced
+    size_t cap_ = 0, front_ = 0, back_ = 0, used_ = 0, peak_ = 0;
+    std::map<size_t, size_t> free_;                  // holes below front_: offset -> size, coalesced
+    std::map<size_t, size_t> free_hi_;               // holes from back_ up
+    size_t take_low(size_t req, std::map<size_t, size_t> &holes);
+    size_t take_high(size_t req, std::map<size_t, size_t> &holes);
     std::unordered_map<size_t, size_t> alloc_;       // offset -> size
 };
 
@@ -76,6 +84,7 @@ struct Cell {
     bool v_valid = false, h_valid = false;
     int pin = 0;
     hipEvent_t h_busy = nullptr;   // recorded after the last copy that touches hptr
+    hipEvent_t v_ready = nullptr;  // a prefetching upload into the VMem replica is in flight on the copy stream
 };
 
 struct Stats {
@@ -154,10 +163,26 @@ class Ctx {
     // make the VMem replica exist (evicting others if needed) and, if `need_value`, hold
     // the current version (uploading from the host replica)
     int ensure_vmem(CellPtr c, bool need_value);
-    int pool_alloc(size_t bytes, size_t *off);                   // with soft-OOM eviction
+    int pool_alloc(size_t bytes, size_t *off, bool high = false);                   // with soft-OOM eviction
     void pool_free(size_t off) { pool_.free(off); }              // later reuse is ordered on the stream
     int try_soft_oom(size_t need);
     int evict(CellPtr c);                                        // VMem -> Mem, drop VMem
+    // Overlapped spilling (page-locked host memory only).  Downloads and uploads run on two further
+    // streams of the same priority (PCIe carries both directions at once), ordered with events: an
+    // evicted region returns to the pool when its download is done (or the streams that may reuse it
+    // are made to wait for it).  Victims are resident cells whose next use in the compiled log lies
+    // farthest ahead, taken in turn from those that can be dropped without a copy (a valid host
+    // replica: parameters after their use in the forward pass) and those that need a download but no
+    // later upload (their next use overwrites them: the gradients of the cycle before), so that
+    // both directions carry about the same; then any other cell.  Before every thunk a reserve of
+    // free memory is kept by evicting ahead of need, and cells the next thunks read are uploaded
+    // ahead of them.
+    size_t next_use(CellPtr c, bool *overwrite = nullptr) const;  // entry index, beyond the log = next cycle
+    enum VictimClass : int { V_ANY = 0, V_DROP = 1, V_DOWN_ONLY = 2 };
+    int pick_victim(size_t min_bytes, bool allow_prefetched = false, int cls = V_ANY) const;   // 0: none
+    void reclaim(size_t need);                                   // return finished downloads' regions to the pool (need > 0: wait for more until it fits)
+    int keep_reserve();
+    int prefetch_ahead();
 
     // ---- staging (control thread side of the spine)
     void reset();                                                // src/ctx.rs:150-235
@@ -207,7 +232,33 @@ class Ctx {
     int run_entry(const Entry &e);
     int host_alloc(Cell &c);
     void host_free(Cell &c);
+    hipEvent_t ev_get();
+    void ev_put(hipEvent_t e) { if (e) ev_spare_.push_back(e); }
+    int order_after_compute(hipStream_t st);                     // st waits for the compute work queued so far
 
+    struct PendingFree { size_t off, bytes; hipEvent_t done; };
+    struct HostBuf { void *ptr; hipEvent_t busy; };
+    hipStream_t down_stream_ = nullptr, up_stream_ = nullptr;
+    size_t sum_dropped_ = 0, sum_downloaded_ = 0;               // bytes evicted per class so far
+    // Downloads that a cycle had to wait for are started early in the next one: as soon as a thunk
+    // has written a cell that this cycle does not touch again and the next one overwrites (a
+    // gradient), the cell is evicted, until as many bytes have gone as the cycle before downloaded
+    // in all.  The first such cells are written early in the backward pass, so their downloads
+    // overlap the rest of it instead of the forward pass that needs the memory.  The budget is half
+    // of what the cycle before evicted in any way: the other half is left to cells that are dropped
+    // without a copy and come back on the upload stream, so that both directions of the link work.
+    size_t eager_left_ = 0, cyc_eager_ = 0, cyc_demand_down_ = 0, cyc_dropped_ = 0;
+    bool in_eager_ = false;
+    size_t pf_cursor_ = 0;                                       // entries before it have had their far prefetch
+    int spill_eagerly(const Entry &e);
+    int upload_ahead(Cell &c, bool *ordered);                    // one cell, on the upload stream
+    size_t reserve_bytes() const { return std::min<size_t>(pool_.cap() / 24, (size_t)640 << 20); }
+    bool async_spill_ = false;
+    std::vector<PendingFree> pending_;                           // regions of evicted cells, oldest first
+    size_t pending_bytes_ = 0;
+    std::deque<hipEvent_t> ev_spare_;                            // recycled oldest first, and only when plenty
+    std::unordered_map<CellPtr, std::vector<uint32_t>> uses_;    // compiled log: entries that touch a cell
+    std::multimap<size_t, HostBuf> host_pool_;                   // page-locked buffers of dead cells, by size
     int dev_ = 0;
     hipStream_t stream_ = nullptr;
     bool own_stream_ = false;

@@ -109,6 +109,7 @@ SIGNATURES = {
     "cacti_mempool_create": (ci, [pvp, C.c_uint64]),
     "cacti_mempool_destroy": (ci, [vp]),
     "cacti_mempool_alloc": (C.c_uint64, [vp, C.c_uint64]),
+    "cacti_mempool_alloc_high": (C.c_uint64, [vp, C.c_uint64]),
     "cacti_mempool_free": (ci, [vp, C.c_uint64]),
     "cacti_mempool_stats": (ci, [vp, C.POINTER(C.c_uint64)]),
     "cacti_reset": (ci, [vp]),

@@ -20,8 +20,10 @@ class MemPool:
         self._p = C.c_void_p()
         ffi.call("cacti_mempool_create", C.byref(self._p), cap)
 
-    def alloc(self, nbytes):
-        off = ffi.lib().cacti_mempool_alloc(self._p, nbytes)
+    def alloc(self, nbytes, high=False):
+        """high: packed downwards from the top (cells that live across cycles)."""
+        f = ffi.lib().cacti_mempool_alloc_high if high else ffi.lib().cacti_mempool_alloc
+        off = f(self._p, nbytes)
         return None if off == 2 ** 64 - 1 else off
 
     def free(self, off):

@@ -68,11 +68,17 @@ int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap);
  * touched, so it can be exercised on a host without a GPU): first fit over the coalesced
  * free regions, else bump the front cursor; 256-byte granules; freeing the last region
  * retracts the cursor (src/pctx/nvgpu.rs:30, 1633-1655).  alloc returns the offset, or
- * UINT64_MAX when the request does not fit. */
+ * UINT64_MAX when the request does not fit.  alloc_high is the mirror image from the top of
+ * the range (highest hole first, else a back cursor that moves down): the runtime places
+ * the cells that live across cycles (parameters, gradients) there, so that a cycle's
+ * short-lived regions are not scattered between them; the reference has one front
+ * allocator and no counterpart.  Either kind takes a hole of the other end before it
+ * reports that the request does not fit. */
 typedef struct cacti_mempool cacti_mempool;
 int cacti_mempool_create(cacti_mempool **pool, uint64_t cap);
 int cacti_mempool_destroy(cacti_mempool *pool);
 uint64_t cacti_mempool_alloc(cacti_mempool *pool, uint64_t bytes);
+uint64_t cacti_mempool_alloc_high(cacti_mempool *pool, uint64_t bytes);
 int cacti_mempool_free(cacti_mempool *pool, uint64_t offset);
 /* out[0..4] = cap, used, peak, front cursor, largest request that fits now */
 int cacti_mempool_stats(cacti_mempool *pool, uint64_t out[5]);
