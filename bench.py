@@ -107,6 +107,15 @@ def gemm_flops(label):
 N_CUS = 256
 
 
+def attention_flops(label, cfg):
+    """Algorithmic flops of the fused attention thunks: the causal half of Q K^T and P V in the
+    forward pass (2 products of S^2/2 x Dh per head), of dV, dP, dQ and dK in the adjoint (4); what the
+    kernels recompute (Q K^T again in both passes of the forward kernel and in both adjoint kernels) is
+    not counted."""
+    per = 2.0 * cfg["H"] * (cfg["S"] * (cfg["S"] + 1) // 2) * cfg["Dh"]
+    return {"attention": 2 * per, "attention_bwd": 4 * per}.get(label)
+
+
 def gemm_dims(label):
     m = GEMM_RE.match(label)
     return (m.group(2) == "T", m.group(3) == "T") + tuple(int(m.group(i)) for i in (4, 5, 6, 7))
@@ -194,6 +203,45 @@ def cpu_baseline(cfg):
                       % (CPU_SAMPLE_LAYERS, cfg["L"], layer, times[0], cfg["S"], cfg["L"])}
 
 
+CAPPED_POOL_BYTES = 16 << 30       # the reference's 16 GiB card (examples/open_llama_3b_train.rs runs on one)
+CAPPED_WARMUP = 6                  # the spill plan of a cycle follows the cycles before it: a few to settle
+
+
+def run_capped(cfg, args):
+    """The same step on a device pool capped at 16 GiB, so that it has to spill to page-locked host
+    memory: K timed steps after its own warmup.  Returns the record and the loss, which the caller
+    compares bit for bit with the uncapped run's.  (It runs before the uncapped leg: a 16 GiB pool
+    allocated after the uncapped leg's pool of 90 % of the device has been freed measured 10 % slower.)"""
+    import torch
+    from cacti_amd.runtime import Ctx, Llama
+    ctx = Ctx(0, CAPPED_POOL_BYTES, True)
+    model = Llama(ctx, **cfg)
+    synth_params(model)
+    tok, lm_tok, scale = synth_inputs(cfg)
+    for _ in range(max(args.warmup, CAPPED_WARMUP)):
+        model.step(tok, lm_tok, scale, want_loss=False)
+    ctx.sync()
+    torch.cuda.synchronize()
+    st0 = ctx.stats()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        model.step(tok, lm_tok, scale, want_loss=False)
+    ctx.sync()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st1 = ctx.stats()
+    loss = model.step(tok, lm_tok, scale)
+    model.close()
+    ctx.close()
+    per = lambda k: (st1[k] - st0[k]) / args.steps
+    log("capped at %.0f GiB: %.2f ms/step, %.0f evictions, %.2f GB down, %.2f GB up per step"
+        % (CAPPED_POOL_BYTES / 2 ** 30, dt / args.steps * 1e3, per("n_evict"), per("bytes_d2h") / 1e9, per("bytes_h2d") / 1e9))
+    return {"pool_cap_bytes": CAPPED_POOL_BYTES, "ms_per_step": dt / args.steps * 1e3,
+            "tokens_per_s": cfg["S"] * args.steps / dt, "evictions": per("n_evict"),
+            "d2h_bytes": per("bytes_d2h"), "h2d_bytes": per("bytes_h2d"), "pool_peak_bytes": st1["pool_peak"],
+            "steps": args.steps, "warmup": max(args.warmup, CAPPED_WARMUP)}, loss
+
+
 def run_step(args):
     import torch
     from cacti_amd.runtime import Ctx, Llama
@@ -201,6 +249,8 @@ def run_step(args):
     if args.layers is not None:
         cfg["L"] = args.layers
     pool = int(args.pool_gb * (1 << 30)) if args.pool_gb else 0
+    # the same configuration on the reference's 16 GiB card: a second run, on a capped pool
+    capped, capped_loss = (None, None) if pool or args.no_capped else run_capped(cfg, args)
     ctx = Ctx(0, pool, True)
     model = Llama(ctx, **cfg)
     t0 = time.time()
@@ -227,10 +277,19 @@ def run_step(args):
     kernels = []
     for label, (cnt, tot_ms) in sorted(rep.items(), key=lambda kv: -kv[1][1]):
         fl = gemm_flops(label)
-        ent = {"label": label, "launches_per_step": cnt / n_survey, "avg_us": tot_ms / cnt * 1e3,
+        sec = tot_ms / cnt * 1e-3
+        ent = {"label": label, "launches_per_step": cnt / n_survey, "avg_us": sec * 1e6,
                "total_ms_per_step": tot_ms / n_survey}
+        # every entry against the roof that bounds it: the products (attention included) by
+        # their algorithmic flops against dense fp16 MFMA, everything else by its operand
+        # bytes (each input read once, each output written once) against HBM
+        ent["bytes"] = ctx.operand_bytes.get(label, 0)
+        afl = attention_flops(label, cfg) if fl is None else fl
+        if afl is not None:
+            ent.update(bound="mfma", flops=afl, tflops=afl / sec / 1e12, frac=afl / sec / 1e12 / PEAK_MFMA_F16_TFLOPS)
+        else:
+            ent.update(bound="hbm", GBs=ent["bytes"] / sec / 1e9, frac=ent["bytes"] / sec / 1e9 / PEAK_HBM_GBS)
         if fl is not None:
-            ent["tflops"] = fl / (tot_ms / cnt * 1e-3) / 1e12
             if label.startswith("matmul") and not is_split(label):     # one thunk = one launch
                 s_ = by_sym.setdefault(kernel_symbol(label), [0.0, set()])
                 s_[0] += tot_ms
@@ -297,6 +356,11 @@ def run_step(args):
     }
     model.close()
     ctx.close()
+    if capped is not None:
+        assert np.array_equal(np.asarray(loss).view(np.uint32), np.asarray(capped_loss).view(np.uint32)), \
+            "the capped run's loss differs from the uncapped run's"
+        capped["loss_bit_identical"] = True
+        out["config"]["capped"] = capped
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(LLAMA_3B)
     else:
@@ -816,6 +880,7 @@ def main():
                     help="cap of the device pool in GiB (0 = 90.01%% of the device); 16 exercises the host spill")
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-capped", action="store_true", help="skip the second run on a pool capped at 16 GiB")
     ap.add_argument("--ckpt-format", choices=["safetensors", "pickle"], default="safetensors",
                     help="file format of the ingest workload's checkpoint")
     ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest", "decode", "cycle"], default="step")

@@ -121,8 +121,9 @@ CACTI_API int cacti_ctx_timing_report(cacti_ctx *ctx, char *buf, size_t cap)
     int rc = ctx->c.collect_timings();
     if (rc) return rc;
     for (auto &kv : ctx->c.timings()) {
-        int w = snprintf(buf + n, cap - n, "%s %llu %.4f\n", kv.first.c_str(),
-                         (unsigned long long)kv.second.second, kv.second.first);
+        int w = snprintf(buf + n, cap - n, "%s %llu %.4f %llu\n", kv.first.c_str(),
+                         (unsigned long long)kv.second.second, kv.second.first,
+                         (unsigned long long)ctx->c.operand_bytes(kv.first));
         if (w < 0 || (size_t)w >= cap - n) break;
         n += (size_t)w;
     }

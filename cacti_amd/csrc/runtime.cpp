@@ -920,7 +920,12 @@ void Ctx::reset()
     while (cells_.size() > 1 && !cells_.back().alive) cells_.pop_back();
     log_.clear();
     uses_.clear();
-    if (pc_ > 0) eager_left_ = (cyc_eager_ + cyc_demand_down_ + cyc_dropped_) / 2;
+    if (pc_ > 0) {
+        // what the forward pass of the cycle that ends here needed: the early downloads of the cycle
+        // before it, and what it evicted itself
+        eager_left_ = (prev_eager_ + cyc_demand_down_ + cyc_dropped_) / 2;
+        prev_eager_ = cyc_eager_;
+    }
     cyc_eager_ = cyc_demand_down_ = cyc_dropped_ = 0;
     pf_cursor_ = 0;
     thunks_.clear();
@@ -1228,6 +1233,14 @@ int Ctx::run_entry(const Entry &e)
                 e1 = ev_pool_[ev_keys_.size()].second;
                 ev_keys_.push_back(key);
             }
+        }
+        if (timing) {
+            // operand bytes of one launch: every argument read once, every output written once,
+            // an output that is accumulated into read as well
+            uint64_t b = 0;
+            for (auto &t : aty) b += t.bytes();
+            for (size_t k = 0; k < oty.size(); k++) b += oty[k].bytes() * (((e.acc_mask >> k) & 1) ? 2 : 1);
+            op_bytes_[timing == 2 ? key : sp.key(aty, e.acc_mask)] = b;
         }
         if (timing) hipEventRecord(e0, stream_);
         rc = sp.run(*this, aty, ap.data(), oty, op.data(), e.acc_mask,

@@ -226,6 +226,11 @@ class Ctx {
     }
     int collect_timings();
     void clear_timings() { times_.clear(); }
+    uint64_t operand_bytes(const std::string &key) const
+    {
+        auto it = op_bytes_.find(key);
+        return it == op_bytes_.end() ? 0 : it->second;
+    }
     const std::map<std::string, std::pair<double, uint64_t>> &timings() const { return times_; }
 
    private:
@@ -247,7 +252,7 @@ class Ctx {
     // overlap the rest of it instead of the forward pass that needs the memory.  The budget is half
     // of what the cycle before evicted in any way: the other half is left to cells that are dropped
     // without a copy and come back on the upload stream, so that both directions of the link work.
-    size_t eager_left_ = 0, cyc_eager_ = 0, cyc_demand_down_ = 0, cyc_dropped_ = 0;
+    size_t eager_left_ = 0, cyc_eager_ = 0, prev_eager_ = 0, cyc_demand_down_ = 0, cyc_dropped_ = 0;
     bool in_eager_ = false;
     size_t pf_cursor_ = 0;                                       // entries before it have had their far prefetch
     int spill_eagerly(const Entry &e);
@@ -287,6 +292,7 @@ class Ctx {
     std::vector<std::pair<hipEvent_t, hipEvent_t>> ev_pool_;
     std::vector<std::string> ev_keys_;
     std::map<std::string, std::pair<double, uint64_t>> times_;
+    std::map<std::string, uint64_t> op_bytes_;                   // label -> operand bytes of one launch
     hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
     // cell_ingest: two page-locked staging buffers and the event after the last upload from each
     void *ingest_host_[2] = {nullptr, nullptr};

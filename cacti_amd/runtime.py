@@ -43,6 +43,7 @@ class MemPool:
 class Ctx:
     def __init__(self, dev=0, pool_bytes=0, host_pagelocked=True):
         self._c = C.c_void_p()
+        self.operand_bytes = {}   # label -> operand bytes of one launch (filled by timing_report)
         ffi.call("cacti_ctx_create", C.byref(self._c), dev, pool_bytes, int(host_pagelocked))
 
     def close(self):
@@ -79,8 +80,9 @@ class Ctx:
         ffi.call("cacti_ctx_timing_report", self._c, buf, len(buf))
         out = {}
         for line in buf.value.decode().splitlines():
-            name, cnt, ms = line.rsplit(" ", 2)
+            name, cnt, ms, nbytes = line.rsplit(" ", 3)
             out[name] = (int(cnt), float(ms))
+            self.operand_bytes[name] = int(nbytes)
         return out
 
     # ---- spine

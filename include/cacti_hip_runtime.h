@@ -54,8 +54,10 @@ void *cacti_ctx_stream(cacti_ctx *ctx);                 /* the hipStream_t all w
 /* per-thunk device times (CACTI_DEBUG_TIMING, src/ctx.rs:114-133).  mode 1 syncs after
  * every thunk; mode 2 records a HIP event pair around every launch without syncing and
  * reads them back in the report, so a run is measured undisturbed; 0 switches timing off
- * and clears the totals.  The report is text, one "label count total_ms" line per label;
- * GEMM labels carry the transposes and nblk x M x N x K.  A filter restricts mode 2 to the
+ * and clears the totals.  The report is text, one "label count total_ms operand_bytes" line
+ * per label (operand bytes of one launch: every argument read once, every output written
+ * once, an accumulated output read as well); GEMM labels carry the transposes and
+ * nblk x M x N x K.  A filter restricts mode 2 to the
  * launches whose label starts with the given text (an event pair costs a few microseconds
  * of stream time per launch, about 10 % of a whole step when every launch carries one);
  * NULL or "" matches every launch; of the matching launches every `every`-th is timed

@@ -274,15 +274,19 @@ def test_cached_pass_in_one_call_matches_the_training_forward_pass(oracle):
     from cacti_amd.runtime import LlamaCached
     cfg, flat, tok, lm_tok, scale = _inputs(seed=6)
     ctx, m = _gpu_model(cfg, flat)
-    m.step(tok, lm_tok, scale, want_grad=False)
-    io = m.io_cells()
-    ref = ctx.cell_get(io["logit"], np.float16, (cfg.S, cfg.V))
     k = LlamaCached(m, cfg.S)
     k.set_tokens(tok)
     k.apply(0, cfg.S)
     got = k.outputs()["logit"]
-    assert_parity(got, ref, "cached vs training forward")
-    assert np.mean(got.view(np.uint16) == ref.view(np.uint16)) > 0.95
+    # the cached pass runs the attention block as separate kernels: against the training pass staged
+    # the same way nearly every logit is the same f16; the fused attention thunk rounds its softmax
+    # differently in the last place, so there the bar is the parity tolerance alone
+    for mode, same in (("thunks", 0.95), ("fused", 0.0)):
+        m.set_attention(mode)
+        m.step(tok, lm_tok, scale, want_grad=False)
+        ref = ctx.cell_get(m.io_cells()["logit"], np.float16, (cfg.S, cfg.V))
+        assert_parity(got, ref, "cached vs training forward, attention " + mode)
+        assert np.mean(got.view(np.uint16) == ref.view(np.uint16)) > same
     k.close(); m.close(); ctx.close()
 
 
