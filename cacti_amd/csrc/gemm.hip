@@ -305,18 +305,16 @@ CACTI_API int cacti_hip_gemm_f16_strided_batched_tri(int ta, int tb, int64_t nbl
     if (vec >= 4 && !ta && tb && K <= 128 && beta == 0.f && tri <= 1)
         return gemm_nt_smallk_launch(p, nblk, st);
     // one to four rows against a weight matrix (decoding): a stream over B
-    static const bool no_skinny = getenv("CACTI_GEMM_NO_SKINNY") != nullptr;
-    if (vec == 8 && !ta && tb && M <= 4 && nblk == 1 && beta == 0.f && tri == 0 && !no_skinny)
+    if (vec == 8 && !ta && tb && M <= 4 && nblk == 1 && beta == 0.f && tri == 0)
         return gemm_skinny_nt_launch(M, N, K, alpha, p.A, lda, p.B, ldb, p.C, ldc, st);
     // The attention products with a [sequence, heads, head_dim] operand: A (probabilities or
     // their adjoint) is 16-byte aligned, B and C are per-head slabs whose offset (head_dim 100)
     // is only a multiple of 8 bytes.  Addressed from the 16-byte boundary below each slab they
     // take the direct-load path; the extra columns read stay inside the columns the blocks
     // cover in one row of B (checked here).
-    static const bool no_window = getenv("CACTI_GEMM_NO_WINDOW") != nullptr;
     if (vec == 4 && !tb && nblk > 1 && mult(K, 64) && mult(ta ? M : K, 8) && mult(lda, 8) &&
         mult(stride_a, 8) && aligned(A, 16) && mult(ldb, 8) && mult(ldc, 8) && aligned(B, 16) &&
-        aligned(C, 16) && (stride_b & 7) == (stride_c & 7) && !no_window) {
+        aligned(C, 16) && (stride_b & 7) == (stride_c & 7)) {
         const int64_t row_end = (nblk - 1) * stride_b + N;
         bool inside = stride_b >= 0 && row_end <= ldb;
         for (int64_t bz = 0; bz < nblk && inside; bz++) {

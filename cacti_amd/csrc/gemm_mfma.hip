@@ -1009,8 +1009,7 @@ int launch_auto(int tile, int64_t cols_main, int align, const GemmArgs &p, int64
         const int rc = launch_tile<TA, TB>(tile, align, a, nblk, st);
         // the remaining columns on 64 x 64 tiles loaded straight into LDS, three buffers (the
         // register path with two stages: 23.7 -> ~20 us for 448 columns at K = 3200)
-        static const int rem_tile = getenv("CACTI_GEMM_REM_TILE") ? atoi(getenv("CACTI_GEMM_REM_TILE")) : 8;
-        return rc ? rc : launch_tile<TA, TB>(rem_tile, align, b, nblk, st);
+        return rc ? rc : launch_tile<TA, TB>(8, align, b, nblk, st);
     }
     return launch_tile<TA, TB>(tile, align, p, nblk, st);
 }
@@ -1024,27 +1023,11 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
                      hipStream_t st)
 {
     GemmArgs q = p;
-    {
-        static int gm = 0, xcd = -1;
-        if (gm == 0) {
-            const char *e = getenv("CACTI_GEMM_GM");
-            gm = e ? atoi(e) : -1;                  // -1: chosen per launch
-            e = getenv("CACTI_GEMM_XCD");
-            xcd = e ? atoi(e) : 1;
-        }
-        q.gm = gm;
-        q.xcd = xcd;
-    }
+    q.gm = -1;                                    // rows of tiles per group: chosen per launch
+    q.xcd = 1;                                    // consecutive tiles to the workgroups of one XCD
     int64_t cols_main = 0;                        // > 0: a second launch takes the columns from here on
     if (tile < 0) {
-        static int forced = -2;
-        if (forced == -2) {
-            const char *e = getenv("CACTI_GEMM_TILE");
-            forced = e ? atoi(e) : -1;
-        }
-        if (forced >= 0) {
-            tile = forced;
-        } else {
+        {
             // measured on MI355X at the step's shapes (TFLOP/s on cold operands, register
             // path 128 x 128 or 256 x 128 -> direct loads).  A not transposed (forward and dgrad,
             // M = tokens): NT 661..821 -> 707..881, NN 702..787 -> 773..864 on 256 x 128, one
@@ -1052,18 +1035,14 @@ int gemm_mfma_launch(int ta, int tb, const GemmArgs &p, int64_t nblk, int align,
             // operands strided, weight-sized outputs): 256 x 256, 558..715 -> 755..932.
             // Small and batched products stay on 128 x 128 through registers.
             tile = 0;
-            static const bool no_direct = getenv("CACTI_GEMM_NO_DIRECT") != nullptr;
             // the attention products on per-head slabs: 128 x 128, 8 waves of 64 x 32, three
             // LDS buffers (-5 us per launch against the register path with 8 waves)
             if (p.win) tile = 7;
-            static const bool no_split = getenv("CACTI_GEMM_NO_SPLIT") != nullptr;
             // (a pointer-table batch is a handful of whole products: planned like a single one)
             if ((nblk == 1 || p.ztab) && p.M >= 1024 && p.N >= 1024) {
-                if (no_direct) {
-                    tile = ta ? 0 : 1;
-                } else if (!ta) {
+                if (!ta) {
                     const bool direct_ok = align >= 8 && p.K % BK == 0;     // else launch_tile ignores the tile
-                    const Plan plan = plan_tokens_product(p.M, p.N, direct_ok && p.tri == 0 && !no_split);
+                    const Plan plan = plan_tokens_product(p.M, p.N, direct_ok && p.tri == 0);
                     tile = plan.tile;
                     cols_main = plan.cols_main;
                 } else if (p.M >= 2048 && p.N >= 2048) {

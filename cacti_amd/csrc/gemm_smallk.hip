@@ -279,9 +279,8 @@ int gemm_nt_smallk_launch(const GemmArgs &p, int64_t nblk, hipStream_t st)
     // 2: 64.3, 3: 58.3, 4: 68.7, 5: 74.9, 6: 56.9, 7: 59.4, 8: 69.5, 16: 75.3 -- the counts of
     // workgroups per head that are powers of two (16 x 4, 16 x 2, ..) are the slow ones: the
     // workgroups resident together then write tiles whose addresses differ by multiples of the
-    // same large power of two.  CACTI_SMALLK_TPB overrides.
-    static const int tpb_env = getenv("CACTI_SMALLK_TPB") ? atoi(getenv("CACTI_SMALLK_TPB")) : 0;
-    a.tpb = tpb_env > 0 ? tpb_env : a.g.tiles_n >= 6 ? (a.g.tiles_n + 2) / 3 : kTilesPerBlock;
+    // same large power of two.
+    a.tpb = a.g.tiles_n >= 6 ? (a.g.tiles_n + 2) / 3 : kTilesPerBlock;
     a.chunks = (a.g.tiles_n + a.tpb - 1) / a.tpb;
     CACTI_REQUIRE(p.ldb < ((int64_t)1 << 22), CACTI_E_NOTIMPL, "gemm: ldb %lld too large for the short-K kernel",
                   (long long)p.ldb);

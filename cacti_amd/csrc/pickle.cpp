@@ -22,6 +22,7 @@
 #include <sys/stat.h>
 
 #include <algorithm>
+#include <deque>
 #include <memory>
 #include <unordered_map>
 
@@ -64,7 +65,7 @@ int zip_records(const MappedFile &mf, std::map<std::string, ZipRecord> *out)
         CACTI_REQUIRE(eocd >= 20 && rd32(b + eocd - 20) == 0x07064b50u, CACTI_E_FORMAT,
                       "pickle_dir: %s: ZIP64 locator missing", path);
         const uint64_t z = rd64(b + eocd - 20 + 8);
-        CACTI_REQUIRE(z <= n - 56 && rd32(b + z) == 0x06064b50u, CACTI_E_FORMAT, "pickle_dir: %s: ZIP64 record missing", path);
+        CACTI_REQUIRE(n >= 56 && z <= n - 56 && rd32(b + z) == 0x06064b50u, CACTI_E_FORMAT, "pickle_dir: %s: ZIP64 record missing", path);
         count = rd64(b + z + 32);
         cd_size = rd64(b + z + 40);
         cd_off = rd64(b + z + 48);
@@ -110,32 +111,40 @@ int zip_records(const MappedFile &mf, std::map<std::string, ZipRecord> *out)
     return 0;
 }
 
-// ---- pickle: a tree of plain values ---------------------------------------------------------------
+// ---- pickle: a graph of plain values --------------------------------------------------------------
+// The values belong to the unpickler that made them (one flat list, freed in a loop) and refer to each
+// other by plain pointers: a pickle can make a value its own descendant through the memo, or hang a
+// chain of any length below a value after that value was attached elsewhere, and neither may turn into
+// a leak or into a teardown that recurses once per level.  Nothing here walks the graph deeper than the
+// fixed shape of a tensor entry.
 struct PV;
-using P = std::shared_ptr<PV>;
+using P = PV *;
 struct PV {
     enum Kind { NONE, BOOL, INT, FLOAT, STR, BYTES, TUPLE, LIST, DICT, SET, GLOBAL, REDUCE, PERSID } kind = NONE;
     int64_t i = 0;
-    int depth = 1;                     // nesting below this value, bounded so that teardown cannot exhaust the call stack
+    int depth = 1;                     // nesting below this value when its children were attached (a sanity bound only)
     std::string s, s2;                 // STR / BYTES text; GLOBAL module, name
     std::vector<P> items;              // TUPLE, LIST, SET; DICT and REDUCE: key, value, key, value ...
-    P callable, args, state;           // REDUCE (+ BUILD state); PERSID: args = the id
+    P callable = nullptr, args = nullptr, state = nullptr;     // REDUCE (+ BUILD state); PERSID: args = the id
 };
-
-P mk(PV::Kind k)
-{
-    P v = std::make_shared<PV>();
-    v->kind = k;
-    return v;
-}
 
 struct Unpickler {
     static constexpr int kMaxDepth = 256;
+    static constexpr size_t kMaxValues = (size_t)1 << 22;       // values made + references held in containers
     const uint8_t *p, *end;
     std::vector<P> stack;
     std::vector<size_t> marks;
     std::unordered_map<uint64_t, P> memo;
     std::string err;
+    std::deque<PV> values;             // every value made; addresses stay put as it grows
+    size_t held = 0;                   // references stored in containers so far
+
+    P mk(PV::Kind k)
+    {
+        values.emplace_back();
+        values.back().kind = k;
+        return &values.back();
+    }
 
     bool fail(const char *what)
     {
@@ -207,6 +216,7 @@ struct Unpickler {
         if (stack.empty()) return fail("stack underflow");
         PV &d = *stack.back();
         if (d.kind != PV::DICT && d.kind != PV::REDUCE) return fail("items set on a value that is no dictionary");
+        held += kv.size();
         d.items.insert(d.items.end(), kv.begin(), kv.end());
         return nest(d, kv);
     }
@@ -215,6 +225,7 @@ struct Unpickler {
         if (stack.empty()) return fail("stack underflow");
         PV &d = *stack.back();
         if (d.kind != PV::LIST && d.kind != PV::SET && d.kind != PV::REDUCE) return fail("append to a value that is no list");
+        held += it.size();
         if (d.kind != PV::REDUCE) d.items.insert(d.items.end(), it.begin(), it.end());
         return d.kind == PV::REDUCE || nest(d, it);
     }
@@ -224,6 +235,7 @@ struct Unpickler {
         while (true) {
             if (!need(1)) return false;
             if (stack.size() > (1u << 24)) return fail("stack too deep");
+            if (values.size() + held > kMaxValues) return fail("too many values");
             const uint8_t op = *p++;
             P a, b2, c;
             std::vector<P> items;
@@ -258,6 +270,7 @@ struct Unpickler {
                 case 't': case 'l': case 0x91:                                                          // TUPLE, LIST, FROZENSET
                     if (!pop_mark(&items)) return false;
                     a = mk(op == 't' ? PV::TUPLE : op == 'l' ? PV::LIST : PV::SET);
+                    held += items.size();
                     a->items = std::move(items);
                     if (!nest(*a, a->items)) return false;
                     stack.push_back(a);
@@ -403,12 +416,16 @@ int add_pickle_file(cacti_tensors_dir *d, const std::string &path)
     CACTI_REQUIRE(pkl->method == 0, CACTI_E_FORMAT, "pickle_dir: %s: data.pkl is compressed", path.c_str());
     auto bo = recs.find(root + "byteorder");
     if (bo != recs.end()) {
+        CACTI_REQUIRE(bo->second.method == 0 && bo->second.size <= 16, CACTI_E_FORMAT,
+                      "pickle_dir: %s: the byteorder record is compressed or longer than a byte order's name", path.c_str());
         const std::string order(static_cast<const char *>(mf.base) + bo->second.data_off, (size_t)bo->second.size);
         CACTI_REQUIRE(order == "little", CACTI_E_NOTIMPL, "pickle_dir: %s: byte order %s is not read", path.c_str(), order.c_str());
     }
     const uint8_t *b = static_cast<const uint8_t *>(mf.base);
-    Unpickler up{b + pkl->data_off, b + pkl->data_off + pkl->size, {}, {}, {}, ""};
-    P top;
+    Unpickler up;
+    up.p = b + pkl->data_off;
+    up.end = up.p + pkl->size;
+    P top = nullptr;
     CACTI_REQUIRE(up.run(&top), CACTI_E_FORMAT, "pickle_dir: %s: data.pkl: %s", path.c_str(), up.err.c_str());
     // the state dictionary: a dict, or collections.OrderedDict() filled by SETITEMS
     CACTI_REQUIRE(top->kind == PV::DICT || (top->kind == PV::REDUCE && is_global(top->callable, "collections", "OrderedDict")),
@@ -450,7 +467,8 @@ int add_pickle_file(cacti_tensors_dir *d, const std::string &path)
             CACTI_REQUIRE(e.shape[a] >= 0, CACTI_E_FORMAT, "pickle_dir: %s: tensor %s: negative dimension", path.c_str(), nm);
             CACTI_REQUIRE((uint64_t)stride[a] == elems, CACTI_E_NOTIMPL,
                           "pickle_dir: %s: loading strided (non-packed) tensors is not supported: %s", path.c_str(), nm);
-            elems *= (uint64_t)e.shape[a];
+            CACTI_REQUIRE(!__builtin_mul_overflow(elems, (uint64_t)e.shape[a], &elems), CACTI_E_FORMAT,
+                          "pickle_dir: %s: tensor %s: element count exceeds 64 bits", path.c_str(), nm);
         }
         auto rec = recs.find(root + "data/" + pid->args->items[2]->s);
         CACTI_REQUIRE(rec != recs.end(), CACTI_E_FORMAT, "pickle_dir: %s: tensor %s: storage record %s missing", path.c_str(), nm,
@@ -458,14 +476,19 @@ int add_pickle_file(cacti_tensors_dir *d, const std::string &path)
         CACTI_REQUIRE(rec->second.method == 0, CACTI_E_FORMAT, "pickle_dir: %s: tensor %s: storage is compressed", path.c_str(), nm);
         // byte range: the tensor starts `start` elements into its storage and must fit what is left of it
         // (span <= rem_size, offset + rem_size == storage end: src/util/safepickle.rs:152-166)
+        CACTI_REQUIRE(pid->args->items[4]->i >= 0, CACTI_E_FORMAT, "pickle_dir: %s: tensor %s: negative storage size", path.c_str(), nm);
         const uint64_t start = (uint64_t)args->items[1]->i, numel = (uint64_t)pid->args->items[4]->i;
-        CACTI_REQUIRE(numel * esz == rec->second.size, CACTI_E_FORMAT,
+        // (no product that could wrap: numel is first held to what the record can hold)
+        CACTI_REQUIRE(esz > 0 && numel <= rec->second.size / esz && numel * esz == rec->second.size, CACTI_E_FORMAT,
                       "pickle_dir: %s: tensor %s: storage of %llu elements does not fill its %llu-byte record", path.c_str(), nm,
                       (unsigned long long)numel, (unsigned long long)rec->second.size);
         CACTI_REQUIRE(start <= numel && elems <= numel - start, CACTI_E_FORMAT,
                       "pickle_dir: %s: tensor %s does not fit its storage", path.c_str(), nm);
         e.off = rec->second.data_off + start * esz;
         e.eoff = e.off + elems * esz;
+        CACTI_REQUIRE(e.off <= e.eoff && e.eoff <= rec->second.data_off + rec->second.size &&
+                          rec->second.data_off + rec->second.size <= mf.size,
+                      CACTI_E_FORMAT, "pickle_dir: %s: tensor %s: byte range outside its record", path.c_str(), nm);
         // the reference insists on 64-byte alignment of the first byte (src/util/safepickle.rs:167-177)
         CACTI_REQUIRE(e.off % 64 == 0, CACTI_E_FORMAT, "pickle_dir: %s: tensor %s starts at byte %llu, not 64-byte aligned",
                       path.c_str(), nm, (unsigned long long)e.off);

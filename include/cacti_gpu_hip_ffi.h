@@ -156,7 +156,7 @@ int cacti_hip_accumulate_1d_u16(void *dst, const void *src, int64_t n, void *str
 /* RMSNorm, rms_norm closure src/librarium/llama.rs:442-451
  * (Cast op.rs:621, Square :2522, InnerMean :3150, AddScalar :1395, Sqrt :2609,
  *  BroadcastDiv :2358, BroadcastMul :2058, Cast).
- * x, y: [N,D] f16; w: [D] f16.  D % 8 == 0, D <= 16384. */
+ * x, y: [N,D] f16; w: [D] f16.  D % 8 == 0, D <= 8192. */
 int cacti_hip_rms_norm_fwd(int64_t N, int64_t D, const void *x, const void *w, float eps,
                            void *y, void *stream);
 /* The residual add in front of a norm and the norm in one pass over the rows:

@@ -221,6 +221,113 @@ def test_pickle_dir_errors(ingest, tmp_path):
     assert code(tmp_path / "norec.bin") == -7
 
 
+def _crafted(path, tensors, byteorder=None):
+    """A torch-style archive written by hand, so that the numbers in its pickle can lie: tensors maps a name
+    to (record bytes, storage numel, storage offset, shape, stride[, storage class]).  Records start 64-byte
+    aligned."""
+    import io
+    import pickle
+
+    class Storage:
+        def __init__(self, key, numel, cls):
+            self.key, self.numel, self.cls = key, numel, cls
+
+    class Tensor:
+        def __init__(self, st, off, shape, stride):
+            self.a = (st, off, tuple(shape), tuple(stride), False, collections.OrderedDict())
+
+        def __reduce__(self):
+            return (torch._utils._rebuild_tensor_v2, self.a)
+
+    class Pk(pickle.Pickler):
+        def persistent_id(self, obj):
+            return ("storage", obj.cls, obj.key, "cpu", obj.numel) if isinstance(obj, Storage) else None
+
+    sd = collections.OrderedDict()
+    for i, (name, (data, numel, off, shape, stride, *cls)) in enumerate(tensors.items()):
+        sd[name] = Tensor(Storage(str(i), numel, cls[0] if cls else torch.HalfStorage), off, shape, stride)
+    buf = io.BytesIO()
+    Pk(buf, protocol=2).dump(sd)
+    with zipfile.ZipFile(str(path), "w") as z:
+        z.writestr("archive/data.pkl", buf.getvalue())
+        if byteorder is not None:
+            z.writestr("archive/byteorder", byteorder[0], compress_type=byteorder[1])
+        for i, (data, *_) in enumerate(tensors.values()):
+            info = zipfile.ZipInfo("archive/data/%d" % i)
+            pos = z.fp.tell() + 30 + len(info.filename)
+            pad = (-(pos + 4)) % 64
+            info.extra = struct.pack("<HH", 0x4346, pad) + b"\0" * pad          # an unknown extra field as padding
+            z.writestr(info, data)
+
+
+def test_pickle_dir_refuses_numbers_that_wrap_or_point_outside(ingest, tmp_path):
+    """The element counts of a checkpoint are 64-bit numbers the file's author chose: products that wrap and
+    ranges outside the record must be refused, not turned into a mapping of other memory."""
+    from cacti_amd.ffi import CactiError
+
+    def code(path):
+        with pytest.raises(CactiError) as e:
+            ingest.PickleDir(path)
+        return e.value.code
+
+    x = np.arange(64, dtype=np.float16)
+    ok = tmp_path / "honest.bin"
+    _crafted(ok, {"t": (x.tobytes(), 64, 32, (4, 8), (8, 1))}, byteorder=(b"little", zipfile.ZIP_STORED))
+    d = ingest.PickleDir(ok)                                         # the hand-written archive itself is read
+    dt, arr = d.get("t")
+    assert dt == "F16" and arr.tobytes() == x[32:].tobytes()
+    d.close()
+    cases = {
+        "negative_numel": (x.tobytes(), -1, 0, (64,), (1,)),
+        "numel_wraps": (b"", 1 << 61, 1 << 60, (0,), (1,), torch.DoubleStorage),   # 2^61 * 8 bytes == 0 == the record's size, mod 2^64
+        "numel_short": (x.tobytes(), 65, 0, (65,), (1,)),
+        "shape_wraps": (x.tobytes(), 64, 0, (1 << 32, 1 << 32), (1 << 32, 1)),
+        "offset_past_end": (x.tobytes(), 64, 65, (0,), (1,)),
+        "negative_offset": (x.tobytes(), 64, -64, (64,), (1,)),
+        "too_long": (x.tobytes(), 64, 32, (33,), (1,)),
+    }
+    for name, t in cases.items():
+        _crafted(tmp_path / (name + ".bin"), {"t": t})
+        assert code(tmp_path / (name + ".bin")) == -7, name
+    _crafted(tmp_path / "bo_deflated.bin", {"t": (x.tobytes(), 64, 0, (64,), (1,))}, byteorder=(b"little" * 40, zipfile.ZIP_DEFLATED))
+    assert code(tmp_path / "bo_deflated.bin") == -7
+    _crafted(tmp_path / "bo_big.bin", {"t": (x.tobytes(), 64, 0, (64,), (1,))}, byteorder=(b"big", zipfile.ZIP_STORED))
+    assert code(tmp_path / "bo_big.bin") == -2
+    # 42 bytes that claim to be a ZIP64 archive: the 64-bit end record cannot lie inside the file
+    loc = struct.pack("<IIQI", 0x07064b50, 0, 0x10000000, 1)
+    eocd = struct.pack("<IHHHHIIH", 0x06054b50, 0xffff, 0xffff, 0xffff, 0xffff, 0xffffffff, 0xffffffff, 0)
+    open(str(tmp_path / "zip64_stub.bin"), "wb").write(loc + eocd)
+    assert code(tmp_path / "zip64_stub.bin") == -7
+
+
+def test_pickle_dir_survives_hostile_object_graphs(ingest, tmp_path):
+    """Pickles whose values form cycles or chains of any depth: built through the memo, so that no single
+    opcode nests deeply.  The library refuses or reads them; it neither recurses per level nor leaks."""
+    from cacti_amd.ffi import CactiError
+
+    def open_code(name, pkl):
+        with zipfile.ZipFile(str(tmp_path / name), "w") as z:
+            z.writestr("archive/data.pkl", pkl)
+        try:
+            ingest.PickleDir(tmp_path / name).close()
+            return 0
+        except CactiError as e:
+            return e.code
+
+    # a chain grown from its inner end: every new list is appended to the one before it, 300000 levels
+    step = b"]" + b"r\x00\x00\x00\x00" + b"a" + b"0" + b"j\x00\x00\x00\x00"
+    assert open_code("chain.bin", b"\x80\x02]" + b"r\x01\x00\x00\x00" + step * 300000 + b".") == -7
+    # the same chain below a dictionary, which is what a checkpoint's top value must be: read, and empty
+    grow = b"}q\x01" + b"X\x01\x00\x00\x00k" + b"]q\x00" + b"s" + b"h\x00" + step * 300000 + b"0h\x01."
+    assert open_code("chain_in_dict.bin", b"\x80\x02" + grow) == 0
+    assert open_code("self_list.bin", b"\x80\x02]q\x00h\x00a.") == -7                       # a list that holds itself
+    assert open_code("self_dict.bin", b"\x80\x02}q\x00X\x01\x00\x00\x00kh\x00s.") == 0      # a dictionary that does
+    two = b"\x80\x02]q\x00]q\x01h\x00a0h\x00h\x01a."                                        # two lists that hold each other
+    assert open_code("cycle2.bin", two) == -7
+    assert open_code("many.bin", b"\x80\x02" + b"]" * 5000000 + b".") == -7                  # more values than any checkpoint needs
+    assert open_code("wide.bin", b"\x80\x02](" + b"N" + b"2" * 5000000 + b"e.") == -7         # ... or references to one
+
+
 # ------------------------------------------------------------------------------------------ GPU
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", ["F16", "BF16"])
