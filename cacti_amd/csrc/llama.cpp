@@ -149,7 +149,8 @@ CACTI_API int cacti_resume_put(cacti_ctx *ctx, int cell, const void *host, size_
 }
 CACTI_API int cacti_cell_bytes(cacti_ctx *ctx, int cell, size_t *bytes)
 {
-    CACTI_REQUIRE(ctx && bytes && cell > 0, CACTI_E_INVALID, "cell_bytes: bad arguments");
+    CACTI_REQUIRE(ctx && bytes, CACTI_E_INVALID, "cell_bytes: null argument");
+    CACTI_REQUIRE(ctx->c.is_live(cell), CACTI_E_STATE, "cell_bytes: dead cell %d", cell);
     *bytes = ctx->c.cell(cell).ty.bytes();
     return 0;
 }

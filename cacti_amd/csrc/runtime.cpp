@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <thread>
 
+#include "../../include/cacti_hip_runtime.h"
 #include "common.h"
 
 namespace cacti {
@@ -160,15 +161,24 @@ int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
     CACTI_HIP(hipSetDevice(dev));
     size_t avail = 0, total = 0;
     CACTI_HIP(hipMemGetInfo(&avail, &total));
+    if (host_pagelocked < 0) host_pagelocked_ = cacti_env_host_pagelocked();
     if (pool_bytes == 0) {
-        // default reserve: 90.01 % of the device, src/ctx.rs:43, src/pctx/nvgpu.rs:1434-1463
-        size_t want = (size_t)(((unsigned __int128)total * 9001 + 9999) / 10000);
-        size_t room = avail > (512u << 20) ? avail - (512u << 20) : avail / 2;
-        pool_bytes = std::min(want, room);
+        // CACTI_VMEM_SOFT_LIMIT (a byte size with a unit, or a fraction of the device), else the
+        // default reserve of 90.01 % of the device: src/ctx.rs:43, src/pctx/nvgpu.rs:1434-1463
+        const char *lim = getenv("CACTI_VMEM_SOFT_LIMIT");
+        size_t want = 0;
+        int rc = cacti_vmem_soft_limit(lim, avail, total, &want);
+        if (rc) return rc;
+        if (!lim || !lim[0]) {                                    // the default gives way to other users of the device
+            const size_t room = avail > (512u << 20) ? avail - (512u << 20) : avail / 2;
+            want = std::min(want, room);
+        }
+        pool_bytes = want;
     }
     pool_bytes = (pool_bytes >> 16) << 16;                        // 64 KiB granules
     CACTI_REQUIRE(pool_bytes > 0 && pool_bytes <= avail, CACTI_E_OOM,
-                  "ctx: cannot reserve %zu bytes (%zu available of %zu); lower the pool cap",
+                  "ctx: cannot reserve %zu bytes (%zu available of %zu); lower the pool cap "
+                  "(the pool_bytes argument, or CACTI_VMEM_SOFT_LIMIT when that is 0)",
                   pool_bytes, avail, total);
     CACTI_HIP(hipMalloc((void **)&base_, pool_bytes));
     CACTI_REQUIRE(((uintptr_t)base_ % kAllocAlign) == 0, CACTI_E_STATE, "ctx: misaligned reserve");
@@ -240,6 +250,7 @@ CellPtr Ctx::cell_new(const CellType &ty, bool stable, const char *name)
     c.stable = stable;
     c.name = name ? name : "";
     cells_.push_back(std::move(c));
+    if (stable) stable_end_ = cells_.size();
     return (CellPtr)(cells_.size() - 1);
 }
 
@@ -319,8 +330,8 @@ int Ctx::cell_free_all(CellPtr ci)
 
 int Ctx::cell_put(CellPtr ci, const void *host, size_t bytes)
 {
+    CACTI_REQUIRE(is_live(ci), CACTI_E_STATE, "cell_put: dead cell %d", ci);
     Cell &c = cells_[ci];
-    CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "cell_put: dead cell %d", ci);
     CACTI_REQUIRE(bytes == c.ty.bytes(), CACTI_E_INVALID, "cell_put: %zu bytes given, cell %s has %zu",
                   bytes, c.name.c_str(), c.ty.bytes());
     // an earlier upload from this host buffer may still be in flight
@@ -335,8 +346,8 @@ int Ctx::cell_put(CellPtr ci, const void *host, size_t bytes)
 
 int Ctx::cell_get(CellPtr ci, void *host, size_t bytes)
 {
+    CACTI_REQUIRE(is_live(ci), CACTI_E_STATE, "cell_get: dead cell %d", ci);
     Cell &c = cells_[ci];
-    CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "cell_get: dead cell %d", ci);
     CACTI_REQUIRE(bytes == c.ty.bytes(), CACTI_E_INVALID, "cell_get: %zu bytes asked, cell %s has %zu",
                   bytes, c.name.c_str(), c.ty.bytes());
     if (c.v_valid) {
@@ -873,8 +884,8 @@ int Ctx::pool_alloc(size_t bytes, size_t *off, bool high)
 
 int Ctx::ensure_vmem(CellPtr ci, bool need_value)
 {
+    CACTI_REQUIRE(is_live(ci), CACTI_E_STATE, "use of dead cell %d", ci);
     Cell &c = cells_[ci];
-    CACTI_REQUIRE(ci > 0 && c.alive, CACTI_E_STATE, "use of dead cell %d (%s)", ci, c.name.c_str());
     if (c.voff == kNoOffset) {
         size_t off;
         int rc = pool_alloc(c.ty.bytes(), &off, c.stable);
@@ -916,8 +927,10 @@ void Ctx::reset()
             c.alive = false;
         }
     }
-    // compact trailing dead cells so ids do not grow without bound across cycles
-    while (cells_.size() > 1 && !cells_.back().alive) cells_.pop_back();
+    // compact trailing dead cells so ids do not grow without bound across cycles; never below an id
+    // that a stable cell has had: its owner may still hold the handle after freeing the cell, and
+    // must get "dead cell" for it, not whatever cell a later cycle would put there
+    while (cells_.size() > std::max<size_t>(1, stable_end_) && !cells_.back().alive) cells_.pop_back();
     log_.clear();
     uses_.clear();
     if (pc_ > 0) {

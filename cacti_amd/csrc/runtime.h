@@ -140,6 +140,8 @@ class Ctx {
     // ---- cells
     CellPtr cell_new(const CellType &ty, bool stable, const char *name = "");
     Cell &cell(CellPtr c) { return cells_[c]; }
+    // a handle from outside: in range and not freed
+    bool is_live(CellPtr c) const { return c > 0 && (size_t)c < cells_.size() && cells_[c].alive; }
     void set_const(CellPtr c) { cells_[c].konst = true; }
     int cell_put(CellPtr c, const void *host, size_t bytes);     // host -> cell (Mem, then VMem)
     int cell_get(CellPtr c, void *host, size_t bytes);           // cell -> host (syncs)
@@ -254,6 +256,7 @@ class Ctx {
     // without a copy and come back on the upload stream, so that both directions of the link work.
     size_t eager_left_ = 0, cyc_eager_ = 0, prev_eager_ = 0, cyc_demand_down_ = 0, cyc_dropped_ = 0;
     bool in_eager_ = false;
+    size_t stable_end_ = 0;                                      // one past the largest id a stable cell has had
     size_t pf_cursor_ = 0;                                       // entries before it have had their far prefetch
     int spill_eagerly(const Entry &e);
     int upload_ahead(Cell &c, bool *ordered);                    // one cell, on the upload stream

@@ -33,6 +33,14 @@ SIGNATURES = {
     "cacti_hip_stream_create_nonblocking": (ci, [pvp]),
     "cacti_hip_stream_destroy": (ci, [vp]),
     "cacti_hip_stream_sync": (ci, [vp]),
+    "cacti_hip_primary_ctx_retain": (ci, [ci, pvp]),
+    "cacti_hip_primary_ctx_release": (ci, [ci]),
+    "cacti_hip_primary_ctx_set_flags": (ci, [ci, C.c_uint]),
+    "cacti_hip_primary_ctx_reset": (ci, [ci]),
+    "cacti_hip_stream_null": (vp, []),
+    "cacti_parse_byte_size": (ci, [C.c_char_p, C.POINTER(C.c_uint64)]),
+    "cacti_vmem_soft_limit": (ci, [C.c_char_p, sz, sz, C.POINTER(sz)]),
+    "cacti_env_host_pagelocked": (ci, []),
     "cacti_hip_stream_wait_event": (ci, [vp, vp]),
     "cacti_hip_event_create": (ci, [pvp, ci]),
     "cacti_hip_event_destroy": (ci, [vp]),

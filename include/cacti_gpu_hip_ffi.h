@@ -67,6 +67,11 @@ int cacti_hip_memcpy_async(void *dst, const void *src, size_t bytes, void *strea
 int cacti_hip_memcpy_h2d_async(void *dst, const void *src, size_t bytes, void *stream); /* :254 */
 int cacti_hip_memcpy_d2h_async(void *dst, const void *src, size_t bytes, void *stream); /* :262 */
 int cacti_hip_memset_async(void *dst, int byte, size_t bytes, void *stream);
+int cacti_hip_primary_ctx_retain(int dev, void **pctx);         /* lib.rs:177 (hipDevicePrimaryCtxRetain) */
+int cacti_hip_primary_ctx_release(int dev);                     /* lib.rs:159       */
+int cacti_hip_primary_ctx_set_flags(int dev, unsigned flags);   /* lib.rs:186       */
+int cacti_hip_primary_ctx_reset(int dev);                       /* lib.rs:169       */
+void *cacti_hip_stream_null(void);                              /* lib.rs:512: the null stream's handle (NULL) */
 int cacti_hip_stream_create(void **stream);                     /* lib.rs:518       */
 int cacti_hip_stream_create_nonblocking(void **stream);         /* lib.rs:529       */
 int cacti_hip_stream_destroy(void *stream);                     /* lib.rs:493       */

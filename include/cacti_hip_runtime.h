@@ -45,8 +45,29 @@ typedef struct {
  * cap in bytes (the CACTI_VMEM_SOFT_LIMIT analogue, src/pctx/nvgpu.rs:1434-1463).  The pool
  * is ONE hipMalloc; when it is exhausted live cells are spilled to host memory
  * (_try_soft_oom, src/pctx/nvgpu.rs:2004-2283) and re-uploaded on their next use.
- * host_pagelocked: 1 = hipHostMalloc, 0 = malloc (CACTI_NVGPU_MEM_ALLOC, :995-1002). */
+ * host_pagelocked: 1 = hipHostMalloc, 0 = malloc (CACTI_NVGPU_MEM_ALLOC, :995-1002),
+ * -1 = what the environment says (cacti_env_host_pagelocked).  With pool_bytes = 0 the
+ * environment variable CACTI_VMEM_SOFT_LIMIT, when set, gives the reserve
+ * (cacti_vmem_soft_limit). */
 int cacti_ctx_create(cacti_ctx **ctx, int dev, size_t pool_bytes, int host_pagelocked);
+
+/* ---- configuration from the environment (cacti_cfg_env/src/lib.rs:47-234), as plain functions
+ * so that the rules can be checked without a device.
+ * cacti_parse_byte_size: "10 KB" = 10000, "16 KiB" = 16384, "0.2 MiB" = 209715, "123k" = 123000:
+ * a decimal number (fraction, exponent, '_' and blanks allowed), an optional prefix K M G T P E
+ * (powers of 1000; of 1024 when an 'i' follows), an optional B; results round to nearest
+ * (src/algo/str/parse_size.rs:262-400).  CACTI_E_INVALID for no number, a character that does
+ * not belong, or a result beyond 64 bits.
+ * cacti_vmem_soft_limit: the size of the device reserve for a CACTI_VMEM_SOFT_LIMIT text
+ * (NULL or "" = the default 90.01 % of `total`): a text that reads as a decimal number is a
+ * fraction of `total`, held to [0, 1] and to avail - 32 MiB; else a byte size; else the
+ * default; rounded down to 64 KiB (NvGpuMemPool::new, src/pctx/nvgpu.rs:1434-1463).  A bare
+ * integer reads as a decimal number, so a size in bytes needs its unit ("17179869184B").
+ * cacti_env_host_pagelocked: 1 when CACTI_GPU_MEM_ALLOC (else the reference's name,
+ * CACTI_NVGPU_MEM_ALLOC) is "pagelocked" (src/pctx/nvgpu.rs:995-1002), else 0. */
+int cacti_parse_byte_size(const char *text, uint64_t *bytes);
+int cacti_vmem_soft_limit(const char *text, size_t avail, size_t total, size_t *reserve);
+int cacti_env_host_pagelocked(void);
 int cacti_ctx_destroy(cacti_ctx *ctx);
 int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out);
 int cacti_ctx_sync(cacti_ctx *ctx);      /* stream sync + token-range status check */

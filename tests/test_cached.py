@@ -403,3 +403,32 @@ def test_full_size_decode_agrees_with_one_call_over_the_same_tokens():
     # distance between them is twice the distance of either from exact arithmetic
     assert_parity(got[512:], ref[512:], "decoded rows", l2=3e-3, mx=6e-2)
     k.close(); m.close(); ctx.close()
+
+
+@pytest.mark.gpu
+def test_handles_of_freed_caches_stay_dead(oracle):
+    """The caches are cells that live across cycles; once the cached model is closed their handles must name
+    dead cells for good, not the cells a later cycle happens to create."""
+    import ctypes as C
+    from cacti_amd import ffi
+    from cacti_amd.runtime import LlamaCached
+    cfg, flat, tok, lm_tok, scale = _inputs(seed=2)
+    ctx, m = _gpu_model(cfg, flat)
+    m.step(tok, lm_tok, scale, want_grad=False)
+
+    def live(i):
+        n = C.c_size_t()
+        return ffi.lib().cacti_cell_bytes(ctx._c, i, C.byref(n)) == 0
+
+    top0 = max(i for i in range(1, 4096) if live(i))
+    k = LlamaCached(m, cfg.S)
+    k.set_tokens(tok)
+    k.apply(0, 4)
+    k.outputs()
+    caches = [i for i in range(top0 + 1, top0 + 4096) if live(i)]
+    assert len(caches) >= 2 * cfg.L
+    k.close()
+    for _ in range(2):
+        m.step(tok, lm_tok, scale)                    # reset + a new cycle's cells
+        assert not any(live(i) for i in caches)
+    m.close(); ctx.close()

@@ -139,3 +139,51 @@ def test_random_two_ended_traffic_never_overlaps():
         p.free(off)
     s = p.stats()
     assert s["used"] == 0 and s["front"] == 0 and s["largest_free"] == cap
+
+
+# ---- the reserve's size from the environment (host only)
+def _parse(text):
+    import ctypes as C
+    from cacti_amd import ffi
+    out = C.c_uint64()
+    rc = ffi.lib().cacti_parse_byte_size(text.encode(), C.byref(out))
+    return None if rc else out.value
+
+
+def test_parse_byte_size_vectors():
+    """The examples the reference's parser documents (src/algo/str/parse_size.rs:126-129, 257-260)
+    and the corners of its rules."""
+    assert _parse("10 KB") == 10000 and _parse("20000") == 20000 and _parse("0.2 MiB") == 209715
+    assert _parse("^_^") is None and _parse("") is None and _parse("KB") is None
+    assert _parse("1 KB") == 1000 and _parse("1 KiB") == 1024 and _parse("1 MB") == 10 ** 6 and _parse("1 MiB") == 1 << 20
+    assert _parse("128 B") == 128 and _parse("16 KiB") == 16384 and _parse("123k") == 123000 and _parse("123KB") == 123000
+    assert _parse("16GiB") == 16 << 30 and _parse("16gib") == 16 << 30 and _parse("1_000_000") == 10 ** 6
+    assert _parse("1.5e3") == 1500 and _parse("1e3 KB") == 10 ** 6 and _parse("25e-1") == 3      # 2.5 rounds half up
+    assert _parse("1E") == 10 ** 18 and _parse("1Ei") == 1 << 60 and _parse("16E") == 16 * 10 ** 18
+    assert _parse("19E") is None                                                               # beyond 64 bits
+    assert _parse("18446744073709551615") == 2 ** 64 - 1 and _parse("18446744073709551616") is None
+    assert _parse("0.0000000000000000000000000000000000000001") == 0 and _parse("1e-50") == 0
+    assert _parse("1.2.3") is None and _parse("-5") is None and _parse("5 5") == 55
+
+
+def test_vmem_soft_limit_rules():
+    """NvGpuMemPool::new, src/pctx/nvgpu.rs:1434-1463: default 90.01 %, a decimal number is a fraction of the
+    device, anything else a byte size, rounded down to 64 KiB."""
+    import ctypes as C
+    from cacti_amd import ffi
+
+    def lim(text, avail, total):
+        out = C.c_size_t()
+        assert ffi.lib().cacti_vmem_soft_limit(None if text is None else text.encode(), avail, total, C.byref(out)) == 0
+        return out.value
+
+    total, avail = 288 * 10 ** 9, 287 * 10 ** 9
+    dflt = ((total * 9001 + 9999) // 10000) >> 16 << 16
+    assert lim(None, avail, total) == dflt and lim("", avail, total) == dflt and lim("lots", avail, total) == dflt
+    assert lim("0.5", avail, total) == (total // 2) >> 16 << 16
+    assert lim("16GiB", avail, total) == 16 << 30 and lim("16 GB", avail, total) == (16 * 10 ** 9) >> 16 << 16
+    assert lim("17179869184B", avail, total) == 16 << 30
+    full = (avail - (32 << 20)) >> 16 << 16
+    assert lim("1.0", avail, total) == full and lim("17179869184", avail, total) == full        # a bare integer is a fraction
+    assert lim("7", avail, total) == full and lim("-1", avail, total) == 0 and lim("nan", avail, total) == 0
+    assert lim("1e-3", avail, total) == (total // 1000) >> 16 << 16
