@@ -368,20 +368,23 @@ def run_step(args):
     return out
 
 
-def time_launches(fn, stream_sync, n_warm=3, n_iter=20):
-    """Average device time of fn(i) over n_iter back-to-back launches (torch events on the
-    current stream, which is the stream cacti_amd.ops launches on)."""
+def time_launches(fn, stream_sync, n_warm=3, n_iter=50):
+    """Median device time of fn(i) over n_iter launches, each between its own pair of events (torch
+    events on the current stream, which is the stream cacti_amd.ops launches on).  The pair brackets
+    everything fn(i) queues: a Python wrapper that allocates its outputs or issues a second small
+    kernel (the weight-gradient finalize of the RMSNorm adjoint) is timed with that included; the
+    kernel-trace summaries under profiles/ give the kernels alone."""
     import torch
     for i in range(n_warm):
         fn(i)
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_iter)]
     for i in range(n_iter):
+        ev[i][0].record()
         fn(i)
-    e1.record()
+        ev[i][1].record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / n_iter * 1e-3
+    return float(np.median([a.elapsed_time(b) for a, b in ev])) * 1e-3
 
 
 def run_adjoints(args):
@@ -445,9 +448,9 @@ def run_adjoints(args):
     p_out = [torch.zeros_like(s16[0]) for _ in range(2)]
     tri = 2 * H * (N * (N + 1) // 2)
     add("causal_softmax_fwd", time_launches(lambda i: ffi.call("cacti_hip_causal_softmax_fwd", N, H, s16[i % 2].data_ptr(),
-                                                               p_out[i % 2].data_ptr(), st), None, n_iter=10), 2 * tri)
+                                                               p_out[i % 2].data_ptr(), st), None), 2 * tri)
     add("causal_softmax_bwd", time_launches(lambda i: ffi.call("cacti_hip_causal_softmax_bwd", N, H, s16[i % 2].data_ptr(),
-                                                               dp.data_ptr(), p_out[i % 2].data_ptr(), st), None, n_iter=10), 3 * tri)
+                                                               dp.data_ptr(), p_out[i % 2].data_ptr(), st), None), 3 * tri)
     dom = max(res, key=lambda r: r["algorithmic_bytes"] if r["kernel"] == "silu_gate_bwd" else 0)
     return {"metric": "HBM-bound adjoint kernels at OpenLLaMA-3B shapes", "value": dom["achieved_GBs"],
             "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "dtype": "f16",
@@ -482,17 +485,40 @@ def run_gemm(args):
         M, K = (sa[1], sa[0]) if ta else sa
         Nn = sb[0] if tb else sb[1]
         out = torch.empty(M, Nn, device="cuda", dtype=torch.float16)
-        sec = time_launches(lambda i: ops.gemm(a, b, ta, tb, 1.0, 0.0, out), None, n_iter=10)
+        sec = time_launches(lambda i: ops.gemm(a, b, ta, tb, 1.0, 0.0, out), None)
         fl = 2.0 * M * Nn * K
-        res.append({"shape": name, "M": M, "N": Nn, "K": K, "us": sec * 1e6, "tflops": fl / sec / 1e12})
-        log("%-18s M=%5d N=%5d K=%5d %9.1f us %7.1f TFLOP/s" % (name, M, Nn, K, sec * 1e6, fl / sec / 1e12))
+        ent = {"shape": name, "M": M, "N": Nn, "K": K, "us": sec * 1e6, "tflops": fl / sec / 1e12}
+        if args.yardstick:
+            # the vendor library's GEMM (torch.matmul -> hipBLASLt) on the same operands: a yardstick for
+            # what these shapes allow on this device, no part of the product path
+            A_, B_ = (a.t() if ta else a), (b.t() if tb else b)
+            ysec = time_launches(lambda i: torch.matmul(A_, B_, out=out), None)
+            ent.update(library_us=ysec * 1e6, library_tflops=fl / ysec / 1e12)
+        res.append(ent)
+        log("%-18s M=%5d N=%5d K=%5d %9.1f us %7.1f TFLOP/s%s" % (name, M, Nn, K, sec * 1e6, fl / sec / 1e12,
+            "   library %9.1f us %7.1f TFLOP/s" % (ent["library_us"], ent["library_tflops"]) if args.yardstick else ""))
+    if args.sustain > 0:
+        # the largest product in a loop for that many seconds (sample the clocks from another shell
+        # meanwhile): the rate a power-limited device sustains, against the burst above
+        a, b = rn(N, D), rn(V, D, std=0.02)
+        out = torch.empty(N, V, device="cuda", dtype=torch.float16)
+        t_end, n, t0 = time.time() + args.sustain, 0, time.time()
+        while time.time() < t_end:
+            for _ in range(50):
+                ops.gemm(a, b, False, True, 1.0, 0.0, out)
+            torch.cuda.synchronize()
+            n += 50
+        dt = time.time() - t0
+        res.append({"shape": "head fwd NT, sustained %d s" % args.sustain, "M": N, "N": V, "K": D,
+                    "us": dt / n * 1e6, "tflops": 2.0 * N * V * D * n / dt / 1e12})
+        log("head fwd NT sustained over %.0f s: %.1f us, %.1f TFLOP/s" % (dt, dt / n * 1e6, res[-1]["tflops"]))
     q, k, v = rn(N, H, Dh), rn(N, H, Dh), rn(N, H, Dh)
-    sec = time_launches(lambda i: ops.block_matmul_qk(q, k, 0.1), None, n_iter=5)
+    sec = time_launches(lambda i: ops.block_matmul_qk(q, k, 0.1), None, n_iter=20)
     fl = 2.0 * H * N * N * Dh
     res.append({"shape": "attn QK^T (32 blocks)", "us": sec * 1e6, "tflops": fl / sec / 1e12})
     log("%-18s %9.1f us %7.1f TFLOP/s (dense)" % ("attn QK^T", sec * 1e6, fl / sec / 1e12))
     p = rn(N, H, N)
-    sec = time_launches(lambda i: ops.block_matmul_pv(p, v), None, n_iter=5)
+    sec = time_launches(lambda i: ops.block_matmul_pv(p, v), None, n_iter=20)
     res.append({"shape": "attn PV (32 blocks)", "us": sec * 1e6, "tflops": fl / sec / 1e12})
     log("%-18s %9.1f us %7.1f TFLOP/s (dense)" % ("attn PV", sec * 1e6, fl / sec / 1e12))
     best = max(r["tflops"] for r in res)
@@ -501,6 +527,59 @@ def run_gemm(args):
             "config": {"workload": "f16 GEMM, fp32 accumulate, f16 out"},
             "roofline": {"bound": "mfma", "achieved": best, "peak": PEAK_MFMA_F16_TFLOPS,
                          "unit": "TFLOP/s", "frac": best / PEAK_MFMA_F16_TFLOPS, "traffic": None},
+            "kernels": res}
+
+
+def run_attention(args):
+    """The fused causal attention thunk of one layer at the 3B shape (32 heads x 100, 2048 positions),
+    standalone through the C entry points with outputs and workspace allocated once: forward and adjoint,
+    against dense fp16 MFMA by their algorithmic flops (attention_flops)."""
+    import torch
+    from cacti_amd import ffi
+    cfg = LLAMA_3B
+    S, H, Dh = cfg["S"], cfg["H"], cfg["Dh"]
+    g = torch.Generator(device="cuda").manual_seed(0)
+    R = 4                                                   # operand sets in rotation
+
+    def rn():
+        return [torch.randn(S, H, Dh, device="cuda", generator=g).half() for _ in range(R)]
+
+    q, k, v, dO = rn(), rn(), rn(), rn()
+    o, dq, dk, dv = (torch.empty(S, H, Dh, device="cuda", dtype=torch.float16) for _ in range(4))
+    stats = torch.empty(ffi.lib().cacti_hip_attention_stats_bytes(S, H) // 4, device="cuda")
+    ws_bytes = ffi.lib().cacti_hip_attention_bwd_workspace(S, H)
+    ws = torch.empty(max(ws_bytes, 4) // 4, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    alpha = 1.0 / float(np.sqrt(np.float32(Dh)))
+    ld = H * Dh
+
+    def fwd(i):
+        ffi.call("cacti_hip_attention_fwd", S, H, Dh, alpha, q[i % R].data_ptr(), k[i % R].data_ptr(), v[i % R].data_ptr(),
+                 ld, o.data_ptr(), stats.data_ptr(), st)
+
+    def bwd(i):
+        ffi.call("cacti_hip_attention_bwd", S, H, Dh, alpha, q[0].data_ptr(), k[0].data_ptr(), v[0].data_ptr(),
+                 dO[i % R].data_ptr(), ld, stats.data_ptr(), dq.data_ptr(), 0, dk.data_ptr(), 0, dv.data_ptr(), 0,
+                 ws.data_ptr(), ws_bytes, st)
+
+    res = []
+    t_f = time_launches(fwd, None)
+    fwd(0)                                                  # the statistics of operand set 0 for the adjoint
+    t_b = time_launches(bwd, None)
+    tensor = S * H * Dh * 2
+    for label, sec, nbytes in (("attention", t_f, 4 * tensor + stats.numel() * 4),
+                               ("attention_bwd", t_b, 7 * tensor + stats.numel() * 4)):
+        fl = attention_flops(label, cfg)
+        res.append({"kernel": label, "us": sec * 1e6, "flops": fl, "bytes": nbytes, "tflops": fl / sec / 1e12,
+                    "frac": fl / sec / 1e12 / PEAK_MFMA_F16_TFLOPS, "bound": "mfma"})
+        log("%-14s %8.1f us  %6.1f TFLOP/s (algorithmic, %.1f%% of 2500)  operands %.1f MB"
+            % (label, sec * 1e6, fl / sec / 1e12, 100 * res[-1]["frac"], nbytes / 1e6))
+    tot = t_f + t_b
+    return {"metric": "fused causal attention of one layer, fwd + adjoint", "value": tot * 1e6, "unit": "us",
+            "n_gpus": 1, "higher_is_better": False, "dtype": "f16",
+            "config": {"workload": "causal attention, %d heads x %d, %d positions, one layer" % (H, Dh, S)},
+            "roofline": {"bound": "mfma", "kernel": "attn_bwd (dq + dkv kernels)", "achieved": res[1]["tflops"],
+                         "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": res[1]["frac"], "traffic": None},
             "kernels": res}
 
 
@@ -881,9 +960,11 @@ def main():
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debugging)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-capped", action="store_true", help="skip the second run on a pool capped at 16 GiB")
+    ap.add_argument("--yardstick", action="store_true", help="gemm workload: also time the vendor library on each shape")
+    ap.add_argument("--sustain", type=float, default=0.0, help="gemm workload: loop the largest product for this many seconds")
     ap.add_argument("--ckpt-format", choices=["safetensors", "pickle"], default="safetensors",
                     help="file format of the ingest workload's checkpoint")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "digests", "adamw", "ingest", "decode", "cycle"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "attention", "digests", "adamw", "ingest", "decode", "cycle"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -905,6 +986,8 @@ def main():
         out = run_decode(args)
     elif args.workload == "cycle":
         out = run_cycle(args)
+    elif args.workload == "attention":
+        out = run_attention(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)
