@@ -115,12 +115,17 @@ rope_kernel(int64_t S, int H, int Dh, int tok_per_block, const half_t *__restric
 // left half AND its partner pair (d + Dh/2, ..) of the right half: it reads both, then writes
 // both, so no lane reads what another lane writes and the kernel may run in place.  All
 // accesses are 4 bytes per lane and consecutive across lanes.
+// blockIdx.y = 1 works on a second tensor (in1 -> out1, acc1) with the same tables: the query and the
+// key of a layer in one launch.
 template <bool BWD>
 __global__ void __launch_bounds__(kThreads)
-rope_pair_kernel(int64_t S, int H, int Dh, const half_t *__restrict__ in,
-                 const half_t *__restrict__ cos16, const half_t *__restrict__ sin16, half_t *out,
-                 int acc)
+rope_pair_kernel(int64_t S, int H, int Dh, const half_t *__restrict__ in0,
+                 const half_t *__restrict__ cos16, const half_t *__restrict__ sin16, half_t *out0,
+                 int acc0, const half_t *__restrict__ in1, half_t *out1, int acc1)
 {
+    const half_t *__restrict__ in = blockIdx.y ? in1 : in0;
+    half_t *out = blockIdx.y ? out1 : out0;
+    const int acc = blockIdx.y ? acc1 : acc0;
     const int hf = Dh / 2, pph = hf / 2;            // pairs per half head
     const int64_t per_tok = (int64_t)H * pph, total = S * per_tok;
     for (int64_t it = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; it < total;
@@ -354,11 +359,17 @@ CACTI_API int cacti_hip_rope_tables(int64_t S, int64_t Dh, void *cos16, void *si
     return launch_status("rope_tables");
 }
 
+// in1 / out1 / acc1: an optional second tensor for the same launch (nullptr: none)
 static int rope_launch(bool bwd, int64_t S, int64_t H, int64_t Dh, const void *in, const void *c,
-                       const void *s, void *out, int acc, void *stream)
+                       const void *s, void *out, int acc, void *stream, const void *in1 = nullptr,
+                       void *out1 = nullptr, int acc1 = 0)
 {
     CACTI_REQUIRE(S > 0 && H > 0 && Dh > 0 && in && c && s && out, CACTI_E_INVALID,
                   "rope: null pointer or empty shape");
+    if (in1) {
+        CACTI_REQUIRE(out1 && Dh % 4 == 0 && aligned(c, 4) && aligned(s, 4) && aligned(in1, 16) && aligned(out1, 16),
+                      CACTI_E_NOTIMPL, "rope: two tensors in one launch need Dh %% 4 == 0 and aligned tensors");
+    }
     CACTI_REQUIRE(Dh % 2 == 0 && (H * Dh) % 8 == 0, CACTI_E_NOTIMPL,
                   "rope: need Dh even and H*Dh %% 8 == 0 (H=%lld Dh=%lld)", (long long)H,
                   (long long)Dh);
@@ -368,14 +379,17 @@ static int rope_launch(bool bwd, int64_t S, int64_t H, int64_t Dh, const void *i
     if (Dh % 4 == 0 && aligned(c, 4) && aligned(s, 4)) {
         const int64_t items = S * H * (Dh / 4);
         const int grid = grid_for(items, kThreads, 4096);
+        const dim3 g(grid, in1 ? 2 : 1);
         if (bwd)
-            hipLaunchKernelGGL(rope_pair_kernel<true>, dim3(grid), dim3(kThreads), 0,
+            hipLaunchKernelGGL(rope_pair_kernel<true>, g, dim3(kThreads), 0,
                                (hipStream_t)stream, S, (int)H, (int)Dh, (const half_t *)in,
-                               (const half_t *)c, (const half_t *)s, (half_t *)out, acc);
+                               (const half_t *)c, (const half_t *)s, (half_t *)out, acc,
+                               (const half_t *)in1, (half_t *)out1, acc1);
         else
-            hipLaunchKernelGGL(rope_pair_kernel<false>, dim3(grid), dim3(kThreads), 0,
+            hipLaunchKernelGGL(rope_pair_kernel<false>, g, dim3(kThreads), 0,
                                (hipStream_t)stream, S, (int)H, (int)Dh, (const half_t *)in,
-                               (const half_t *)c, (const half_t *)s, (half_t *)out, 0);
+                               (const half_t *)c, (const half_t *)s, (half_t *)out, 0,
+                               (const half_t *)in1, (half_t *)out1, 0);
         return launch_status("rope");
     }
     int tok = 2;
@@ -410,6 +424,31 @@ CACTI_API int cacti_hip_rope_bwd(int64_t S, int64_t H, int64_t Dh, const void *d
 {
     CACTI_REQUIRE(!(dx_acc && dx == dy), CACTI_E_INVALID, "rope_bwd: accumulate cannot run in place");
     return rope_launch(true, S, H, Dh, dy, cos16, sin16, dx, dx_acc, stream);
+}
+
+CACTI_API int cacti_hip_rope_fwd_pair(int64_t S, int64_t H, int64_t Dh, const void *x0, const void *x1,
+                                      const void *cos16, const void *sin16, void *y0, void *y1, void *stream)
+{
+    CACTI_REQUIRE(x1 && y1, CACTI_E_INVALID, "rope_fwd_pair: null pointer");
+    if (Dh % 4 != 0) {                            // the staged kernel takes one tensor per launch
+        const int rc = rope_launch(false, S, H, Dh, x0, cos16, sin16, y0, 0, stream);
+        return rc ? rc : rope_launch(false, S, H, Dh, x1, cos16, sin16, y1, 0, stream);
+    }
+    return rope_launch(false, S, H, Dh, x0, cos16, sin16, y0, 0, stream, x1, y1, 0);
+}
+
+CACTI_API int cacti_hip_rope_bwd_pair(int64_t S, int64_t H, int64_t Dh, const void *dy0, const void *dy1,
+                                      const void *cos16, const void *sin16, void *dx0, int dx0_acc, void *dx1,
+                                      int dx1_acc, void *stream)
+{
+    CACTI_REQUIRE(dy1 && dx1, CACTI_E_INVALID, "rope_bwd_pair: null pointer");
+    CACTI_REQUIRE(!(dx0_acc && dx0 == dy0) && !(dx1_acc && dx1 == dy1), CACTI_E_INVALID,
+                  "rope_bwd_pair: accumulate cannot run in place");
+    if (Dh % 4 != 0) {
+        const int rc = rope_launch(true, S, H, Dh, dy0, cos16, sin16, dx0, dx0_acc, stream);
+        return rc ? rc : rope_launch(true, S, H, Dh, dy1, cos16, sin16, dx1, dx1_acc, stream);
+    }
+    return rope_launch(true, S, H, Dh, dy0, cos16, sin16, dx0, dx0_acc, stream, dy1, dx1, dx1_acc);
 }
 
 CACTI_API int cacti_hip_silu_gate_fwd(int64_t n, const void *g, const void *u, void *h,

@@ -459,9 +459,15 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
         CellPtr pre, q, k, v, qr, kr, s16, p16, attn, o, post, up, gate, h, down;
         TRY(norm_of_stream(w.pre_norm, &pre));
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.q}, &q));
-        TRY(ap(c, make_rope(g.H), {q, m->cos, m->sin}, &qr));
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
-        TRY(ap(c, make_rope(g.H), {k, m->cos, m->sin}, &kr));
+        {
+            // symplectic_embed on the query and on the key (llama.rs:483, 490) as one two-output thunk:
+            // one launch, the values and the order of the adjoint's accumulations as with two thunks
+            std::vector<CellPtr> ro;
+            TRY(c.stage_apply(c.add_thunk(make_rope2(g.H)), {q, k, m->cos, m->sin}, &ro));
+            qr = ro[0];
+            kr = ro[1];
+        }
         TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.v}, &v));
         if (m->attention_mode == 0) {
             // scores, mask, softmax and the product with v as one thunk: the [S, H, S] cells of

@@ -331,6 +331,61 @@ struct RopeBwdSpec : ThunkSpec {
     }
 };
 
+// The map on the query and the key of a layer in one launch: (q, k, cos, sin) -> (qr, kr), adjoint
+// (dqr, dkr, cos, sin) -> (dq, dk); values as from two RopeSpec thunks.
+struct Rope2BwdSpec : ThunkSpec {
+    int64_t H;
+    explicit Rope2BwdSpec(int64_t h) : H(h) {}
+    const char *name() const override { return "rope2_bwd"; }
+    int arity() const override { return 4; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] % H == 0 && a[1] == a[0],
+                   "rope2_bwd: two dy f16 [S,H*Dh] expected");
+        o = {a[0], a[1]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        const auto &s = aty[0].shape;
+        return cacti_hip_rope_bwd_pair(s[0], H, s[1] / H, a[0], a[1], a[2], a[3], o[0], acc & 1, o[1], (acc >> 1) & 1, S(c));
+    }
+};
+
+struct Rope2Spec : ThunkSpec {
+    int64_t H;
+    explicit Rope2Spec(int64_t h) : H(h) {}
+    const char *name() const override { return "rope2"; }
+    int arity() const override { return 4; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] % H == 0 && a[1] == a[0] &&
+                       a[2].shape.size() == 2 && a[2].shape[0] >= a[0].shape[0] &&
+                       a[2].shape[1] == a[0].shape[1] / H && a[2] == a[3],
+                   "rope2: (q, k f16 [S,H*Dh], cos [S,Dh], sin [S,Dh]) expected");
+        o = {a[0], a[1]};
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t, void *, size_t) const override
+    {
+        const auto &s = aty[0].shape;
+        return cacti_hip_rope_fwd_pair(s[0], H, s[1] / H, a[0], a[1], a[2], a[3], o[0], o[1], S(c));
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        // one of the two without an adjoint: the single-tensor thunk for the other
+        if (!dy[0] && !dy[1]) return 0;
+        if (!dy[0] || !dy[1]) {
+            const int k = dy[0] ? 0 : 1;
+            return c.adj_add({e.args[k]}, std::unique_ptr<ThunkSpec>(new RopeBwdSpec(H)), {dy[k], e.args[2], e.args[3]});
+        }
+        return c.adj_add({e.args[0], e.args[1]}, std::unique_ptr<ThunkSpec>(new Rope2BwdSpec(H)),
+                         {dy[0], dy[1], e.args[2], e.args[3]});
+    }
+};
+
 struct RopeSpec : ThunkSpec {
     int64_t H;
     explicit RopeSpec(int64_t h) : H(h) {}
@@ -579,6 +634,7 @@ std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H)
     return std::unique_ptr<ThunkSpec>(new MatMulSpec(false, false, 1.f, H, CAUSAL_A));
 }
 std::unique_ptr<ThunkSpec> make_rope(int64_t H) { return std::unique_ptr<ThunkSpec>(new RopeSpec(H)); }
+std::unique_ptr<ThunkSpec> make_rope2(int64_t H) { return std::unique_ptr<ThunkSpec>(new Rope2Spec(H)); }
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H)
 {
     return std::unique_ptr<ThunkSpec>(new CausalSoftmaxSpec(H));

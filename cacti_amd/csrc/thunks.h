@@ -17,6 +17,7 @@ std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H);                    // (p16
 // the whole block (scores, mask, softmax, product with v) as one thunk: (q, k, v) -> o, row statistics
 std::unique_ptr<ThunkSpec> make_attention(float alpha, int64_t H);
 std::unique_ptr<ThunkSpec> make_rope(int64_t H);                      // (x [S,H*Dh], cos, sin) -> y
+std::unique_ptr<ThunkSpec> make_rope2(int64_t H);                     // (q, k, cos, sin) -> (qr, kr), one launch
 std::unique_ptr<ThunkSpec> make_causal_softmax(int64_t H);            // (s16 [S,H*S]) -> p16
 std::unique_ptr<ThunkSpec> make_add();                                // (a, b) -> y
 std::unique_ptr<ThunkSpec> make_add_rms_norm(float eps);              // (a, b, w) -> a + b, norm

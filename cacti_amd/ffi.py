@@ -68,6 +68,8 @@ SIGNATURES = {
     "cacti_hip_rope_tables": (ci, [i64, i64, vp, vp, vp]),
     "cacti_hip_rope_fwd": (ci, [i64, i64, i64, vp, vp, vp, vp, vp]),
     "cacti_hip_rope_bwd": (ci, [i64, i64, i64, vp, vp, vp, vp, ci, vp]),
+    "cacti_hip_rope_fwd_pair": (ci, [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp]),
+    "cacti_hip_rope_bwd_pair": (ci, [i64, i64, i64, vp, vp, vp, vp, vp, ci, vp, ci, vp]),
     "cacti_hip_silu_gate_fwd": (ci, [i64, vp, vp, vp, vp]),
     "cacti_hip_silu_gate_bwd": (ci, [i64, vp, vp, vp, vp, ci, vp, ci, vp]),
     "cacti_hip_causal_softmax_fwd": (ci, [i64, i64, vp, vp, vp]),

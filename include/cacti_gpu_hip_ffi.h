@@ -206,6 +206,13 @@ int cacti_hip_rope_fwd(int64_t S, int64_t H, int64_t Dh, const void *x, const vo
                        const void *sin16, void *y, void *stream);
 int cacti_hip_rope_bwd(int64_t S, int64_t H, int64_t Dh, const void *dy, const void *cos16,
                        const void *sin16, void *dx, int dx_acc, void *stream);
+/* The same on two tensors of one shape in one launch: the query and the key of a layer
+ * (src/librarium/llama.rs:483, 490 apply the map to both), results as from two calls. */
+int cacti_hip_rope_fwd_pair(int64_t S, int64_t H, int64_t Dh, const void *x0, const void *x1,
+                            const void *cos16, const void *sin16, void *y0, void *y1, void *stream);
+int cacti_hip_rope_bwd_pair(int64_t S, int64_t H, int64_t Dh, const void *dy0, const void *dy1,
+                            const void *cos16, const void *sin16, void *dx0, int dx0_acc, void *dx1,
+                            int dx1_acc, void *stream);
 
 /* SiLU gate, src/librarium/llama.rs:526-527: h = f16(f16(silu(g)) * u)
  * (StandardSiluFutThunkSpec op.rs:2867-2909, MulFutThunkSpec :2001-2055), and

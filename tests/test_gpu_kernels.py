@@ -532,3 +532,26 @@ def test_fused_attention(ops, oracle, S, H, Dh):
     dq2, dk2, dv2 = ops.attention_bwd(Q, K_, V_, DO, stats, alpha)
     for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
         assert_bits(host(a), host(b), "repeat")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("S,H,Dh", [(64, 4, 64), (2048, 32, 100), (37, 4, 20), (16, 4, 6)])
+def test_rope_on_two_tensors_in_one_launch(S, H, Dh):
+    """cacti_hip_rope_{fwd,bwd}_pair: bit for bit what two single launches give, accumulation included
+    (Dh = 6 takes the staged kernel, one launch per tensor behind the same entry point)."""
+    import torch
+    from cacti_amd import ffi, ops
+    g = torch.Generator(device="cuda").manual_seed(S + Dh)
+    x0, x1, a0, a1 = (torch.randn(S, H, Dh, device="cuda", generator=g).half() for _ in range(4))
+    cos, sin = ops.rope_tables(S, Dh)
+    st = torch.cuda.current_stream().cuda_stream
+    y0, y1 = torch.empty_like(x0), torch.empty_like(x1)
+    ffi.call("cacti_hip_rope_fwd_pair", S, H, Dh, x0.data_ptr(), x1.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+             y0.data_ptr(), y1.data_ptr(), st)
+    assert torch.equal(y0, ops.rope_fwd(x0, cos, sin)) and torch.equal(y1, ops.rope_fwd(x1, cos, sin))
+    d0, d1 = a0.clone(), torch.empty_like(x1)
+    ffi.call("cacti_hip_rope_bwd_pair", S, H, Dh, x0.data_ptr(), x1.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+             d0.data_ptr(), 1, d1.data_ptr(), 0, st)
+    w0 = a0.clone()
+    ffi.call("cacti_hip_rope_bwd", S, H, Dh, x0.data_ptr(), cos.data_ptr(), sin.data_ptr(), w0.data_ptr(), 1, st)
+    assert torch.equal(d0, w0) and torch.equal(d1, ops.rope_bwd(x1, cos, sin))
