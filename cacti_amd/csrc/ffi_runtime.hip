@@ -21,6 +21,9 @@ int hip_status(hipError_t e, const char *what)
 {
     if (e == hipSuccess) return 0;
     set_error("%s: %s (%d)", what, hipGetErrorString(e), (int)e);
+    // the runtime also remembers the failure per thread; it has been reported here, and left in place it
+    // would be taken for the status of the next kernel launch (launch_status reads that record)
+    (void)hipGetLastError();
     return (int)e;
 }
 

@@ -65,6 +65,11 @@ def test_primary_context_retain_release():
     ffi.call("cacti_hip_primary_ctx_release", 0)
     with pytest.raises(ffi.CactiError):
         ffi.call("cacti_hip_primary_ctx_retain", 4096, C.byref(a))   # no such device: a status, not an abort
+    # a reported failure does not linger as the status of the next kernel launch
+    import torch
+    from cacti_amd import ops
+    x = torch.ones(8, 16, device="cuda", dtype=torch.float16)
+    assert torch.equal(ops.add_f16(x, x), x + x)
 
 
 def test_reserve_sized_from_the_environment(monkeypatch):
