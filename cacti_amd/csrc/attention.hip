@@ -139,6 +139,91 @@ struct TileLoader {
     }
 };
 
+// 16 bytes from device memory at an address that is only 8-byte aligned (the heads of a [S, H, 100]
+// tensor start every 200 bytes): one global_load_dwordx4, which needs dword alignment only
+typedef uint32_t u32x4_a8_t __attribute__((ext_vector_type(4), aligned(8)));
+__device__ __forceinline__ uint4 gload16(gptr_t q)
+{
+    const u32x4_a8_t v = *reinterpret_cast<const __attribute__((address_space(1))) u32x4_a8_t *>(q);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+// Per-lane constants of the mapping between a 64 x Dh tile of a [S, H, Dh] tensor and its LDS tile, for
+// the 256 lanes of one wave group: piece `it` of a lane (16 bytes, 4 per lane) is row r0 + 16 it,
+// columns 8 pc .. 8 pc + 7, r0 = lane / 16, pc = lane % 16.  Its element offset from the tile's first
+// row is goff0 + 16 it ld (a wave-uniform step), its byte offset in the LDS tile loff + 4096 it (16
+// more rows leave the chunk swizzle g(r) as it is).  A memory instruction costs the address unit the
+// same for 8 as for 16 bytes per lane, and the address unit, not the arithmetic, is what these kernels
+// wait for: 4 loads per tile and lane instead of 8.  Lanes whose columns lie beyond the head load a
+// duplicate and store nothing: the pad columns of every tile buffer are zeroed once when the kernel
+// starts.  The piece that straddles the end of the head (Dh % 8 = 4: columns Dh - 4 .. Dh + 3) is
+// loaded 4 columns early, so that it stays inside the head, and shifted into place.
+struct FastTileMap {
+    unsigned goff0, loff;
+    int r0, gcol;
+    int64_t ld;
+    bool colok, tail, narrow;                            // narrow: a head of 4 columns, one 8-byte piece per row
+    __device__ __forceinline__ FastTileMap(int64_t ld_, int Dh)
+    {
+        const int t = threadIdx.x & (kNT - 1), pc = t & 15;
+        r0 = t >> 4;
+        ld = ld_;
+        narrow = Dh < 8;
+        colok = pc * 8 < Dh;
+        tail = !narrow && colok && pc * 8 + 8 > Dh;
+        gcol = narrow ? 0 : tail ? Dh - 8 : min(pc * 8, Dh - 8);
+        goff0 = (unsigned)(r0 * ld_ + gcol);
+        loff = (unsigned)toff(r0, pc);
+    }
+};
+
+__device__ __forceinline__ void zero_lds(unsigned char *smem, int bytes)
+{
+    for (int o = threadIdx.x * 16; o < bytes; o += blockDim.x * 16) *reinterpret_cast<uint4 *>(smem + o) = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+}
+
+// 64 rows x Dh of a [S, H, Dh] tensor -> registers -> LDS tile, by the 256 lanes of one wave group, with
+// the constants above (the forward kernel; the adjoint kernels have no registers to spare for them and
+// keep the loader further up: with this one the dQ kernel spills 16 registers and runs 7 % slower).
+// Whole tiles take the straight path: 4 loads at a lane-constant offset from 4 uniform row pointers, 4
+// stores at a lane-constant LDS address with immediate offsets.  The last tile of a ragged sequence
+// clamps its rows and zeroes the ones beyond the end.
+struct FastTileLoader {
+    static constexpr int NP = kTileRows * 16 / kNT;      // 16-byte pieces per lane
+    uint4 v[NP];
+    int rows;                                            // rows of the tile inside the tensor (uniform)
+    // src = &X[row0][head column 0]; rows_left = S - row0 >= 1
+    __device__ __forceinline__ void load(const FastTileMap &m, gptr_t src, int rows_left)
+    {
+        rows = __builtin_amdgcn_readfirstlane(min(rows_left, kTileRows));
+        if (m.narrow) {
+#pragma unroll
+            for (int it = 0; it < NP; it++) {
+                const uint2 a = gload8(src + (int64_t)min(m.r0 + 16 * it, rows - 1) * m.ld);
+                v[it] = make_uint4(a.x, a.y, 0u, 0u);
+            }
+        } else if (rows == kTileRows) {
+#pragma unroll
+            for (int it = 0; it < NP; it++) v[it] = gload16(src + (int64_t)(16 * it) * m.ld + m.goff0);
+        } else {
+#pragma unroll
+            for (int it = 0; it < NP; it++) v[it] = gload16(src + (int64_t)min(m.r0 + 16 * it, rows - 1) * m.ld + m.gcol);
+        }
+    }
+    __device__ __forceinline__ void store(const FastTileMap &m, unsigned char *tile) const
+    {
+        if (!m.colok) return;
+#pragma unroll
+        for (int it = 0; it < NP; it++) {
+            uint4 x = v[it];
+            if (m.tail) x = make_uint4(x.z, x.w, 0u, 0u);
+            if (rows != kTileRows && m.r0 + 16 * it >= rows) x = make_uint4(0u, 0u, 0u, 0u);
+            *reinterpret_cast<uint4 *>(tile + m.loff + 4096 * it) = x;
+        }
+    }
+};
+
 // The fixed operand of a lane: row `row` of a [S, H, Dh] tensor as KS fragments (k step ks: the 8
 // halves at d = 16 ks + 8 lh ..), zero beyond Dh and for rows beyond S
 template <int KS>
@@ -299,6 +384,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    zero_lds(smem, 2 * kGroupLds);                 // the pad columns of the tile buffers: zero from here on
     // wave-uniform values kept in scalar registers, so that the branches on them are scalar branches
     const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8), tig = threadIdx.x & (kNT - 1);
     unsigned char *Ks = smem + g * kGroupLds, *Vs = Ks + 2 * kTileB;
@@ -317,19 +403,20 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 
         const int kend = min(i0 + kBM, S);                 // keys [0, kend) are visible to the tile
         const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
-        TileLoader tk, tv;
+        const FastTileMap tm(ld, Dh);
+        FastTileLoader tk, tv;
 
         // ---- pass 1: row maximum and sum; each lane over its half of the keys of its group's tiles
         float m_run = -INFINITY, l_run = 0.f;
         if (g < njt) {
-            tk.load(K + (int64_t)g * kTileRows * ld, ld, S - g * kTileRows, Dh);
-            tk.store(Ks);
+            tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+            tk.store(tm, Ks);
         }
         __syncthreads();
         for (int it = 0; it < niter; it++) {
             const int jt = 2 * it + g, cur = it & 1;
             const bool nxt = jt + 2 < njt;
-            if (nxt) tk.load(K + (int64_t)(jt + 2) * kTileRows * ld, ld, S - (jt + 2) * kTileRows, Dh);
+            if (nxt) tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
             if (jt < njt) {
 #pragma unroll
                 for (int kt = 0; kt < 2; kt++) {
@@ -365,7 +452,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                     }
                 }
             }
-            if (nxt) tk.store(Ks + (cur ^ 1) * kTileB);
+            if (nxt) tk.store(tm, Ks + (cur ^ 1) * kTileB);
             __syncthreads();
         }
         float m, l;
@@ -401,18 +488,18 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
         if (g < njt) {
-            tk.load(K + (int64_t)g * kTileRows * ld, ld, S - g * kTileRows, Dh);
-            tv.load(V + (int64_t)g * kTileRows * ld, ld, S - g * kTileRows, Dh);
-            tk.store(Ks);
-            tv.store(Vs);
+            tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+            tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+            tk.store(tm, Ks);
+            tv.store(tm, Vs);
         }
         __syncthreads();
         for (int it = 0; it < niter; it++) {
             const int jt = 2 * it + g, cur = it & 1;
             const bool nxt = jt + 2 < njt;
             if (nxt) {
-                tk.load(K + (int64_t)(jt + 2) * kTileRows * ld, ld, S - (jt + 2) * kTileRows, Dh);
-                tv.load(V + (int64_t)(jt + 2) * kTileRows * ld, ld, S - (jt + 2) * kTileRows, Dh);
+                tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
+                tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
             }
             if (jt < njt) {
 #pragma unroll
@@ -437,8 +524,8 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                 }
             }
             if (nxt) {
-                tk.store(Ks + (cur ^ 1) * kTileB);
-                tv.store(Vs + (cur ^ 1) * kTileB);
+                tk.store(tm, Ks + (cur ^ 1) * kTileB);
+                tv.store(tm, Vs + (cur ^ 1) * kTileB);
             }
             __syncthreads();
         }
