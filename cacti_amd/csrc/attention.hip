@@ -184,8 +184,8 @@ __device__ __forceinline__ void zero_lds(unsigned char *smem, int bytes)
 }
 
 // 64 rows x Dh of a [S, H, Dh] tensor -> registers -> LDS tile, by the 256 lanes of one wave group, with
-// the constants above (the forward kernel; the adjoint kernels have no registers to spare for them and
-// keep the loader further up: with this one the dQ kernel spills 16 registers and runs 7 % slower).
+// the constants above (the forward and the dK / dV kernel; the dQ kernel has no registers to spare for
+// them and keeps the loader further up: with this one it spills 16 registers and runs 7 % slower).
 // Whole tiles take the straight path: 4 loads at a lane-constant offset from 4 uniform row pointers, 4
 // stores at a lane-constant LDS address with immediate offsets.  The last tile of a ragged sequence
 // clamps its rows and zeroes the ones beyond the end.
@@ -678,6 +678,7 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    zero_lds(smem, 4 * kTileB);                    // the pad columns of the tile buffers: zero from here on
     unsigned char *Qs = smem, *Gs = smem + 2 * kTileB;
     float *St = reinterpret_cast<float *>(smem + 4 * kTileB);          // [2][4][64]: m, l, y, sigma of the tile's rows
     const int lane = threadIdx.x & 63, wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l32 = lane & 31,
@@ -708,25 +709,26 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 vacc[dt][r] = 0.f;
             }
         const int iq0 = c00 / kTileRows, niq = (S + kTileRows - 1) / kTileRows;
-        TileLoader tq, tg;
+        const FastTileMap tm(ld, Dh);
+        FastTileLoader tq, tg;
         float st;
         auto load_stat = [&](int iq) __attribute__((always_inline)) {
             const int row = iq * kTileRows + lane;
             const float t = stat_src[row < S ? row : S - 1];
             st = row < S ? t : stat_pad;
         };
-        tq.load(Q + (int64_t)iq0 * kTileRows * ld, ld, S - iq0 * kTileRows, Dh);
-        tg.load(G + (int64_t)iq0 * kTileRows * ld, ld, S - iq0 * kTileRows, Dh);
+        tq.load(tm, Q + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows);
+        tg.load(tm, G + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows);
         load_stat(iq0);
-        tq.store(Qs);
-        tg.store(Gs);
+        tq.store(tm, Qs);
+        tg.store(tm, Gs);
         St[wid * 64 + lane] = st;
         __syncthreads();
         for (int iq = iq0; iq < niq; iq++) {
             const int cur = (iq - iq0) & 1;
             if (iq + 1 < niq) {
-                tq.load(Q + (int64_t)(iq + 1) * kTileRows * ld, ld, S - (iq + 1) * kTileRows, Dh);
-                tg.load(G + (int64_t)(iq + 1) * kTileRows * ld, ld, S - (iq + 1) * kTileRows, Dh);
+                tq.load(tm, Q + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows);
+                tg.load(tm, G + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows);
                 load_stat(iq + 1);
             }
             const float *stc = St + cur * 256;
@@ -760,8 +762,8 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 prod_tr<DT>(kacc, Qs + cur * kTileB, 32 * qb, pack8(de), pack8(de + 8), lane);
             }
             if (iq + 1 < niq) {
-                tq.store(Qs + (cur ^ 1) * kTileB);
-                tg.store(Gs + (cur ^ 1) * kTileB);
+                tq.store(tm, Qs + (cur ^ 1) * kTileB);
+                tg.store(tm, Gs + (cur ^ 1) * kTileB);
                 St[(cur ^ 1) * 256 + wid * 64 + lane] = st;
             }
             __syncthreads();
