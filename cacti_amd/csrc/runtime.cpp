@@ -351,6 +351,11 @@ int Ctx::cell_get(CellPtr ci, void *host, size_t bytes)
     CACTI_REQUIRE(bytes == c.ty.bytes(), CACTI_E_INVALID, "cell_get: %zu bytes asked, cell %s has %zu",
                   bytes, c.name.c_str(), c.ty.bytes());
     if (c.v_valid) {
+        if (c.v_ready) {                       // uploaded ahead of its use: the upload may still be under way
+            CACTI_HIP(hipStreamWaitEvent(stream_, c.v_ready, 0));
+            ev_put(c.v_ready);
+            c.v_ready = nullptr;
+        }
         CACTI_HIP(hipMemcpyAsync(host, dev_ptr(c.voff), bytes, hipMemcpyDeviceToHost, stream_));
         CACTI_HIP(hipStreamSynchronize(stream_));
         bytes_d2h_ += bytes;
