@@ -387,6 +387,35 @@ def time_launches(fn, stream_sync, n_warm=3, n_iter=50):
     return float(np.median([a.elapsed_time(b) for a, b in ev])) * 1e-3
 
 
+def cpu_baseline_adjoints(N, D, H, Dh, F, V):
+    """The CPU port (the oracle, OpenMP) on the same adjoint shapes, one call each after a warm-up call;
+    value = GB/s of the SiLU-gate adjoint by its algorithmic bytes, like the GPU line."""
+    from oracle import oracle as o
+    r = np.random.default_rng(0)
+    rn = lambda *s: r.standard_normal(s, dtype=np.float32).astype(np.float16)
+    x, dy, w = rn(N, D), rn(N, D), rn(D)
+    cos, sin = o.rope_tables(N, Dh)
+    q = rn(N, H, Dh)
+    g_, u_, dh_ = rn(N, F), rn(N, F), rn(N, F)
+    rows = 256                                                    # softmax-CE: a slice of the rows, scaled up
+    lg = (r.standard_normal((rows, V), dtype=np.float32) * 2).astype(np.float16)
+    tok = r.integers(0, V, rows).astype(np.uint16)
+    sc = np.full(rows, 1.0 / N, np.float32)
+    jobs = {"rms_norm_bwd": (lambda: o.rmsnorm_bwd(x, w, 1e-6, dy), 1.0), "rope_bwd": (lambda: o.rope_bwd(q, cos, sin), 1.0),
+            "silu_gate_bwd": (lambda: o.silu_gate_bwd(g_, u_, dh_), 1.0),
+            "softmax_ce_bwd": (lambda: o.softmax_ce_bwd(lg, tok, sc), N / rows)}
+    per = {}
+    for name, (fn, scale) in jobs.items():
+        fn()
+        t0 = time.time()
+        fn()
+        per[name] = (time.time() - t0) * scale * 1e6
+        log("cpu_baseline: oracle %-16s %10.0f us" % (name, per[name]))
+    return {"value": 5 * 2 * N * F / (per["silu_gate_bwd"] * 1e-6) / 1e9, "unit": "GB/s", "cores": o.num_threads(), "kind": "port",
+            "sample": "oracle, one call per kernel at the full shapes (softmax-CE: %d of %d rows, scaled)" % (rows, N),
+            "per_kernel_us": per}
+
+
 def run_adjoints(args):
     """BASELINE config 2-4 kernels at 3B shapes; buffers rotate over > 256 MB so every launch
     reads HBM, not the Infinity Cache."""
@@ -452,13 +481,14 @@ def run_adjoints(args):
     add("causal_softmax_bwd", time_launches(lambda i: ffi.call("cacti_hip_causal_softmax_bwd", N, H, s16[i % 2].data_ptr(),
                                                                dp.data_ptr(), p_out[i % 2].data_ptr(), st), None), 3 * tri)
     dom = max(res, key=lambda r: r["algorithmic_bytes"] if r["kernel"] == "silu_gate_bwd" else 0)
+    cpu = None if args.no_cpu_baseline else cpu_baseline_adjoints(N, D, H, Dh, F, V)
     return {"metric": "HBM-bound adjoint kernels at OpenLLaMA-3B shapes", "value": dom["achieved_GBs"],
             "unit": "GB/s", "n_gpus": 1, "higher_is_better": True, "dtype": "f16",
             "config": {"workload": "adjoint microbench: RMSNorm [2048,3200], RoPE [2048,32,100], "
                                    "SiLU-gate [2048,8640], softmax-CE [2048,32000], causal softmax [2048,32,2048] (causal half)"},
             "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["achieved_GBs"],
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_of_8TBs"], "traffic": None},
-            "kernels": res}
+            "cpu_baseline": cpu, "kernels": res}
 
 
 def run_gemm(args):
@@ -575,12 +605,27 @@ def run_attention(args):
         log("%-14s %8.1f us  %6.1f TFLOP/s (algorithmic, %.1f%% of 2500)  operands %.1f MB"
             % (label, sec * 1e6, fl / sec / 1e12, 100 * res[-1]["frac"], nbytes / 1e6))
     tot = t_f + t_b
+    cpu = None
+    if not args.no_cpu_baseline:
+        # the CPU port (the oracle's chain of separate thunks) on 4 of the 32 heads, scaled
+        from oracle import oracle as o
+        hs = 4
+        qc, kc, vc, gc = (t[0][:, :hs].contiguous().cpu().numpy() for t in (q, k, v, dO))
+        t0 = time.time()
+        o.attention_fwd(qc, kc, vc, alpha)
+        t1 = time.time()
+        o.attention_bwd(qc, kc, vc, gc, alpha)
+        t2 = time.time()
+        cpu = {"value": ((t1 - t0) + (t2 - t1)) * H / hs * 1e6, "unit": "us", "cores": o.num_threads(), "kind": "port",
+               "sample": "oracle attention_fwd + attention_bwd (dense, as the reference executes it) on %d of %d heads, "
+                         "scaled: fwd %.0f us, bwd %.0f us" % (hs, H, (t1 - t0) * H / hs * 1e6, (t2 - t1) * H / hs * 1e6)}
+        log("cpu_baseline: " + cpu["sample"])
     return {"metric": "fused causal attention of one layer, fwd + adjoint", "value": tot * 1e6, "unit": "us",
             "n_gpus": 1, "higher_is_better": False, "dtype": "f16",
             "config": {"workload": "causal attention, %d heads x %d, %d positions, one layer" % (H, Dh, S)},
             "roofline": {"bound": "mfma", "kernel": "attn_bwd (dq + dkv kernels)", "achieved": res[1]["tflops"],
                          "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": res[1]["frac"], "traffic": None},
-            "kernels": res}
+            "cpu_baseline": cpu, "kernels": res}
 
 
 def run_digests(args):
