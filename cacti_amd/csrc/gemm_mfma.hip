@@ -734,8 +734,7 @@ gemm_mfma_kernel(GemmArgs p)
         const int cb = DMA ? cbv : (t & 1), nb1 = next_buf(cb);
         if (MAIN || t + LOOK < nk) {
             if (DMA) {
-                const int dst = NBUF == 2 ? nb1 : next_buf(nb1);
-                static_assert(!DMA || NBUF == 2 || NBUF == 3, "destination buffer above");
+                const int dst = cb == 0 ? NBUF - 1 : cb - 1;      // the buffer tile t - 1 has left
                 la.dma(lds_addr(As + dst * BM * BK), Ao, (int64_t)(t + LOOK) * BK);
                 lb.dma(lds_addr(Bs + dst * BN * BK), Bo, (int64_t)(t + LOOK) * BK);
             } else {
@@ -920,7 +919,8 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
 // tile: 0 = 128 x 128 on 4 waves, two register stages (every loader is branch-free on 256
 // lanes); 1 = 256 x 128 on 8 waves, two register stages; 3 = 64 x 64 on 4 waves; 4 = 256 x 128,
 // 5 = 256 x 256 (128 x 64 per wave), 6 = 256 x 192 (64 x 96 per wave) and 7 = 128 x 128 (64 x 32
-// per wave) on 8 waves with both operands loaded straight into LDS
+// per wave) on 8 waves with both operands loaded straight into LDS; 8 = 64 x 64 on 4 waves the same way,
+// five k tiles ahead
 template <bool TA, bool TB>
 int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_t st)
 {
@@ -940,7 +940,7 @@ int launch_tile(int tile, int align, const GemmArgs &p, int64_t nblk, hipStream_
         case 5: return launch_cfg<TA, TB, 256, 256, 2, 4, 8, false, 1, 2, true>(p, nblk, st);
         case 6: return launch_cfg<TA, TB, 256, 192, 4, 2, 8, false, 1, 2, true>(p, nblk, st);
         case 7: return launch_cfg<TA, TB, 128, 128, 2, 4, 8, false, 1, 3, true>(p, nblk, st);
-        case 8: return launch_cfg<TA, TB, 64, 64, 2, 2, 8, false, 1, 3, true>(p, nblk, st);
+        case 8: return launch_cfg<TA, TB, 64, 64, 2, 2, 8, false, 1, 6, true>(p, nblk, st);
         default: return launch_cfg<TA, TB, 256, 128, 4, 2, 8, false, 2>(p, nblk, st);
     }
 }
@@ -1007,8 +1007,10 @@ int launch_auto(int tile, int64_t cols_main, int align, const GemmArgs &p, int64
         b.B = p.B + (TB ? a.N * p.ldb : a.N);
         b.C = p.C + a.N;
         const int rc = launch_tile<TA, TB>(tile, align, a, nblk, st);
-        // the remaining columns on 64 x 64 tiles loaded straight into LDS, three buffers (the
-        // register path with two stages: 23.7 -> ~20 us for 448 columns at K = 3200)
+        // the remaining columns on 64 x 64 tiles loaded straight into LDS, six buffers: a tile this
+        // small has 4 MFMAs per wave and k tile, so a k step costs the latency of its loads unless
+        // they were issued several steps earlier (448 columns at K = 3200: register path with two
+        // stages 23.7 us, three buffers 21.4, six 15.2 .. 16.5)
         return rc ? rc : launch_tile<TA, TB>(8, align, b, nblk, st);
     }
     return launch_tile<TA, TB>(tile, align, p, nblk, st);
