@@ -60,7 +60,8 @@ struct AttnArgs {
     const half_t *q, *k, *v, *dO;
     half_t *out, *dq, *dk, *dv;
     float *m, *l;                        // [H][S] row maximum and sum (forward output)
-    float *y, *sig;                      // [H][S] reciprocal of l, sigma (adjoint scratch)
+    float *y, *sig;                      // [H][S] adjoint scratch: sigma, and 1 / l (exact arithmetic) or the
+                                         // exponent offset m log2(e) + log2(l) (fast arithmetic) of each row
     int acc_dq, acc_dk, acc_dv;
 };
 
@@ -314,8 +315,8 @@ __device__ __forceinline__ float recip_refined(float l)
 
 // The f32 arithmetic between the rounding points.  EXACT: exponential with range reduction and a
 // correctly rounded quotient, the arithmetic of the separate softmax kernels; FAST: v_exp_f32 of the
-// scaled difference and a multiplication by the reciprocal (a few ulp of f32 away, two thirds of the
-// instructions).
+// scaled difference, with the division folded into the exponent (exp2_mix below; a few ulp of f32
+// away, under half of the instructions).
 template <bool FAST>
 struct AttnMath {
     static __device__ __forceinline__ float ex(float s, float m)
@@ -329,6 +330,40 @@ struct AttnMath {
         return div_by(exp_diff(s, m), l, y);
     }
 };
+
+// FAST arithmetic on scores that stay f16 between their rounding point and the exponent: one fused
+// multiply-add that reads the f16 value (v_fma_mix_f32) forms s log2(e) - c, where c holds the row's
+// maximum (and, for a probability, log2 of the row's sum as well), and v_exp_f32 does the rest.
+constexpr float kLog2e = 0x1.715476p+0f;
+typedef _Float16 half2v_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float exp2_mix(half_t s, float c)
+{
+    return __builtin_amdgcn_exp2f(__builtin_fmaf((float)s, kLog2e, -c));
+}
+// maximum of 16 f16 values (exact in f16), two per instruction
+__device__ __forceinline__ float max16(const half_t (&h)[16])
+{
+    half2v_t mx = {h[0], h[1]};
+#pragma unroll
+    for (int e = 2; e < 16; e += 2) mx = __builtin_elementwise_max(mx, half2v_t{h[e], h[e + 1]});
+    return (float)__builtin_fmaxf16(mx[0], mx[1]);
+}
+// 16 f32 -> f16 (round to nearest even), two per instruction
+typedef float float2v_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void round16(half_t (&h)[16], const float16_t &a)
+{
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        const half2v_t t = __builtin_convertvector(float2v_t{a[e], a[e + 1]}, half2v_t);
+        h[e] = t[0];
+        h[e + 1] = t[1];
+    }
+}
+// the exponent offset of a row's probabilities: m log2(e) + log2(l)
+__device__ __forceinline__ float prob_shift(float m, float l)
+{
+    return __builtin_fmaf(m, kLog2e, __builtin_amdgcn_logf(l));
+}
 
 // 4 consecutive d of one output row: f16(scale a[0..3] [+ old])
 __device__ __forceinline__ void store_row4(half_t *dst, float a0, float a1, float a2, float a3, float scale,
@@ -425,7 +460,30 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                     const float16_t acc = prod_direct<KS>(Ks + cur * kTileB, 32 * kt, qf, l32, lh);
                     const bool full = kb + 31 <= r0;
                     float sv[16], mt = -INFINITY, sum = 0.f;
-                    if (full) {                          // no masks on tiles wholly below the diagonal
+                    if constexpr (FAST) {
+                        half_t sh[16];
+                        if (full) {
+#pragma unroll
+                            for (int e = 0; e < 16; e++) sh[e] = f2h(p.alpha * acc[e]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 16; e++) {
+                                const int key = kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+                                sh[e] = key <= myrow ? f2h(p.alpha * acc[e]) : (half_t)-INFINITY;
+                            }
+                        }
+                        const float m_new = fmaxf(m_run, max16(sh)), c = m_new * kLog2e;
+                        if (full) {
+#pragma unroll
+                            for (int e = 0; e < 16; e++) sum += exp2_mix(sh[e], c);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 16; e++)
+                                sum += (sh[e] == (half_t)-INFINITY) ? 0.f : exp2_mix(sh[e], c);
+                        }
+                        l_run = ((m_run == -INFINITY) ? 0.f : l_run * M::ex(m_run, m_new)) + sum;
+                        m_run = m_new;
+                    } else if (full) {                   // no masks on tiles wholly below the diagonal
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             sv[e] = rnd16(p.alpha * acc[e]);
@@ -480,6 +538,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             }
         }
         const float y = recip_refined(l);
+        const float cs = prob_shift(m, l);
 
         // ---- pass 2: probabilities and O
         float16_t oacc[DT];
@@ -509,7 +568,18 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                     const float16_t acc = prod_direct<KS>(Ks + cur * kTileB, 32 * kt, qf, l32, lh);
                     const bool full = kb + 31 <= r0;
                     float pe[16];
-                    if (full) {
+                    if constexpr (FAST) {
+                        if (full) {
+#pragma unroll
+                            for (int e = 0; e < 16; e++) pe[e] = exp2_mix(f2h(p.alpha * acc[e]), cs);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 16; e++) {
+                                const int key = kb + 8 * (e >> 2) + 4 * lh + (e & 3);
+                                pe[e] = key <= myrow ? exp2_mix(f2h(p.alpha * acc[e]), cs) : 0.f;
+                            }
+                        }
+                    } else if (full) {
 #pragma unroll
                         for (int e = 0; e < 16; e++) pe[e] = M::prob(rnd16(p.alpha * acc[e]), m, l, y);
                     } else {
@@ -578,6 +648,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             l = 1.f;
         }
         const float y = recip_refined(l);
+        const float cs = prob_shift(m, l);
 
         const int kend = min(i0 + kBM, S);
         const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
@@ -609,7 +680,29 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
                         const float16_t pacc = prod_direct<KS>(Vs + cur * kTileB, 32 * kt, gf, l32, lh);
                         const bool full = kb + 31 <= r0;
                         float de[16];
-                        if (full) {
+                        if constexpr (FAST) {
+                            // sigma and dS with the f16 value of dP read by the fused multiply-add
+                            half_t dph[16];
+                            round16(dph, pacc);
+                            if (full) {
+#pragma unroll
+                                for (int e = 0; e < 16; e++) {
+                                    const float pr_ = exp2_mix(f2h(p.alpha * sacc[e]), cs);
+                                    const half_t dp = dph[e];
+                                    if (PASS == 0) part = __builtin_fmaf((float)dp, pr_, part);
+                                    else de[e] = __builtin_fmaf((float)dp, pr_, -(sig * pr_));
+                                }
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < 16; e++) {
+                                    const bool live = kb + 8 * (e >> 2) + 4 * lh + (e & 3) <= myrow;
+                                    const float pr_ = exp2_mix(f2h(p.alpha * sacc[e]), cs);
+                                    const half_t dp = dph[e];
+                                    if (PASS == 0) part += live ? (float)dp * pr_ : 0.f;
+                                    else de[e] = live ? __builtin_fmaf((float)dp, pr_, -(sig * pr_)) : 0.f;
+                                }
+                            }
+                        } else if (full) {
 #pragma unroll
                             for (int e = 0; e < 16; e++) {
                                 const float pr_ = M::prob(rnd16(p.alpha * sacc[e]), m, l, y);
@@ -645,7 +738,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             __syncthreads();
             sig = xs[wid * 32 + l32] + xs[kBM + wid * 32 + l32];
             if (g == 0 && lh == 0 && myrow < S) {
-                p.y[(int64_t)h * S + myrow] = y;
+                p.y[(int64_t)h * S + myrow] = FAST ? cs : y;      // what the dK / dV kernel wants per row
                 p.sig[(int64_t)h * S + myrow] = sig;
             }
         }
@@ -715,7 +808,7 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
         auto load_stat = [&](int iq) __attribute__((always_inline)) {
             const int row = iq * kTileRows + lane;
             const float t = stat_src[row < S ? row : S - 1];
-            st = row < S ? t : stat_pad;
+            st = row < S ? t : stat_pad;          // rows beyond S are masked; the pad only has to be finite
         };
         tq.load(tm, Q + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows);
         tg.load(tm, G + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows);
@@ -740,24 +833,40 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 const float16_t pacc = prod_direct<KS>(Gs + cur * kTileB, 32 * qb, vf, l32, lh);
                 const bool full = qb0 >= c0 + 31 && qb0 + 32 <= S;
                 float pe[16], de[16];
+                half_t dph[16];
+                if constexpr (FAST) round16(dph, pacc);
+                auto elems = [&](auto full_c) __attribute__((always_inline)) {
+                    constexpr bool FULL = decltype(full_c)::value;
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const int qi = 32 * qb + 8 * q + 4 * lh;
-                    const float4_t mm = *reinterpret_cast<const float4_t *>(stc + 0 * 64 + qi);
-                    const float4_t ll = *reinterpret_cast<const float4_t *>(stc + 1 * 64 + qi);
-                    const float4_t yy = *reinterpret_cast<const float4_t *>(stc + 2 * 64 + qi);
-                    const float4_t sg = *reinterpret_cast<const float4_t *>(stc + 3 * 64 + qi);
+                    for (int q = 0; q < 4; q++) {
+                        const int qi = 32 * qb + 8 * q + 4 * lh;
+                        float4_t mm, ll;
+                        if constexpr (!FAST) {
+                            mm = *reinterpret_cast<const float4_t *>(stc + 0 * 64 + qi);
+                            ll = *reinterpret_cast<const float4_t *>(stc + 1 * 64 + qi);
+                        }
+                        const float4_t yy = *reinterpret_cast<const float4_t *>(stc + 2 * 64 + qi);
+                        const float4_t sg = *reinterpret_cast<const float4_t *>(stc + 3 * 64 + qi);
 #pragma unroll
-                    for (int r = 0; r < 4; r++) {
-                        const int e = 4 * q + r, query = iq * kTileRows + qi + r;
-                        const float pr_ = M::prob(rnd16(p.alpha * sacc[e]), mm[r], ll[r], yy[r]);
-                        const float tt = pr_ * rnd16(pacc[e]);
-                        const float ds = tt - sg[r] * pr_;
-                        const bool live = full || (query >= mykey && query < S);
-                        pe[e] = live ? pr_ : 0.f;
-                        de[e] = live ? ds : 0.f;
+                        for (int r = 0; r < 4; r++) {
+                            const int e = 4 * q + r, query = iq * kTileRows + qi + r;
+                            float pr_, ds;
+                            if constexpr (FAST) {                 // yy holds the exponent offset of the row
+                                pr_ = exp2_mix(f2h(p.alpha * sacc[e]), yy[r]);
+                                ds = __builtin_fmaf((float)dph[e], pr_, -(sg[r] * pr_));
+                            } else {
+                                pr_ = M::prob(rnd16(p.alpha * sacc[e]), mm[r], ll[r], yy[r]);
+                                const float tt = pr_ * rnd16(pacc[e]);
+                                ds = tt - sg[r] * pr_;
+                            }
+                            const bool live = FULL || (query >= mykey && query < S);
+                            pe[e] = live ? pr_ : 0.f;
+                            de[e] = live ? ds : 0.f;
+                        }
                     }
-                }
+                };
+                if (full) elems(std::true_type{});           // no masks on blocks wholly past the diagonal
+                else elems(std::false_type{});
                 prod_tr<DT>(vacc, Gs + cur * kTileB, 32 * qb, pack8(pe), pack8(pe + 8), lane);
                 prod_tr<DT>(kacc, Qs + cur * kTileB, 32 * qb, pack8(de), pack8(de + 8), lane);
             }
