@@ -212,15 +212,33 @@ struct FastTileLoader {
             for (int it = 0; it < NP; it++) v[it] = gload16(src + (int64_t)min(m.r0 + 16 * it, rows - 1) * m.ld + m.gcol);
         }
     }
+    // the straddling piece moves into place by four selects per piece and the test for a ragged tile is
+    // made once (a shuffle under a lane mask per piece took five times the instructions: forward and
+    // dK / dV kernel -4 us each)
     __device__ __forceinline__ void store(const FastTileMap &m, unsigned char *tile) const
     {
         if (!m.colok) return;
+        if (rows == kTileRows) {
 #pragma unroll
-        for (int it = 0; it < NP; it++) {
-            uint4 x = v[it];
-            if (m.tail) x = make_uint4(x.z, x.w, 0u, 0u);
-            if (rows != kTileRows && m.r0 + 16 * it >= rows) x = make_uint4(0u, 0u, 0u, 0u);
-            *reinterpret_cast<uint4 *>(tile + m.loff + 4096 * it) = x;
+            for (int it = 0; it < NP; it++) {
+                uint4 x;
+                x.x = m.tail ? v[it].z : v[it].x;
+                x.y = m.tail ? v[it].w : v[it].y;
+                x.z = m.tail ? 0u : v[it].z;
+                x.w = m.tail ? 0u : v[it].w;
+                *reinterpret_cast<uint4 *>(tile + m.loff + 4096 * it) = x;
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < NP; it++) {
+                const bool in = m.r0 + 16 * it < rows;
+                uint4 x;
+                x.x = !in ? 0u : m.tail ? v[it].z : v[it].x;
+                x.y = !in ? 0u : m.tail ? v[it].w : v[it].y;
+                x.z = (!in || m.tail) ? 0u : v[it].z;
+                x.w = (!in || m.tail) ? 0u : v[it].w;
+                *reinterpret_cast<uint4 *>(tile + m.loff + 4096 * it) = x;
+            }
         }
     }
 };
