@@ -99,46 +99,10 @@ __device__ __forceinline__ half8_t as_h8(uint2 lo, uint2 hi)
     return f;
 }
 
-// 64 rows x Dh of a [S, H, Dh] tensor -> registers -> LDS tile (zero beyond Dh and beyond the last row),
-// by the 256 lanes of one wave group.  (Loading straight into LDS with global_load_lds_dword -- dword
-// granularity because the heads of a [S, H, 100] tensor start on 8-byte, not 16-byte, boundaries --
-// was measured slower: 2.5 times the memory instructions, forward 126 -> 153 us.)
-struct TileLoader {
-    static constexpr int NP = kTileRows * 32 / kNT;      // 8-byte pieces per lane
-    uint2 v[NP];
-    unsigned okbits;                                     // bit it: piece it lies inside the tensor
-    // src = &X[row0][head column 0]; rows_left = S - row0 >= 1
-    __device__ __forceinline__ void load(gptr_t src, int64_t ld, int rows_left, int Dh)
-    {
-#pragma unroll
-        for (int it = 0; it < NP; it++) {
-            const int p = (threadIdx.x & (kNT - 1)) + it * kNT;
-            const int row = p >> 5, pc = p & 31;
-            // every lane loads from an address inside the tile (row and column clamped) and the pieces
-            // beyond it are zeroed afterwards: a load under a lane mask is waited for where the mask ends
-            const int rc = min(row, rows_left - 1), cc = min(pc * 4, Dh - 4);
-            v[it] = gload8(src + (int64_t)rc * ld + cc);
-        }
-        // the zeroing waits for the data, so it is left to store(): here only which pieces it concerns
-        okbits = 0;
-#pragma unroll
-        for (int it = 0; it < NP; it++) {
-            const int p = (threadIdx.x & (kNT - 1)) + it * kNT;
-            okbits |= ((p >> 5) < rows_left && (p & 31) * 4 < Dh) ? 1u << it : 0u;
-        }
-    }
-    __device__ __forceinline__ void store(unsigned char *tile) const
-    {
-#pragma unroll
-        for (int it = 0; it < NP; it++) {
-            const int p = (threadIdx.x & (kNT - 1)) + it * kNT;
-            const int row = p >> 5, pc = p & 31;
-            const bool ok = (okbits >> it) & 1;
-            *reinterpret_cast<uint2 *>(tile + toff(row, pc >> 1) + ((pc & 1) << 3)) =
-                make_uint2(ok ? v[it].x : 0u, ok ? v[it].y : 0u);
-        }
-    }
-};
+// The K / V (Q / dO) tiles go from device memory through registers into LDS.  (Loading straight into LDS
+// with global_load_lds_dword -- dword granularity because the heads of a [S, H, 100] tensor start on
+// 8-byte, not 16-byte, boundaries -- was measured slower: 2.5 times the memory instructions, forward
+// 126 -> 153 us.)
 
 // 16 bytes from device memory at an address that is only 8-byte aligned (the heads of a [S, H, 100]
 // tensor start every 200 bytes): one global_load_dwordx4, which needs dword alignment only
@@ -186,7 +150,7 @@ __device__ __forceinline__ void zero_lds(unsigned char *smem, int bytes)
 
 // 64 rows x Dh of a [S, H, Dh] tensor -> registers -> LDS tile, by the 256 lanes of one wave group, with
 // the constants above (the forward and the dK / dV kernel; the dQ kernel has no registers to spare for
-// them and keeps the loader further up: with this one it spills 16 registers and runs 7 % slower).
+// it -- it spills 56 registers with it -- and uses the 8-byte form further down).
 // Whole tiles take the straight path: 4 loads at a lane-constant offset from 4 uniform row pointers, 4
 // stores at a lane-constant LDS address with immediate offsets.  The last tile of a ragged sequence
 // clamps its rows and zeroes the ones beyond the end.
@@ -238,6 +202,61 @@ struct FastTileLoader {
                 x.z = (!in || m.tail) ? 0u : v[it].z;
                 x.w = (!in || m.tail) ? 0u : v[it].w;
                 *reinterpret_cast<uint4 *>(tile + m.loff + 4096 * it) = x;
+            }
+        }
+    }
+};
+
+// The same with 8-byte pieces (8 per lane: row r0 + 8 it, columns 4 pc .. 4 pc + 3, r0 = lane / 32,
+// pc = lane % 32), for the kernel whose registers do not hold the 16-byte loader: no piece straddles the
+// end of a head (Dh % 4 = 0), the chunk swizzle of rows r0 + 8 it alternates between two values.  With
+// per-piece index arithmetic instead of these lane constants a tile cost 5 times the instructions
+// (dQ kernel 129 -> 125 us).
+struct TileMap8 {
+    unsigned goff0, loff0, loff1;
+    int r0, gcol;
+    int64_t ld;
+    bool colok;
+    __device__ __forceinline__ TileMap8(int64_t ld_, int Dh)
+    {
+        const int t = threadIdx.x & (kNT - 1), pc = t & 31;
+        r0 = t >> 5;
+        ld = ld_;
+        colok = pc * 4 < Dh;
+        gcol = min(pc * 4, Dh - 4);
+        goff0 = (unsigned)(r0 * ld_ + gcol);
+        loff0 = (unsigned)(toff(r0, pc >> 1) + ((pc & 1) << 3));
+        loff1 = (unsigned)(toff(r0 + 8, pc >> 1) + ((pc & 1) << 3)) - 8 * kRowB;
+    }
+};
+struct TileLoader8 {
+    static constexpr int NP = kTileRows * 32 / kNT;      // 8-byte pieces per lane
+    uint2 v[NP];
+    int rows;
+    __device__ __forceinline__ void load(const TileMap8 &m, gptr_t src, int rows_left)
+    {
+        rows = __builtin_amdgcn_readfirstlane(min(rows_left, kTileRows));
+        if (rows == kTileRows) {
+#pragma unroll
+            for (int it = 0; it < NP; it++) v[it] = gload8(src + (int64_t)(8 * it) * m.ld + m.goff0);
+        } else {
+#pragma unroll
+            for (int it = 0; it < NP; it++) v[it] = gload8(src + (int64_t)min(m.r0 + 8 * it, rows - 1) * m.ld + m.gcol);
+        }
+    }
+    __device__ __forceinline__ void store(const TileMap8 &m, unsigned char *tile) const
+    {
+        if (!m.colok) return;
+        if (rows == kTileRows) {
+#pragma unroll
+            for (int it = 0; it < NP; it++)
+                *reinterpret_cast<uint2 *>(tile + ((it & 1) ? m.loff1 : m.loff0) + 8 * kRowB * it) = v[it];
+        } else {
+#pragma unroll
+            for (int it = 0; it < NP; it++) {
+                const bool in = m.r0 + 8 * it < rows;
+                *reinterpret_cast<uint2 *>(tile + ((it & 1) ? m.loff1 : m.loff0) + 8 * kRowB * it) =
+                    make_uint2(in ? v[it].x : 0u, in ? v[it].y : 0u);
             }
         }
     }
@@ -642,6 +661,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    zero_lds(smem, 2 * kGroupLds);                 // the pad columns of the tile buffers: zero from here on
     const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8), tig = threadIdx.x & (kNT - 1);
     unsigned char *Ks = smem + g * kGroupLds, *Vs = Ks + 2 * kTileB;
     float *xs = reinterpret_cast<float *>(smem + kXsOff);
@@ -670,24 +690,25 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 
         const int kend = min(i0 + kBM, S);
         const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
-        TileLoader tk, tv;
+        const TileMap8 tm(ld, Dh);
+        TileLoader8 tk, tv;
         float16_t dacc[DT];
         auto run_pass = [&](auto pass_c) __attribute__((always_inline)) {
             constexpr int PASS = decltype(pass_c)::value;
             float part = 0.f;
             if (g < njt) {
-                tk.load(K + (int64_t)g * kTileRows * ld, ld, S - g * kTileRows, Dh);
-                tv.load(V + (int64_t)g * kTileRows * ld, ld, S - g * kTileRows, Dh);
-                tk.store(Ks);
-                tv.store(Vs);
+                tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+                tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+                tk.store(tm, Ks);
+                tv.store(tm, Vs);
             }
             __syncthreads();
             for (int it = 0; it < niter; it++) {
                 const int jt = 2 * it + g, cur = it & 1;
                 const bool nxt = jt + 2 < njt;
                 if (nxt) {
-                    tk.load(K + (int64_t)(jt + 2) * kTileRows * ld, ld, S - (jt + 2) * kTileRows, Dh);
-                    tv.load(V + (int64_t)(jt + 2) * kTileRows * ld, ld, S - (jt + 2) * kTileRows, Dh);
+                    tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
+                    tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
                 }
                 if (jt < njt) {
 #pragma unroll
@@ -742,8 +763,8 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
                     }
                 }
                 if (nxt) {
-                    tk.store(Ks + (cur ^ 1) * kTileB);
-                    tv.store(Vs + (cur ^ 1) * kTileB);
+                    tk.store(tm, Ks + (cur ^ 1) * kTileB);
+                    tv.store(tm, Vs + (cur ^ 1) * kTileB);
                 }
                 __syncthreads();
             }
