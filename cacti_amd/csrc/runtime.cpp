@@ -189,7 +189,7 @@ int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
     own_stream_ = true;
     // spill copies overlap compute only from page-locked memory (a copy from pageable memory is staged
     // synchronously by the runtime); default priority, like the compute stream
-    async_spill_ = host_pagelocked != 0;
+    async_spill_ = host_pagelocked_ != 0;
     if (async_spill_) {
         CACTI_HIP(hipStreamCreateWithFlags(&down_stream_, hipStreamNonBlocking));
         CACTI_HIP(hipStreamCreateWithFlags(&up_stream_, hipStreamNonBlocking));
