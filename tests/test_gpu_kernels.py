@@ -291,6 +291,10 @@ DIRECT_SHAPES = [
     (1, 0, 2056, 2304, 64),      # 256 x 256 tiles
     (1, 0, 3200, 3200, 64),      # 256 x 192 tiles
     (0, 1, 1024, 8640, 64),      # 64 full-round column tiles + 448 columns on 64 x 64 tiles
+    # the same with 5 .. 13 k tiles: the small tiles load five k tiles ahead (shorter than the
+    # pipeline, exactly as long, every length of the peeled tail)
+    (0, 1, 1024, 8640, 320), (0, 0, 1024, 8640, 384), (0, 1, 1024, 8640, 448), (0, 0, 1024, 8640, 512),
+    (0, 1, 1024, 8640, 576), (0, 0, 1024, 8640, 640), (0, 1, 1024, 8640, 704), (0, 0, 1024, 8640, 832),
     (0, 1, 2048, 24584, 64),     # forward product with at least 768 tiles of 256 x 256
 ]
 
