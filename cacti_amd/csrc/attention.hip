@@ -279,8 +279,11 @@ __device__ __forceinline__ void load_frags(half8_t (&f)[KS], gptr_t X, int64_t l
     }
 }
 
-// acc = sum over d of X[row_base + .][d] Y[.][d]: X from the LDS tile (16-byte reads), Y = fixed fragments
-template <int KS>
+// acc = sum over d of X[row_base + .][d] Y[.][d]: X from the LDS tile (16-byte reads), Y = fixed fragments.
+// PRIO: the wave runs its chain of dependent MFMAs at raised priority, so that the other wave of the SIMD
+// fills the gaps of the chain with its arithmetic instead of delaying it (forward and dQ kernel -2 %; the
+// dK / dV kernel has a SIMD to itself and only pays for the two extra instructions)
+template <int KS, bool PRIO = true>
 __device__ __forceinline__ float16_t prod_direct(const unsigned char *tile, int row_base, const half8_t (&yf)[KS],
                                                  int l32, int lh)
 {
@@ -293,8 +296,10 @@ __device__ __forceinline__ float16_t prod_direct(const unsigned char *tile, int 
     half8_t x[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) x[ks] = *reinterpret_cast<const half8_t *>(rp + (((2 * ks + lh) ^ g) << 4));
+    if (PRIO) __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks], yf[ks], acc, 0, 0, 0);
+    if (PRIO) __builtin_amdgcn_s_setprio(0);
     // all fragment reads in flight before the first product (the scheduler would otherwise pair each
     // read with its use and expose the LDS latency once per k step)
     __builtin_amdgcn_sched_group_barrier(0x100, KS, 0);
@@ -869,8 +874,8 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
             for (int qb = 0; qb < 2; qb++) {
                 const int qb0 = iq * kTileRows + 32 * qb;
                 if (qb0 + 31 < c0 || qb0 >= S) continue;     // every query of the block is before every key of the wave
-                const float16_t sacc = prod_direct<KS>(Qs + cur * kTileB, 32 * qb, kf, l32, lh);
-                const float16_t pacc = prod_direct<KS>(Gs + cur * kTileB, 32 * qb, vf, l32, lh);
+                const float16_t sacc = prod_direct<KS, false>(Qs + cur * kTileB, 32 * qb, kf, l32, lh);
+                const float16_t pacc = prod_direct<KS, false>(Gs + cur * kTileB, 32 * qb, vf, l32, lh);
                 const bool full = qb0 >= c0 + 31 && qb0 + 32 <= S;
                 float pe[16], de[16];
                 half_t dph[16];
