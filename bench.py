@@ -203,14 +203,32 @@ def cpu_baseline(cfg):
                       % (CPU_SAMPLE_LAYERS, cfg["L"], layer, times[0], cfg["S"], cfg["L"])}
 
 
+# gradients read back after the capped and the uncapped leg and compared bit for bit (the layers are
+# clipped to the model's depth): the first and last layers, one of every kind of tensor
+CAPPED_PROBES = ["embed", "l0.q", "l0.pre_norm", "l3.k", "l7.down", "l12.up", "l18.gate", "l25.v", "l25.o",
+                 "l25.post_norm", "head_norm", "lm_head"]
+
+
+def probe_grads(model, cfg):
+    """{name: f16 gradient} of CAPPED_PROBES for this model."""
+    idx = {name: i for i, (name, _) in enumerate(model.params)}
+    out = {}
+    for n in CAPPED_PROBES:
+        if n.startswith("l") and "." in n and n[1].isdigit():
+            layer, rest = n.split(".", 1)
+            n = "l%d.%s" % (min(int(layer[1:]), cfg["L"] - 1), rest)
+        out[n] = model.grad(idx[n])
+    return out
+
+
 CAPPED_POOL_BYTES = 16 << 30       # the reference's 16 GiB card (examples/open_llama_3b_train.rs runs on one)
 CAPPED_WARMUP = 6                  # the spill plan of a cycle follows the cycles before it: a few to settle
 
 
 def run_capped(cfg, args):
     """The same step on a device pool capped at 16 GiB, so that it has to spill to page-locked host
-    memory: K timed steps after its own warmup.  Returns the record and the loss, which the caller
-    compares bit for bit with the uncapped run's.  (It runs before the uncapped leg: a 16 GiB pool
+    memory: K timed steps after its own warmup.  Returns the record, the loss and the probe gradients,
+    which the caller compares bit for bit with the uncapped run's.  (It runs before the uncapped leg: a 16 GiB pool
     allocated after the uncapped leg's pool of 90 % of the device has been freed measured 10 % slower.)"""
     import torch
     from cacti_amd.runtime import Ctx, Llama
@@ -231,6 +249,7 @@ def run_capped(cfg, args):
     dt = time.perf_counter() - t0
     st1 = ctx.stats()
     loss = model.step(tok, lm_tok, scale)
+    grads = probe_grads(model, cfg)
     model.close()
     ctx.close()
     per = lambda k: (st1[k] - st0[k]) / args.steps
@@ -239,7 +258,7 @@ def run_capped(cfg, args):
     return {"pool_cap_bytes": CAPPED_POOL_BYTES, "ms_per_step": dt / args.steps * 1e3,
             "tokens_per_s": cfg["S"] * args.steps / dt, "evictions": per("n_evict"),
             "d2h_bytes": per("bytes_d2h"), "h2d_bytes": per("bytes_h2d"), "pool_peak_bytes": st1["pool_peak"],
-            "steps": args.steps, "warmup": max(args.warmup, CAPPED_WARMUP)}, loss
+            "steps": args.steps, "warmup": max(args.warmup, CAPPED_WARMUP)}, loss, grads
 
 
 def run_step(args):
@@ -250,7 +269,7 @@ def run_step(args):
         cfg["L"] = args.layers
     pool = int(args.pool_gb * (1 << 30)) if args.pool_gb else 0
     # the same configuration on the reference's 16 GiB card: a second run, on a capped pool
-    capped, capped_loss = (None, None) if pool or args.no_capped else run_capped(cfg, args)
+    capped, capped_loss, capped_grads = (None, None, None) if pool or args.no_capped else run_capped(cfg, args)
     ctx = Ctx(0, pool, True)
     model = Llama(ctx, **cfg)
     t0 = time.time()
@@ -319,6 +338,7 @@ def run_step(args):
     ctx.set_timing_filter("")
     loss = model.step(tok, lm_tok, scale)
     assert np.all(np.isfinite(loss)), "non-finite loss"
+    grads = probe_grads(model, cfg) if capped is not None else None
     ms = dt / args.steps * 1e3
     tokens_s = cfg["S"] * args.steps / dt
 
@@ -360,6 +380,11 @@ def run_step(args):
         assert np.array_equal(np.asarray(loss).view(np.uint32), np.asarray(capped_loss).view(np.uint32)), \
             "the capped run's loss differs from the uncapped run's"
         capped["loss_bit_identical"] = True
+        for n, g in grads.items():
+            assert np.array_equal(g.view(np.uint16), capped_grads[n].view(np.uint16)), \
+                "gradient %s of the capped run differs from the uncapped run's" % n
+        capped["grads_bit_identical"] = True
+        capped["grads_compared"] = sorted(grads)
         out["config"]["capped"] = capped
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(LLAMA_3B)

@@ -40,6 +40,7 @@
 #include "common.h"
 #include "softmax_math.h"
 
+#include <atomic>
 #include <type_traits>
 
 using namespace cacti;
@@ -954,15 +955,16 @@ int set_smem(K kern, size_t bytes)
 // differ by 3e-5 .. 4e-5 relative L2 in O, dQ, dK, dV, and O, dQ, dK, dV of the fast form agree with
 // the CPU restatement of the reference to 4.9e-5 .. 7.1e-5.
 constexpr bool kFastMath = true;
+std::atomic<int> g_exact{0};             // cacti_hip_attention_set_exact: launch the exactly rounded forms
 
 template <int KS, int DT, bool FAST = kFastMath>
 int launch_fwd(const AttnArgs &p, hipStream_t st)
 {
-    static bool ready = false;
-    if (!ready) {
+    static DeviceOnce ready;
+    if (!ready.fresh()) {
         int rc = set_smem(attn_fwd_kernel<KS, DT, FAST>, kQmSmem);
         if (rc) return rc;
-        ready = true;
+        ready.mark();
     }
     const int nqt = (p.S + kBM - 1) / kBM;
     hipLaunchKernelGGL((attn_fwd_kernel<KS, DT, FAST>), dim3((unsigned)(nqt * p.H)), dim3(kNT2), kQmSmem, st, p);
@@ -972,12 +974,12 @@ int launch_fwd(const AttnArgs &p, hipStream_t st)
 template <int KS, int DT, bool FAST = kFastMath>
 int launch_bwd(const AttnArgs &p, hipStream_t st)
 {
-    static bool ready = false;
-    if (!ready) {
+    static DeviceOnce ready;
+    if (!ready.fresh()) {
         int rc = set_smem(attn_bwd_dq_kernel<KS, DT, FAST>, kQmSmem);
         if (rc) return rc;
         if ((rc = set_smem(attn_bwd_dkv_kernel<KS, DT, FAST>, kDkvSmem))) return rc;
-        ready = true;
+        ready.mark();
     }
     const int nqt = (p.S + kBM - 1) / kBM;
     hipLaunchKernelGGL((attn_bwd_dq_kernel<KS, DT, FAST>), dim3((unsigned)(nqt * p.H)), dim3(kNT2), kQmSmem, st, p);
@@ -996,10 +998,19 @@ int check_shape(const char *who, int64_t S, int64_t H, int64_t Dh, int64_t ld)
                   who, (long long)ld);
     CACTI_REQUIRE(S <= (1 << 24) && S * H < ((int64_t)1 << 31) / 2, CACTI_E_NOTIMPL, "%s: S = %lld is too large", who,
                   (long long)S);
+    // the tile loaders keep (row within a tile) * ld + column as a 32-bit offset
+    CACTI_REQUIRE(ld <= ((int64_t)1 << 26), CACTI_E_NOTIMPL, "%s: row stride %lld is beyond the 2^26 elements the "
+                  "tile loaders address", who, (long long)ld);
     return 0;
 }
 
 }  // namespace
+
+CACTI_API int cacti_hip_attention_set_exact(int on)
+{
+    g_exact.store(on ? 1 : 0, std::memory_order_relaxed);
+    return 0;
+}
 
 CACTI_API size_t cacti_hip_attention_stats_bytes(int64_t S, int64_t H)
 {
@@ -1026,6 +1037,11 @@ CACTI_API int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float al
     p.m = (float *)stats;
     p.l = p.m + S * H;
     hipStream_t st = (hipStream_t)stream;
+    if (g_exact.load(std::memory_order_relaxed)) {
+        if (Dh <= 64) return launch_fwd<4, 2, false>(p, st);
+        if (Dh <= 112) return launch_fwd<7, 4, false>(p, st);
+        return launch_fwd<8, 4, false>(p, st);
+    }
     if (Dh <= 64) return launch_fwd<4, 2>(p, st);
     if (Dh <= 112) return launch_fwd<7, 4>(p, st);
     return launch_fwd<8, 4>(p, st);
@@ -1057,6 +1073,11 @@ CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float al
     p.y = (float *)workspace;
     p.sig = p.y + S * H;
     hipStream_t st = (hipStream_t)stream;
+    if (g_exact.load(std::memory_order_relaxed)) {
+        if (Dh <= 64) return launch_bwd<4, 2, false>(p, st);
+        if (Dh <= 112) return launch_bwd<7, 4, false>(p, st);
+        return launch_bwd<8, 4, false>(p, st);
+    }
     if (Dh <= 64) return launch_bwd<4, 2>(p, st);
     if (Dh <= 112) return launch_bwd<7, 4>(p, st);
     return launch_bwd<8, 4>(p, st);

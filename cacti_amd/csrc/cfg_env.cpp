@@ -167,7 +167,12 @@ CACTI_API int cacti_hip_primary_ctx_set_flags(int dev, unsigned flags)
 }
 CACTI_API int cacti_hip_primary_ctx_reset(int dev)
 {
+    using namespace cacti;
+    CACTI_REQUIRE(live_contexts(dev) == 0, CACTI_E_STATE,
+                  "primary_ctx_reset: %d device context(s) of this library are alive on device %d; destroy "
+                  "them first (a reset frees their pool, streams and events)", live_contexts(dev), dev);
     CACTI_HIP(hipDevicePrimaryCtxReset(dev));
+    module_epoch_advance();        // function attributes and symbol addresses are looked up again
     return 0;
 }
 

@@ -29,6 +29,31 @@ int hip_status(hipError_t e, const char *what);
         }                                       \
     } while (0)
 
+// State a launcher establishes once per device and keeps (a kernel's dynamic-LDS attribute, the device
+// address of a file-scope array) belongs to the device's loaded modules.  cacti_hip_primary_ctx_reset
+// unloads them, so it advances an epoch, and every such cache is tagged with (device, epoch) and set up
+// again when either differs.
+unsigned module_epoch();
+void module_epoch_advance();
+// device contexts (cacti_ctx) alive on a device: a primary-context reset under one would free its pool,
+// streams and events behind its back, so the reset entry point refuses while any exists
+int live_contexts(int dev);
+void live_contexts_add(int dev, int n);
+struct DeviceOnce {
+    int dev = -1;
+    unsigned epoch = 0;
+    bool fresh() const
+    {
+        int d = -2;
+        return hipGetDevice(&d) == hipSuccess && d == dev && epoch == module_epoch();
+    }
+    void mark()
+    {
+        if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+        epoch = module_epoch();
+    }
+};
+
 inline int launch_status(const char *what) { return hip_status(hipGetLastError(), what); }
 
 inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }

@@ -1,6 +1,7 @@
 // Device / memory / stream / event entry points of the C ABI: thin, checked
 // wrappers over the HIP runtime (the counterpart of cacti_gpu_cu_ffi/src/lib.rs:98-565).
 #include <stdarg.h>
+#include <atomic>
 #include <string.h>
 
 #include "common.h"
@@ -15,6 +16,16 @@ void set_error(const char *fmt, ...)
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+static std::atomic<unsigned> g_module_epoch{1};
+unsigned module_epoch() { return g_module_epoch.load(std::memory_order_relaxed); }
+void module_epoch_advance() { g_module_epoch.fetch_add(1, std::memory_order_relaxed); }
+static std::atomic<int> g_live_contexts[64];
+int live_contexts(int dev) { return dev >= 0 && dev < 64 ? g_live_contexts[dev].load() : 0; }
+void live_contexts_add(int dev, int n)
+{
+    if (dev >= 0 && dev < 64) g_live_contexts[dev].fetch_add(n);
 }
 
 int hip_status(hipError_t e, const char *what)

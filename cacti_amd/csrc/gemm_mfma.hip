@@ -882,11 +882,11 @@ int launch_cfg(GemmArgs p, int64_t nblk, hipStream_t st)
     p.tiles_n = (int)((p.N + (p.win ? 4 : 0) + BN - 1) / BN);
     const size_t smem = (size_t)NBUF * (BM + BN) * BK * sizeof(half_t);
     auto kern = gemm_mfma_kernel<TA, TB, BM, BN, WM, WN, AL, KTAIL, STAGES, NBUF, DMA>;
-    static bool attr_set = false;                 // one flag per instantiation
-    if (!attr_set) {
+    static DeviceOnce attr_set;                   // one per instantiation
+    if (!attr_set.fresh()) {
         CACTI_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                       (int)smem));
-        attr_set = true;
+        attr_set.mark();
     }
     if (p.gm <= 0) {
         // tile rows per group of the walk.  An XCD works on a band of tiles / 8 consecutive tiles,

@@ -96,6 +96,15 @@ CACTI_API int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out)
     return 0;
 }
 
+CACTI_API int cacti_ctx_usage_report(cacti_ctx *ctx, char *buf, size_t cap)
+{
+    CACTI_REQUIRE(ctx && buf && cap > 0, CACTI_E_INVALID, "ctx_usage_report: null pointer");
+    const std::string s = ctx->c.usage_report();
+    CACTI_REQUIRE(s.size() < cap, CACTI_E_INVALID, "ctx_usage_report: the report needs %zu bytes", s.size() + 1);
+    memcpy(buf, s.c_str(), s.size() + 1);
+    return 0;
+}
+
 CACTI_API int cacti_ctx_sync(cacti_ctx *ctx) { return ctx->c.check_status(); }
 CACTI_API void *cacti_ctx_stream(cacti_ctx *ctx) { return (void *)ctx->c.stream(); }
 

@@ -254,11 +254,11 @@ void launch_bwd(int64_t N, int D, const half_t *x, const half_t *w, float eps, c
     const int wide_lds = wide <= 144 * 1024;
     const size_t smem = wide_lds ? wide : (size_t)D * 4;
     auto kern = rms_norm_bwd_kernel<CH>;
-    static bool attr_set = false;                 // one flag per instantiation
-    if (!attr_set) {
+    static DeviceOnce attr_set;                   // one per instantiation
+    if (!attr_set.fresh()) {
         (void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   144 * 1024);
-        attr_set = true;
+        attr_set.mark();
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)((N + kWaves - 1) / kWaves)), dim3(kThreads), smem, st,
                        N, D, x, w, eps, dy, dx, dx_acc, part, wide_lds);
@@ -349,6 +349,7 @@ constexpr size_t kStaticScratchBytes = 8u << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
 void *g_scratch_ptr[kMaxDevices];          // per device, nullptr until first use on that device
+unsigned g_scratch_epoch[kMaxDevices];     // the module epoch each address was taken in
 }  // namespace
 
 CACTI_API size_t cacti_hip_rms_norm_bwd_static_max_bytes(void) { return kStaticScratchBytes; }
@@ -367,11 +368,12 @@ CACTI_API int cacti_hip_rms_norm_bwd_static(int64_t N, int64_t D, const void *x,
     CACTI_REQUIRE(dev >= 0 && dev < kMaxDevices, CACTI_E_NOTIMPL,
                   "rms_norm_bwd_static: device %d is beyond the %d this entry point keeps a buffer for",
                   dev, kMaxDevices);
-    if (!g_scratch_ptr[dev]) {
+    if (!g_scratch_ptr[dev] || g_scratch_epoch[dev] != module_epoch()) {   // first use, or the modules were reloaded
         void *p = nullptr;
         CACTI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
         CACTI_REQUIRE(p != nullptr, CACTI_E_STATE, "rms_norm_bwd_static: no device address for the scratch array");
         g_scratch_ptr[dev] = p;
+        g_scratch_epoch[dev] = module_epoch();
     }
     return cacti_hip_rms_norm_bwd(N, D, x, w, eps, dy, dx, dx_acc, dw, dw_acc, g_scratch_ptr[dev],
                                   kStaticScratchBytes, stream);

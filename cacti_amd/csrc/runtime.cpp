@@ -152,6 +152,7 @@ Ctx::~Ctx()
     }
     if (base_) hipFree(base_);
     if (own_stream_ && stream_) hipStreamDestroy(stream_);
+    if (counted_) live_contexts_add(dev_, -1);
 }
 
 int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
@@ -181,6 +182,8 @@ int Ctx::init(int dev, size_t pool_bytes, int host_pagelocked)
                   "(the pool_bytes argument, or CACTI_VMEM_SOFT_LIMIT when that is 0)",
                   pool_bytes, avail, total);
     CACTI_HIP(hipMalloc((void **)&base_, pool_bytes));
+    live_contexts_add(dev_, 1);
+    counted_ = true;
     CACTI_REQUIRE(((uintptr_t)base_ % kAllocAlign) == 0, CACTI_E_STATE, "ctx: misaligned reserve");
     pool_.reset(pool_bytes);
     status_off_ = pool_.alloc(kAllocAlign);
@@ -876,9 +879,17 @@ int Ctx::pool_alloc(size_t bytes, size_t *off, bool high)
         int rc = try_soft_oom(bytes);
         if (rc == 0) o = pool_.alloc(bytes, high);
         if (o == kNoOffset) {
-            set_error("device pool exhausted: request %zu bytes, cap %zu, used %zu, front %zu, "
-                      "largest free %zu (every other cell is pinned by the running thunk)",
-                      bytes, pool_.cap(), pool_.used(), pool_.front(), pool_.largest_free());
+            // the reference dumps the pool's usage before it panics (src/pctx/nvgpu.rs:2424-2440); here the
+            // full table goes to stderr and the status message carries the pool's line of it
+            const std::string rep = usage_report();
+            fprintf(stderr, "cacti: device pool exhausted, request of %zu bytes does not fit after eviction\n%s", bytes,
+                    rep.c_str());
+            size_t pinned = 0;
+            for (const Cell &c : cells_)
+                if (c.alive && c.voff != kNoOffset && c.pin > 0) pinned += c.ty.bytes();
+            set_error("device pool exhausted: request %zu bytes, cap %zu, used %zu, front %zu, largest free %zu, "
+                      "pinned by the running thunk %zu, downloads in flight %zu (usage by class of cell on stderr)",
+                      bytes, pool_.cap(), pool_.used(), pool_.front(), pool_.largest_free(), pinned, pending_bytes_);
             return CACTI_E_OOM;
         }
     }
@@ -925,6 +936,10 @@ int Ctx::ensure_vmem(CellPtr ci, bool need_value)
 
 void Ctx::reset()
 {
+    // CACTI_VERBOSE: the usage dump at every reset, i.e. once per cycle, before the cycle's cells are
+    // collected (Ctx::reset, src/ctx.rs:150-167)
+    static const bool verbose = getenv("CACTI_VERBOSE") && !getenv("CACTI_SILENT");
+    if (verbose && pc_ > 0) fprintf(stderr, "cacti: usage at the end of a cycle\n%s", usage_report().c_str());
     for (size_t i = 1; i < cells_.size(); i++) {
         Cell &c = cells_[i];
         if (c.alive && !c.stable) {
@@ -1333,6 +1348,60 @@ int Ctx::resume_put(CellPtr c, const void *host, size_t bytes)
     if (rc) return rc;
     pc_++;
     return 0;
+}
+
+// One line per class of cell: bytes resident on the device (pinned ones apart) and bytes held only
+// by a host replica; then the pool's own figures.  The classes follow the cells' roles in the cycle:
+// parameters, gradients and optimiser state live across cycles and are what a capped pool spills;
+// everything else is an activation or an adjoint of the running cycle.
+std::string Ctx::usage_report() const
+{
+    struct Row { const char *what; size_t n = 0, dev = 0, pinned = 0, host_only = 0, largest = 0; };
+    Row rows[5];
+    rows[0].what = "parameters";
+    rows[1].what = "gradients";
+    rows[2].what = "optimiser state";
+    rows[3].what = "tables, inputs, caches";
+    rows[4].what = "cycle cells";
+    for (size_t i = 1; i < cells_.size(); i++) {
+        const Cell &c = cells_[i];
+        if (!c.alive) continue;
+        int k = 4;
+        if (c.stable) {
+            const std::string &n = c.name;
+            if (n.compare(0, 5, "grad:") == 0) k = 1;
+            else if (n.compare(0, 7, "master:") == 0 || n.compare(0, 9, "grad_avg:") == 0 || n.compare(0, 10, "grad2_avg:") == 0) k = 2;
+            else if (n == "cos" || n == "sin" || n.compare(0, 3, "in_") == 0 || n.find("cache") != std::string::npos ||
+                     n.compare(0, 6, "cached") == 0) k = 3;
+            else k = 0;
+        }
+        Row &r = rows[k];
+        const size_t b = c.ty.bytes();
+        r.n++;
+        if (c.voff != kNoOffset) {
+            r.dev += b;
+            if (c.pin > 0) r.pinned += b;
+            r.largest = std::max(r.largest, b);
+        } else if (c.hptr && c.h_valid) {
+            r.host_only += b;
+        }
+    }
+    char line[256];
+    std::string out;
+    snprintf(line, sizeof line, "pool: cap=%zu used=%zu peak=%zu front=%zu largest_free=%zu pending_downloads=%zu (%zu regions) "
+             "host=%zu\n", pool_.cap(), pool_.used(), pool_.peak(), pool_.front(), pool_.largest_free(), pending_bytes_,
+             pending_.size(), (size_t)host_bytes_);
+    out += line;
+    for (const Row &r : rows) {
+        snprintf(line, sizeof line, "  %-24s cells=%zu device=%zu (pinned %zu, largest %zu) host_only=%zu\n", r.what, r.n, r.dev,
+                 r.pinned, r.largest, r.host_only);
+        out += line;
+    }
+    snprintf(line, sizeof line, "  evictions=%llu uploads=%llu d2h=%llu h2d=%llu soft_oom=%llu entry=%zu/%zu\n",
+             (unsigned long long)n_evict_, (unsigned long long)n_upload_, (unsigned long long)bytes_d2h_,
+             (unsigned long long)bytes_h2d_, (unsigned long long)n_soft_oom_, pc_, log_.size());
+    out += line;
+    return out;
 }
 
 void Ctx::stats(Stats *s) const

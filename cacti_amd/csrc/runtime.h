@@ -214,6 +214,9 @@ class Ctx {
     void *status_ptr() { return base_ + status_off_; }
     int check_status();
     void stats(Stats *s) const;
+    // the pool's usage by class of cell, as text (NvGpuPCtx::_dump_usage / _dump_sizes / _dump_free,
+    // src/pctx/nvgpu.rs:690-742): what an exhausted pool prints, and the per-cycle report
+    std::string usage_report() const;
     const std::vector<Entry> &log() const { return log_; }
     const ThunkSpec &thunk(int i) const { return *thunks_[i]; }
     const char *entry_name(size_t i) const;
@@ -268,6 +271,7 @@ class Ctx {
     std::unordered_map<CellPtr, std::vector<uint32_t>> uses_;    // compiled log: entries that touch a cell
     std::multimap<size_t, HostBuf> host_pool_;                   // page-locked buffers of dead cells, by size
     int dev_ = 0;
+    bool counted_ = false;                      // this context is in the device's live-context count
     hipStream_t stream_ = nullptr;
     bool own_stream_ = false;
     char *base_ = nullptr;

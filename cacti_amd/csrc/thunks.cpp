@@ -338,6 +338,7 @@ struct Rope2BwdSpec : ThunkSpec {
     explicit Rope2BwdSpec(int64_t h) : H(h) {}
     const char *name() const override { return "rope2_bwd"; }
     int arity() const override { return 4; }
+    int nout() const override { return 2; }
     int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
     {
         TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] % H == 0 && a[1] == a[0],
@@ -358,6 +359,7 @@ struct Rope2Spec : ThunkSpec {
     explicit Rope2Spec(int64_t h) : H(h) {}
     const char *name() const override { return "rope2"; }
     int arity() const override { return 4; }
+    int nout() const override { return 2; }
     int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
     {
         TY_REQUIRE(a[0].dtype == F16 && a[0].shape.size() == 2 && a[0].shape[1] % H == 0 && a[1] == a[0] &&

@@ -74,6 +74,7 @@ SIGNATURES = {
     "cacti_hip_silu_gate_bwd": (ci, [i64, vp, vp, vp, vp, ci, vp, ci, vp]),
     "cacti_hip_causal_softmax_fwd": (ci, [i64, i64, vp, vp, vp]),
     "cacti_hip_causal_softmax_bwd": (ci, [i64, i64, vp, vp, vp, vp]),
+    "cacti_hip_attention_set_exact": (ci, [ci]),
     "cacti_hip_attention_stats_bytes": (sz, [i64, i64]),
     "cacti_hip_attention_fwd": (ci, [i64, i64, i64, f32, vp, vp, vp, i64, vp, vp, vp]),
     "cacti_hip_attention_bwd_workspace": (sz, [i64, i64]),
@@ -111,6 +112,7 @@ SIGNATURES = {
     "cacti_ctx_create": (ci, [pvp, ci, sz, ci]),
     "cacti_ctx_destroy": (ci, [vp]),
     "cacti_ctx_stats": (ci, [vp, vp]),
+    "cacti_ctx_usage_report": (ci, [vp, C.c_char_p, sz]),
     "cacti_ctx_sync": (ci, [vp]),
     "cacti_ctx_stream": (vp, [vp]),
     "cacti_ctx_set_timing": (ci, [vp, ci]),

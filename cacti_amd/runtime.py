@@ -59,6 +59,11 @@ class Ctx:
         ffi.call("cacti_ctx_stats", self._c, C.byref(s))
         return {n: getattr(s, n) for n, _ in ffi.Stats._fields_}
 
+    def usage_report(self):
+        buf = C.create_string_buffer(4096)
+        ffi.call("cacti_ctx_usage_report", self._c, buf, C.c_size_t(len(buf)))
+        return buf.value.decode()
+
     def sync(self):
         ffi.call("cacti_ctx_sync", self._c)
 

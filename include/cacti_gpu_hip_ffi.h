@@ -69,6 +69,11 @@ int cacti_hip_memcpy_d2h_async(void *dst, const void *src, size_t bytes, void *s
 int cacti_hip_memset_async(void *dst, int byte, size_t bytes, void *stream);
 int cacti_hip_primary_ctx_retain(int dev, void **pctx);         /* lib.rs:177 (hipDevicePrimaryCtxRetain) */
 int cacti_hip_primary_ctx_release(int dev);                     /* lib.rs:159       */
+/* set_flags on a primary context that is already active returns the runtime's error as its positive
+ * hipError_t (a status, never an abort).  reset destroys everything on the device, so it is refused with CACTI_E_STATE
+ * while a cacti_ctx of this library exists on `dev`; after a reset the library looks its per-device
+ * state (kernel attributes, the address of its built-in scratch array) up again on the next launch.
+ * Memory, streams and events the caller created on the device are the caller's to forget. */
 int cacti_hip_primary_ctx_set_flags(int dev, unsigned flags);   /* lib.rs:186       */
 int cacti_hip_primary_ctx_reset(int dev);                       /* lib.rs:169       */
 void *cacti_hip_stream_null(void);                              /* lib.rs:512: the null stream's handle (NULL) */
@@ -250,7 +255,17 @@ int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const vo
  * memory, written by the forward call (row maximum and sum per head and row, f32) and read by the
  * adjoint; workspace: cacti_hip_attention_bwd_workspace(S, H) bytes, contents undefined on return.
  * *_acc: 0 first write, 1 the product is added to the tensor in fp32 before the one rounding (the
- * GEMMs' beta = 1). */
+ * GEMMs' beta = 1).
+ * Arithmetic between the rounding points.  By default a probability is formed as
+ * 2^(s log2 e - c) with one fp32 offset c = m log2 e + log2 l per row (row maximum m, row sum l): the
+ * rounding of c is an error common to the row, at most half an ulp of c times ln 2 relative -- 3e-6 for
+ * |m| < 90, 2e-5 at |m| = 500 -- and in a row whose probability sits on one key it breaks the exact
+ * cancellation dP - sigma = 0 the reference has there.  Results agree with the reference's chain to 1e-4
+ * relative L2 for row maxima up to some hundreds; beyond that (|m| in the thousands: measured 7e-3 on dQ
+ * at |m| = 1500 .. 2600) call cacti_hip_attention_set_exact(1): every later launch of this process uses
+ * the exactly rounded forms of the separate softmax kernels (range-reduced exp of s - m, correctly
+ * rounded quotient by l) at 5 % / 12 % more time forward / adjoint; 0 restores the default. */
+int cacti_hip_attention_set_exact(int on);
 size_t cacti_hip_attention_stats_bytes(int64_t S, int64_t H);
 int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float alpha, const void *q, const void *k,
                             const void *v, int64_t ld, void *o, void *stats, void *stream);

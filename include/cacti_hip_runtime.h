@@ -70,6 +70,15 @@ int cacti_vmem_soft_limit(const char *text, size_t avail, size_t total, size_t *
 int cacti_env_host_pagelocked(void);
 int cacti_ctx_destroy(cacti_ctx *ctx);
 int cacti_ctx_stats(cacti_ctx *ctx, cacti_stats *out);
+/* The pool's usage as text (NvGpuPCtx::_dump_usage / _dump_sizes / _dump_free,
+ * src/pctx/nvgpu.rs:690-742): one line for the pool (cap, used, peak, front, largest free region,
+ * downloads in flight, host bytes), one per class of cell (parameters, gradients, optimiser state,
+ * tables and inputs, the running cycle's cells: count, bytes on the device, of those pinned, largest,
+ * bytes held by a host replica only) and the spill counters.  The same text goes to stderr when the pool
+ * is exhausted with everything else pinned (the reference dumps and panics, :2424-2440; here the call
+ * returns CACTI_E_OOM) and, with CACTI_VERBOSE set, at every reset, i.e. once per cycle
+ * (src/ctx.rs:150-167).  The buffer must hold the text (4 KiB is enough), else CACTI_E_INVALID. */
+int cacti_ctx_usage_report(cacti_ctx *ctx, char *buf, size_t cap);
 int cacti_ctx_sync(cacti_ctx *ctx);      /* stream sync + token-range status check */
 void *cacti_ctx_stream(cacti_ctx *ctx);                 /* the hipStream_t all work runs on */
 /* per-thunk device times (CACTI_DEBUG_TIMING, src/ctx.rs:114-133).  mode 1 syncs after

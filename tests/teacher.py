@@ -27,8 +27,10 @@ def _c(a):
     return np.ascontiguousarray(a)
 
 
-def trace_step(cfg, flat, tok, lm_tok, scale):
-    """Returns (calls, loss, grads dict).  Every array in a Call is a private copy."""
+def trace_step(cfg, flat, tok, lm_tok, scale, sink=None):
+    """Returns (calls, loss, grads dict).  Every array in a Call is a private copy.  With `sink`, each Call is
+    handed to sink(call) as soon as it is recorded instead of being kept (large shapes: the trace of one
+    3B-shaped layer is several GB) and the returned list is empty."""
     S, D, H, Dh, F, V, L = cfg.S, cfg.D, cfg.H, cfg.Dh, cfg.F, cfg.V, cfg.L
     eps = float(cfg.eps)
     alpha = float(np.float32(1.0) / np.sqrt(np.float32(Dh)))
@@ -37,8 +39,12 @@ def trace_step(cfg, flat, tok, lm_tok, scale):
     calls = []
 
     def rec(kind, where, ins, outs):
-        calls.append(Call(kind, where, {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in ins.items()},
-                          {k: v.copy() for k, v in outs.items()}))
+        c = Call(kind, where, {k: (v.copy() if isinstance(v, np.ndarray) else v) for k, v in ins.items()},
+                 {k: v.copy() for k, v in outs.items()})
+        if sink is None:
+            calls.append(c)
+        else:
+            sink(c)
 
     def mm(where, ta, tb, A, B, alpha_=1.0, beta=0.0, C_init=None):
         out = o.matmul(ta, tb, A, B, alpha_, beta, C_init)

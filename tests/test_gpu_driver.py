@@ -65,6 +65,18 @@ def test_primary_context_retain_release():
     ffi.call("cacti_hip_primary_ctx_release", 0)
     with pytest.raises(ffi.CactiError):
         ffi.call("cacti_hip_primary_ctx_retain", 4096, C.byref(a))   # no such device: a status, not an abort
+    # flags of a primary context that is already active (torch made it so): a status, not an abort
+    try:
+        ffi.call("cacti_hip_primary_ctx_set_flags", 0, 0)
+    except ffi.CactiError as e:
+        assert e.code > 0                                       # the runtime's hipError_t
+    # a reset is refused while a device context of this library lives on the device (nothing is reset here)
+    from cacti_amd.runtime import Ctx
+    ctx = Ctx(0, 64 << 20, 0)
+    with pytest.raises(ffi.CactiError) as e:
+        ffi.call("cacti_hip_primary_ctx_reset", 0)
+    assert e.value.code == -5 and "alive" in str(e.value)
+    ctx.close()
     # a reported failure does not linger as the status of the next kernel launch
     import torch
     from cacti_amd import ops

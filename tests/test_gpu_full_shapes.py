@@ -166,3 +166,50 @@ def test_one_layer_cycle_full_shape(oracle, one_layer_case, attention):
         say("  %-12s rel_l2 %.2e max_rel %.2e%s" % (n, e2, em, "" if e2 <= 1e-3 and em <= 2e-2 else "   (outside 1e-3 / 2e-2)"))
     say("  pool peak %.2f GB" % (peak / 1e9))
     assert_inside_envelope(grads, want, k["env"], "one layer, full shape, " + attention)
+
+
+def test_every_thunk_of_one_layer_full_shape(oracle):
+    """Teacher-forced at the 3B shapes: the oracle's cycle of one decoder layer + head is traced thunk by
+    thunk (tests/teacher.py) and every recorded call is replayed on the device with the ORACLE's inputs and
+    held to the literal 1e-3 / 2e-2 — every projection and FFN product layout at M = 2048 (forward, dgrad,
+    accumulating dgrad, wgrad), the LM-head products, both norms with their accumulating adjoints, the SiLU
+    gate, RoPE, the attention block as separate thunks and as the fused kernels, loss and embedding."""
+    from cacti_amd import ops
+    from tests.llama_ref import make_inputs
+    from tests.teacher import trace_step
+    from tests.test_gpu_teacher import _replay
+    say("every thunk of one layer, full shape, on the oracle's inputs")
+    cfgd = dict(S=S, D=D, H=H, Dh=DH, F=F, V=V, L=1, eps=1e-6)
+    cfg, flat, tok, lm_tok, scale = make_inputs(cfgd, seed=7, norm_mean=1.0, grad_scale=1024.0)
+    worst, count = {}, [0]
+
+    def check(c):
+        got = _replay(ops, c)
+        if got is None:
+            return
+        for name, g in got.items():
+            want = c.outs[name]
+            tag = "%s@%s.%s" % (c.kind, c.where, name)
+            if want.dtype == np.uint16:                                  # arg max: first maximum, ties aside
+                lg = c.ins["logit"].astype(np.float32)
+                rows = np.arange(lg.shape[0])
+                assert np.array_equal(lg[rows, g], lg[rows, want]), tag
+                continue
+            if c.kind == "embed_fwd":                                    # gather: bit-exact
+                assert np.array_equal(g.view(np.uint16), want.view(np.uint16)), tag
+                continue
+            e2, em = assert_parity(g.reshape(want.shape), want, tag)
+            key = c.kind if c.kind != "matmul" else "matmul %s%s%s" % (
+                "T" if c.ins["ta"] else "N", "T" if c.ins["tb"] else "N", "+" if c.ins["beta"] else "")
+            worst[key] = max(worst.get(key, (0.0, 0.0)), (e2, em))
+            count[0] += 1
+        torch.cuda.empty_cache()
+
+    trace_step(cfg, flat, tok, lm_tok, scale, sink=check)
+    say("  %d thunk outputs inside 1e-3 / 2e-2; worst (rel_l2, max_rel) per kind:" % count[0])
+    for k, v in sorted(worst.items()):
+        say("    %-22s %.2e %.2e" % (k, v[0], v[1]))
+    kinds = set(worst)
+    assert {"matmul NT", "matmul NN", "matmul NN+", "matmul TN", "rms_norm_bwd", "rope_bwd", "silu_gate_bwd",
+            "attention_bwd", "softmax_ce_bwd", "embed_bwd"} <= kinds
+    assert count[0] >= 55

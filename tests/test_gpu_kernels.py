@@ -539,6 +539,46 @@ def test_fused_attention(ops, oracle, S, H, Dh):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("gain,exact", [(8.0, False), (24.0, True), (2.0, True)])
+def test_fused_attention_with_large_scores(ops, oracle, gain, exact):
+    """Scores of large magnitude (row maxima in the hundreds for gain 8, 1500 .. 2600 for 24): by default
+    the fused kernels fold the row maximum and the logarithm of the row sum into one fp32 exponent offset,
+    whose rounding error is common to a row and grows with |m|; the probabilities are nearly one-hot here,
+    the case in which the adjoint's dP - sigma cancels exactly in the reference.  The default forms hold
+    the literal bar at gain 8; at gain 24 they do not (dQ 7e-3) and cacti_hip_attention_set_exact(1)
+    selects the exactly rounded forms, which do -- they are also run once on ordinary scores."""
+    from cacti_amd import ffi
+    ffi.call("cacti_hip_attention_set_exact", int(exact))
+    try:
+        _large_scores_case(ops, oracle, gain)
+    finally:
+        ffi.call("cacti_hip_attention_set_exact", 0)
+
+
+def _large_scores_case(ops, oracle, gain):
+    S, H, Dh = 384, 3, 100
+    say("fused attention, large scores, gain", gain)
+    r = rng(1300 + int(gain))
+    alpha = float(np.float32(1.0) / np.sqrt(np.float32(Dh)))
+    q, k = (randn16(r, (S, H, Dh), gain) for _ in range(2))
+    v, dO = (randn16(r, (S, H, Dh)) for _ in range(2))
+    ws16, _, wo = oracle.attention_fwd(q, k, v, alpha)
+    low = np.arange(S)[:, None, None] >= np.arange(S)[None, None, :]
+    m = np.where(low, ws16.astype(np.float32), -np.inf).max(2)
+    say("  row maxima of the scores: median %.0f, largest %.0f" % (np.median(np.abs(m)), np.abs(m).max()))
+    assert np.abs(m).max() > 9 * gain and np.all(np.isfinite(ws16.astype(np.float32)))
+    dq_, dk_, dv_ = oracle.attention_bwd(q, k, v, dO, alpha)
+    Q, K_, V_, DO = dev(q), dev(k), dev(v), dev(dO)
+    o, stats = ops.attention_fwd(Q, K_, V_, alpha)
+    e2, em = assert_parity(host(o), wo, "o")
+    say("  o  rel_l2 %.2e max_rel %.2e" % (e2, em))
+    dq, dk, dv = ops.attention_bwd(Q, K_, V_, DO, stats, alpha)
+    for name, got, want in (("dv", dv, dv_), ("dq", dq, dq_), ("dk", dk, dk_)):
+        e2, em = assert_parity(host(got), want, name)
+        say("  %s rel_l2 %.2e max_rel %.2e" % (name, e2, em))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("S,H,Dh", [(64, 4, 64), (2048, 32, 100), (37, 4, 20), (16, 4, 6)])
 def test_rope_on_two_tensors_in_one_launch(S, H, Dh):
     """cacti_hip_rope_{fwd,bwd}_pair: bit for bit what two single launches give, accumulation included

@@ -261,6 +261,15 @@ def test_pool_too_small_is_a_clean_error(oracle):
     with pytest.raises(CactiError) as e:
         m.step(tok, lm_tok, scale)
     assert e.value.code == -4
+    assert "pinned by the running thunk" in str(e.value) and "largest free" in str(e.value)
+    # the usage table by class of cell (the reference dumps it before it panics, src/pctx/nvgpu.rs:2424-2440)
+    rep = ctx.usage_report()
+    print(rep)
+    lines = rep.splitlines()
+    assert lines[0].startswith("pool: cap=%d " % (1 << 19))
+    assert [l.split()[0] for l in lines[1:6]] == ["parameters", "gradients", "optimiser", "tables,", "cycle"]
+    n_par = int(lines[1].split("cells=")[1].split()[0])
+    assert n_par == 3 + 9 * cfg.L and int(lines[2].split("cells=")[1].split()[0]) == n_par
     m.close(); ctx.close()
 
 
@@ -424,3 +433,41 @@ def test_capped_pool_spills_at_full_shapes():
         assert np.array_equal(ref[cyc][0], got[cyc][0]), "loss, cycle %d" % cyc
         for n in probe:
             assert np.array_equal(ref[cyc][1][n].view(np.uint16), got[cyc][1][n].view(np.uint16)), (cyc, n)
+
+
+def test_full_depth_step_on_a_16_gib_pool():
+    """The whole 26-layer OpenLLaMA-3B-shaped step on a pool capped at 16 GiB (the reference's card,
+    examples/open_llama_3b_train.rs): two cycles; the loss and twelve probed gradients (first and last
+    layers, every kind of tensor, embedding and LM head) are bit-identical to the uncapped run's, and the
+    capped run really spilled."""
+    import bench
+    from cacti_amd.runtime import Ctx, Llama
+    cfg = dict(bench.LLAMA_3B)
+    assert cfg["L"] == 26
+    tok, lm_tok, scale = bench.synth_inputs(cfg)
+
+    def run(pool_bytes):
+        print("26 layers on a pool of %.0f GiB" % (pool_bytes / 2 ** 30), flush=True)
+        ctx = Ctx(0, pool_bytes, True)
+        m = Llama(ctx, **cfg)
+        bench.synth_params(m)
+        out = []
+        for _ in range(2):
+            loss = m.step(tok, lm_tok, scale)
+            out.append((loss, bench.probe_grads(m, cfg)))
+        st = ctx.stats()
+        m.close(); ctx.close()
+        return out, st
+
+    got, st = run(bench.CAPPED_POOL_BYTES)
+    ref, st0 = run(40 << 30)
+    print("uncapped peak %.2f GB; at 16 GiB: %d evictions, %.2f GB down, %.2f GB up over two cycles"
+          % (st0["pool_peak"] / 1e9, st["n_evict"], st["bytes_d2h"] / 1e9, st["bytes_h2d"] / 1e9), flush=True)
+    assert st0["n_evict"] == 0
+    assert st["n_evict"] > 0 and st["bytes_d2h"] > 0 and st["bytes_h2d"] > 0 and st["pool_peak"] <= st["pool_cap"]
+    for cyc in range(2):
+        assert np.all(np.isfinite(ref[cyc][0]))
+        assert np.array_equal(ref[cyc][0], got[cyc][0]), "loss, cycle %d" % cyc
+        assert len(ref[cyc][1]) >= 12
+        for n, g in ref[cyc][1].items():
+            assert np.array_equal(g.view(np.uint16), got[cyc][1][n].view(np.uint16)), (cyc, n)
