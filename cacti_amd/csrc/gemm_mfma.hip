@@ -3,9 +3,11 @@
 //
 //   C[M,N] = alpha op(A) op(B) + beta C,   f16 in, fp32 MFMA accumulate, f16 out.
 //
-// Block tile BM x BN x 64, WM x WN wavefronts, each owning BM / WM x BN / WN outputs as
-// 32 x 32 accumulators fed by v_mfma_f32_32x32x16_f16 (the 32 x 32 tiles of a wave are
-// interleaved with those of the other waves, 32 WM rows / 32 WN columns apart).  Shapes
+// Block tile BM x BN x 64, WM x WN wavefronts, each owning BM / WM x BN / WN outputs as 32 x 32
+// blocks that are interleaved with those of the other waves (32 WM rows / 32 WN columns apart).
+// The register path forms a block with v_mfma_f32_32x32x16_f16; the direct path, which carries the
+// large products of the step, as four 16 x 16 results of v_mfma_f32_16x16x32_f16: under a sustained
+// load the device is limited by power, and that instruction needs less of it per flop.  Shapes
 // instantiated: 128 x 128 on 4 waves (two workgroups per CU), 256 x 128 and 256 x 256 on 8
 // waves (one per CU), 64 x 64 on 4 waves (remainder columns).
 //
@@ -36,7 +38,9 @@
 // that are never stored); a k tail is zeroed with selects (KTAIL instantiations only).
 // With STAGES = 2 the global loads of k tile t+2 are issued before the MFMAs of tile t and
 // stored to LDS after the MFMAs of tile t+1 (two register stages + double-buffered LDS);
-// STAGES = 1 looks one tile ahead.  One barrier per k tile.  Workgroups are numbered so
+// STAGES = 1 looks one tile ahead.  One barrier per k tile; in the direct kernels it sits before
+// the tile's last k step, so that the loads of a later tile and the first fragments of the next
+// one are issued between the MFMAs of that step and no wave waits on LDS behind a barrier.  Workgroups are numbered so
 // that the 8 XCDs (round-robin dispatch) each walk a contiguous band of tiles and reuse
 // the operand panels in their own L2.
 #include "common.h"
@@ -171,6 +175,16 @@ struct LoadKCD {
                          : "memory");
         }
     }
+    // instruction `it` of the NL alone (base = origin + k0): lets the caller place each load between MFMAs
+    __device__ __forceinline__ void dma1(int it, uint32_t lds, const half_t *base) const
+    {
+        const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds + (threadIdx.x & ~63u) * 16 + it * NT * 16);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(m0), "v"(off[it]), "s"(base)
+                     : "memory");
+    }
+    __device__ __forceinline__ const half_t *kbase(const half_t *origin, int64_t k0) const { return origin + k0; }
     __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
     __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
     static constexpr int NREG = 1;
@@ -216,6 +230,15 @@ struct LoadKSD {
                          : "memory");
         }
     }
+    __device__ __forceinline__ void dma1(int it, uint32_t lds, const half_t *base) const
+    {
+        const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds + (threadIdx.x & ~63u) * 16 + it * NT * 16);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(m0), "v"(off[it]), "s"(base)
+                     : "memory");
+    }
+    __device__ __forceinline__ const half_t *kbase(const half_t *origin, int64_t k0) const { return origin + k0 * ld; }
     __device__ __forceinline__ void load(uint4 *, const half_t *, int64_t) const {}
     __device__ __forceinline__ void store(const uint4 *, half_t *) const {}
     static constexpr int NREG = 1;
@@ -620,6 +643,10 @@ gemm_mfma_kernel(GemmArgs p)
     }
     uint4 ra[STAGES][LA::NREG], rb[STAGES][LB::NREG];
 
+    // direct path: 16 x 16 results of v_mfma_f32_16x16x32_f16, [A fragment][B fragment]; lane l holds row
+    // l % 16 of the fragment pair's block and columns 4 (l / 16) .. + 3
+    float4_t c16[DMA ? 2 * TM : 1][DMA ? 2 * TN : 1];
+    const int l16 = lane & 15, kg = lane >> 4;
     float16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -717,13 +744,9 @@ gemm_mfma_kernel(GemmArgs p)
     // (t + j - kt0) % STAGES holds tile t + j for j = 1 .. STAGES - 1 and set (t - kt0) % STAGES
     // is free; a step loads tile t + STAGES into the free set, runs the MFMAs of tile t, moves
     // tile t + 1 from its set to the other LDS buffer and ends in the one barrier of the k tile.
-    // Direct (NBUF LDS buffers): at the start of tile t its buffer is complete behind a barrier
-    // and the loads of tiles t + 1 .. t + NBUF - 2 are in flight; a step issues the loads of tile
-    // t + NBUF - 1 into the buffer tile t - 1 has left, runs the MFMAs of tile t, waits until
-    // only the loads issued after those of tile t + 1 are outstanding, and ends in the barrier.
     // The main loop has no branch (all its loads are inside K); the last tiles are peeled
-    // into steps that test what still exists.
-    constexpr int LOOK = DMA ? NBUF - 1 : STAGES;                 // tiles between load and use
+    // into steps that test what still exists.  (Direct loads: the rotated pipeline further down.)
+    constexpr int LOOK = STAGES;                                  // tiles between load and use
     auto next_buf = [](int b) __attribute__((always_inline)) { return b + 1 == NBUF ? 0 : b + 1; };
     auto lds_addr = [](const half_t *q) __attribute__((always_inline)) {
         return (uint32_t)(uintptr_t)q;                            // LDS byte address of a shared pointer
@@ -731,49 +754,186 @@ gemm_mfma_kernel(GemmArgs p)
     auto step = [&](auto set_c, auto main_c, int t, int cbv) __attribute__((always_inline)) {
         constexpr int U = decltype(set_c)::value, UN = (U + 1) % STAGES;
         constexpr bool MAIN = decltype(main_c)::value;
-        const int cb = DMA ? cbv : (t & 1), nb1 = next_buf(cb);
+        (void)cbv;
+        const int cb = t & 1, nb1 = next_buf(cb);
         if (MAIN || t + LOOK < nk) {
-            if (DMA) {
-                const int dst = cb == 0 ? NBUF - 1 : cb - 1;      // the buffer tile t - 1 has left
-                la.dma(lds_addr(As + dst * BM * BK), Ao, (int64_t)(t + LOOK) * BK);
-                lb.dma(lds_addr(Bs + dst * BN * BK), Bo, (int64_t)(t + LOOK) * BK);
-            } else {
-                la.load(ra[U], Ao, (int64_t)(t + LOOK) * BK);
-                lb.load(rb[U], Bo, (int64_t)(t + LOOK) * BK);
-            }
+            la.load(ra[U], Ao, (int64_t)(t + LOOK) * BK);
+            lb.load(rb[U], Bo, (int64_t)(t + LOOK) * BK);
         }
         compute(cb);
-        if (!DMA && (MAIN || t + 1 < nk)) {
+        if (MAIN || t + 1 < nk) {
             la.store(ra[UN], As + nb1 * BM * BK);
             lb.store(rb[UN], Bs + nb1 * BN * BK);
         }
-        if (DMA) {
-            if (MAIN) wait_vmem<(LOOK - 1) * (LA::NDMA + LB::NDMA)>();
-            else wait_vmem<0>();
-        }
         __syncthreads();
     };
-    {
-        if (DMA) {
+    if constexpr (DMA) {
+        // Direct loads: v_mfma_f32_16x16x32_f16 and a rotated pipeline.
+        //
+        // The 16 x 16 x 32 product: under a sustained load with real operands the device is limited by
+        // power, not by cycles, and per flop this instruction costs less of it than the 32 x 32 x 16 one (a
+        // quarter of the accumulator registers read and written per flop): measured on random operands,
+        // same fragment traffic, 1570 .. 1600 against 1435 TFLOP/s sustained.  A wave's 32-row blocks are
+        // the same as in the register path, each cut into two 16-row fragments; a k tile of 64 is two k steps
+        // of 32, each k step two halves (the first / second TM of the wave's 2 TM A fragments against all
+        // 2 TN B fragments).  Lane l supplies, for row l % 16 of a fragment, the 8 k values of group l / 16,
+        // and holds row l % 16, columns 4 (l / 16) .. + 3 of a 16 x 16 result.
+        //
+        // The pipeline: while the MFMAs of one half run, the A fragments of the next half (and, in a second
+        // half, the B fragments of the next k step) are read.  The one barrier of a k tile sits before its
+        // LAST half: by then a wave has every fragment of the tile in registers, so behind the barrier (a) the
+        // tile's own buffer is free and takes the loads of the tile NBUF tiles further on, and (b) the next
+        // tile, complete behind the same barrier, gives its first fragments while the MFMAs of this tile's
+        // last half run.  The fragment ring never drains and nothing but MFMAs stands right behind the
+        // barrier, where all waves of the workgroup are in step: loads and reads are placed between them.
+        constexpr int ND = LA::NDMA + LB::NDMA;
+        static_assert(BK == 64 && NBUF >= 2, "two k steps of 32 per tile");
+        constexpr int NA = 2 * TM, NB = 2 * TN;                   // 16-row fragments of a wave per k step
+        constexpr int NMH = TM * NB;                              // MFMAs of a half
+        constexpr int RA = (TR_A ? 2 : 1) * TM, RB = (TR_B ? 2 : 1) * NB;   // LDS reads: A fragments of a half, all B
 #pragma unroll
-            for (int u = 0; u < LOOK; u++)
-                if (kt0 + u < nk) {
-                    la.dma(lds_addr(As + u * BM * BK), Ao, (int64_t)(kt0 + u) * BK);
-                    lb.dma(lds_addr(Bs + u * BN * BK), Bo, (int64_t)(kt0 + u) * BK);
-                }
-            wait_vmem<0>();
-        } else {
-            la.load(ra[0], Ao, (int64_t)kt0 * BK);
-            lb.load(rb[0], Bo, (int64_t)kt0 * BK);
+        for (int a = 0; a < NA; a++)
 #pragma unroll
-            for (int u = 1; u < STAGES; u++)
-                if (kt0 + u < nk) {
-                    la.load(ra[u], Ao, (int64_t)(kt0 + u) * BK);
-                    lb.load(rb[u], Bo, (int64_t)(kt0 + u) * BK);
+            for (int b = 0; b < NB; b++) c16[a][b] = float4_t{0.f, 0.f, 0.f, 0.f};
+        half8_t fa[2][TM], fb[2][NB];                             // A fragments of a half, B fragments of a k step
+        // [row][k] tiles: halves offset of the lane's row in a block's upper / lower 16 rows, and its swizzle
+        const int ar[2] = {wm * 32 + l16, wm * 32 + 16 + l16}, br[2] = {wn * 32 + l16, wn * 32 + 16 + l16};
+        const int asw2[2] = {swz(ar[0]), swz(ar[1])}, bsw2[2] = {swz(br[0]), swz(br[1])};
+        // [k][row] tiles: byte offset of the lane's first transposing read; its 16-lane group (= k group)
+        // fetches k rows 8 kg + a4 of rows 4 b4 .. 4 b4 + 3 of the 16
+        auto tr16 = [&](int w16, int pitch) __attribute__((always_inline)) {
+            const int chunk = w16 / 8 + (b4 >> 1);
+            return (8 * kg + a4) * pitch + ((chunk ^ (2 * a4)) << 4) + ((b4 & 1) << 3);
+        };
+        const int atr2[2] = {tr16(wm * 32, BM * 2), tr16(wm * 32 + 16, BM * 2)};
+        const int btr2[2] = {tr16(wn * 32, BN * 2), tr16(wn * 32 + 16, BN * 2)};
+        auto frag_tr = [&](const unsigned char *q, int pitch) __attribute__((always_inline)) {
+            const uint2 lo = lds_read_tr(q), hi = lds_read_tr(q + 4 * pitch);
+            const uint4 v = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            half8_t f;
+            __builtin_memcpy(&f, &v, 16);
+            return f;
+        };
+        // A fragment a (0 .. NA - 1) / B fragment b of k step ks (0, 1) of the tile in buffer `buf`
+        auto read_a = [&](int buf, int ks, int a) __attribute__((always_inline)) {
+            const int blk = a >> 1, sub = a & 1;
+            if (TR_A)
+                return frag_tr(reinterpret_cast<const unsigned char *>(As + buf * BM * BK) + atr2[sub] +
+                                   ks * 32 * (BM * 2) + blk * (32 * WM * 2),
+                               BM * 2);
+            return *reinterpret_cast<const half8_t *>(As + buf * BM * BK + ar[sub] * BK + blk * ASTEP +
+                                                      (((ks * 4 + kg) ^ asw2[sub]) << 3));
+        };
+        auto read_b = [&](int buf, int ks, int b) __attribute__((always_inline)) {
+            const int blk = b >> 1, sub = b & 1;
+            if (TR_B)
+                return frag_tr(reinterpret_cast<const unsigned char *>(Bs + buf * BN * BK) + btr2[sub] +
+                                   ks * 32 * (BN * 2) + blk * (32 * WN * 2),
+                               BN * 2);
+            return *reinterpret_cast<const half8_t *>(Bs + buf * BN * BK + br[sub] * BK + blk * BSTEP +
+                                                      (((ks * 4 + kg) ^ bsw2[sub]) << 3));
+        };
+        // the reads a half issues for what follows it, in the order the MFMAs there first need them (an A
+        // fragment outer, the B fragments inner): A 0, every B, A 1 ..  `nxt` = (buffer, k step, half) of what
+        // follows; unit u of NU
+        auto next_read = [&](int u, int nbuf, int nks, int nh) __attribute__((always_inline)) {
+            if (nh == 1) {                                        // second half of the same k step: its A fragments
+                fa[1][u] = read_a(nbuf, nks, TM + u);
+            } else if (u == 0) {
+                fa[0][0] = read_a(nbuf, nks, 0);
+            } else if (u <= NB) {
+                fb[nks][u - 1] = read_b(nbuf, nks, u - 1);
+            } else {
+                fa[0][u - NB] = read_a(nbuf, nks, u - NB);
+            }
+        };
+        auto mfma1 = [&](int h, int ks, int m) __attribute__((always_inline)) {
+            const int a = m / NB, b = m % NB;
+            c16[h * TM + a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[ks][b], fa[h][a], c16[h * TM + a][b], 0, 0, 0);
+        };
+        // a half with the reads for the next one spread between its MFMAs by the scheduler's groups
+        auto half_pinned = [&](int h, int ks, int buf, int nbuf, int nks, int nh) __attribute__((always_inline)) {
+            const int nu = nh == 1 ? TM : TM + NB;
+#pragma unroll
+            for (int u = 0; u < TM + NB; u++)
+                if (u < nu) next_read(u, nbuf, nks, nh);
+#pragma unroll
+            for (int m = 0; m < NMH; m++) mfma1(h, ks, m);
+        };
+        auto issue_all = [&](int tile, int buf) __attribute__((always_inline)) {
+            la.dma(lds_addr(As + buf * BM * BK), Ao, (int64_t)tile * BK);
+            lb.dma(lds_addr(Bs + buf * BN * BK), Bo, (int64_t)tile * BK);
+        };
+        // the first three halves of the tile in buffer cb (fa[0], fb[0] hold the first half's fragments)
+        auto first_halves = [&](int cb) __attribute__((always_inline)) {
+            half_pinned(0, 0, cb, cb, 0, 1);
+            SchedStep<NMH, RA, 0>::run();
+            half_pinned(1, 0, cb, cb, 1, 0);
+            SchedStep<NMH, RA + RB, 0>::run();
+            half_pinned(0, 1, cb, cb, 1, 1);
+            SchedStep<NMH, RA, 0>::run();
+            __builtin_amdgcn_sched_barrier(0);
+        };
+#pragma unroll
+        for (int u = 0; u < NBUF; u++)
+            if (kt0 + u < nk) issue_all(kt0 + u, u);
+        if (kt0 + NBUF <= nk) wait_vmem<(NBUF - 1) * ND>();       // the first tile; the others stay in flight
+        else wait_vmem<0>();
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < TM + NB; u++) next_read(u, 0, 0, 0);
+        int t = kt0, cb = 0;
+        for (; t + NBUF < nk; t++) {                              // every load of the body lies inside K
+            first_halves(cb);
+            const int nb = next_buf(cb);
+            wait_vmem<(NBUF - 2) * ND>();                         // tile t + 1 has landed (this wave's part of it)
+            __syncthreads();
+            // last half: MFMA by MFMA, with the loads of tile t + NBUF (into the buffer of this tile) and
+            // the first fragments of tile t + 1 between them
+            const half_t *abase = la.kbase(Ao, (int64_t)(t + NBUF) * BK), *bbase = lb.kbase(Bo, (int64_t)(t + NBUF) * BK);
+            const uint32_t alds = lds_addr(As + cb * BM * BK), blds = lds_addr(Bs + cb * BN * BK);
+            constexpr int NU = TM + NB;
+#pragma unroll
+            for (int m = 0; m < NMH; m++) {
+                mfma1(1, 1, m);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int d = m * ND / NMH; d < (m + 1) * ND / NMH; d++) {
+                    if (d < LA::NDMA) la.dma1(d, alds, abase);
+                    else lb.dma1(d - LA::NDMA, blds, bbase);
                 }
-            la.store(ra[0], As + (kt0 & 1) * BM * BK);
-            lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
+#pragma unroll
+                for (int u = m * NU / NMH; u < (m + 1) * NU / NMH; u++) next_read(u, nb, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            cb = nb;
         }
+        for (; t < nk; t++) {                                     // the last NBUF tiles: nothing left to load
+            first_halves(cb);
+            const int nb = next_buf(cb);
+            if (t + 1 < nk) {
+                wait_vmem<0>();
+                __syncthreads();
+#pragma unroll
+                for (int u = 0; u < TM + NB; u++) next_read(u, nb, 0, 0);
+            }
+#pragma unroll
+            for (int m = 0; m < NMH; m++) mfma1(1, 1, m);
+            __builtin_amdgcn_sched_barrier(0);
+            cb = nb;
+        }
+        __syncthreads();                                          // every wave is done with the operand buffers
+    } else {
+        la.load(ra[0], Ao, (int64_t)kt0 * BK);
+        lb.load(rb[0], Bo, (int64_t)kt0 * BK);
+#pragma unroll
+        for (int u = 1; u < STAGES; u++)
+            if (kt0 + u < nk) {
+                la.load(ra[u], Ao, (int64_t)(kt0 + u) * BK);
+                lb.load(rb[u], Bo, (int64_t)(kt0 + u) * BK);
+            }
+        la.store(ra[0], As + (kt0 & 1) * BM * BK);
+        lb.store(rb[0], Bs + (kt0 & 1) * BN * BK);
         __syncthreads();
         int kt = kt0, cb = 0;
         for (; kt + STAGES - 1 + LOOK < nk; kt += STAGES) {
@@ -833,29 +993,51 @@ gemm_mfma_kernel(GemmArgs p)
         }
         __syncthreads();
     }
+    if constexpr (DMA) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int row = i * (32 * WM) + wm * 32 + l32;
+        for (int a = 0; a < 2 * TM; a++) {
+            const int row = (a >> 1) * (32 * WM) + wm * 32 + (a & 1) * 16 + l16;
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int col = j * (32 * WN) + wn * 32 + q * 8 + lh * 4;
+            for (int b = 0; b < 2 * TN; b++) {
+                const int col = (b >> 1) * (32 * WN) + wn * 32 + (b & 1) * 16 + kg * 4;
                 half_t *sp = Cs + row * BN + ((((col >> 3) ^ (row & CSW)) << 3) | (col & 4));
                 half4_t o;
                 if (has_beta) {
                     const half4_t old = *reinterpret_cast<const half4_t *>(sp);
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        o[r] = f2h(p.alpha * acc[i][j][q * 4 + r] + p.beta * h2f(old[r]));
+                    for (int r = 0; r < 4; r++) o[r] = f2h(p.alpha * c16[a][b][r] + p.beta * h2f(old[r]));
                 } else {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) o[r] = f2h(p.alpha * acc[i][j][q * 4 + r]);
+                    for (int r = 0; r < 4; r++) o[r] = f2h(p.alpha * c16[a][b][r]);
                 }
                 *reinterpret_cast<half4_t *>(sp) = o;
             }
         }
-    }
+    } else {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int row = i * (32 * WM) + wm * 32 + l32;
+    #pragma unroll
+            for (int j = 0; j < TN; j++) {
+    #pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int col = j * (32 * WN) + wn * 32 + q * 8 + lh * 4;
+                    half_t *sp = Cs + row * BN + ((((col >> 3) ^ (row & CSW)) << 3) | (col & 4));
+                    half4_t o;
+                    if (has_beta) {
+                        const half4_t old = *reinterpret_cast<const half4_t *>(sp);
+    #pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            o[r] = f2h(p.alpha * acc[i][j][q * 4 + r] + p.beta * h2f(old[r]));
+                    } else {
+    #pragma unroll
+                        for (int r = 0; r < 4; r++) o[r] = f2h(p.alpha * acc[i][j][q * 4 + r]);
+                    }
+                    *reinterpret_cast<half4_t *>(sp) = o;
+                }
+            }
+        }
+}
     __syncthreads();
     for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
         const int row = c / CPRC, cc = c % CPRC;
