@@ -614,16 +614,16 @@ def run_attention(args):
 
     def bwd(i):
         ffi.call("cacti_hip_attention_bwd", S, H, Dh, alpha, q[0].data_ptr(), k[0].data_ptr(), v[0].data_ptr(),
-                 dO[i % R].data_ptr(), ld, stats.data_ptr(), dq.data_ptr(), 0, dk.data_ptr(), 0, dv.data_ptr(), 0,
+                 o.data_ptr(), dO[i % R].data_ptr(), ld, stats.data_ptr(), dq.data_ptr(), 0, dk.data_ptr(), 0, dv.data_ptr(), 0,
                  ws.data_ptr(), ws_bytes, st)
 
     res = []
     t_f = time_launches(fwd, None)
-    fwd(0)                                                  # the statistics of operand set 0 for the adjoint
+    fwd(0)                                                  # the statistics and output of operand set 0 for the adjoint
     t_b = time_launches(bwd, None)
     tensor = S * H * Dh * 2
     for label, sec, nbytes in (("attention", t_f, 4 * tensor + stats.numel() * 4),
-                               ("attention_bwd", t_b, 7 * tensor + stats.numel() * 4)):
+                               ("attention_bwd", t_b, 8 * tensor + stats.numel() * 4)):
         fl = attention_flops(label, cfg)
         res.append({"kernel": label, "us": sec * 1e6, "flops": fl, "bytes": nbytes, "tflops": fl / sec / 1e12,
                     "frac": fl / sec / 1e12 / PEAK_MFMA_F16_TFLOPS, "bound": "mfma"})

@@ -53,12 +53,14 @@ constexpr int kTileRows = 64;
 constexpr int kTileB = kTileRows * kRowB;   // 16 KB
 constexpr int kNT = 256;                 // threads of a wave group (4 waves): the unit that loads a tile
 constexpr int kBM = 128;                 // rows of the fixed operand per wave group (32 per wave)
+constexpr float kSpread = 8.f;           // least row sum of exponentials for the short form of sigma (dQ kernel)
 
 struct AttnArgs {
     int S, H, Dh;
     int64_t ld;
     float alpha;
     const half_t *q, *k, *v, *dO;
+    const half_t *o;                     // the forward output (adjoint only; may be null)
     half_t *out, *dq, *dk, *dv;
     float *m, *l;                        // [H][S] row maximum and sum (forward output)
     float *y, *sig;                      // [H][S] adjoint scratch: sigma, and 1 / l (exact arithmetic) or the
@@ -777,16 +779,37 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             }
             return part;
         };
-        {
+        // sigma_i = sum_j P'_ij f32(dP16_ij).  In exact arithmetic that is sum_d dO_id O_id, which needs no pass
+        // over the keys; in the reference's arithmetic the two differ by the f16 roundings of dP16, P16 and O,
+        // about 2^-11 |dP| sqrt(sum_j P_ij^2).  Where a row's probability mass is spread that is below the
+        // rounding of dS16 itself.  Where it sits on one key it is not: the reference has dP16 - sigma = 0
+        // there exactly, and rows 0 and 1 of a sequence failed the element bound with the short form.  So a
+        // workgroup takes the short form only if every one of its rows has sum_j exp(S16_ij - m_i) >= kSpread
+        // (no probability above 1 / kSpread), else the pass over the keys; the exactly rounded build always
+        // takes the pass.
+        bool short_sigma = false;
+        if constexpr (FAST) {
+            if (p.o) short_sigma = __syncthreads_and(myrow >= S || l >= kSpread) != 0;
+        }
+        if (short_sigma) {
+            half8_t of[KS];
+            load_frags<KS>(of, gp(p.o) + hoff, ld, myrow, S, Dh, lh);
+            float part = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) part = __builtin_fmaf((float)gf[ks][e], (float)of[ks][e], part);
+            sig = part + __shfl_xor(part, 32, 64);                     // the two lanes of a row
+        } else {
             const float part = run_pass(std::integral_constant<int, 0>{});
             const float pg = part + __shfl_xor(part, 32, 64);         // the two lanes of a row, then the two groups
             if (lh == 0) xs[g * kBM + wid * 32 + l32] = pg;
             __syncthreads();
             sig = xs[wid * 32 + l32] + xs[kBM + wid * 32 + l32];
-            if (g == 0 && lh == 0 && myrow < S) {
-                p.y[(int64_t)h * S + myrow] = FAST ? cs : y;      // what the dK / dV kernel wants per row
-                p.sig[(int64_t)h * S + myrow] = sig;
-            }
+        }
+        if (g == 0 && lh == 0 && myrow < S) {
+            p.y[(int64_t)h * S + myrow] = FAST ? cs : y;          // what the dK / dV kernel wants per row
+            p.sig[(int64_t)h * S + myrow] = sig;
         }
 #pragma unroll
         for (int dt = 0; dt < DT; dt++)
@@ -1048,7 +1071,7 @@ CACTI_API int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float al
 }
 
 CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float alpha, const void *q, const void *k,
-                                      const void *v, const void *dO, int64_t ld, const void *stats,
+                                      const void *v, const void *o, const void *dO, int64_t ld, const void *stats,
                                       void *dq, int dq_acc, void *dk, int dk_acc, void *dv, int dv_acc,
                                       void *workspace, size_t workspace_bytes, void *stream)
 {
@@ -1056,7 +1079,7 @@ CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float al
     if (rc) return rc;
     CACTI_REQUIRE(q && k && v && dO && stats && dq && dk && dv && workspace, CACTI_E_INVALID,
                   "attention_bwd: null pointer");
-    CACTI_REQUIRE(aligned(q, 8) && aligned(k, 8) && aligned(v, 8) && aligned(dO, 8) &&
+    CACTI_REQUIRE(aligned(q, 8) && aligned(k, 8) && aligned(v, 8) && aligned(dO, 8) && aligned(o, 8) &&
                       aligned(dq, 8) && aligned(dk, 8) && aligned(dv, 8) && aligned(stats, 4) && aligned(workspace, 4),
                   CACTI_E_INVALID, "attention_bwd: tensors must be 8-byte aligned");
     CACTI_REQUIRE(workspace_bytes >= cacti_hip_attention_bwd_workspace(S, H), CACTI_E_INVALID,
@@ -1066,6 +1089,7 @@ CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float al
     p.S = (int)S; p.H = (int)H; p.Dh = (int)Dh; p.ld = ld; p.alpha = alpha;
     p.q = (const half_t *)q; p.k = (const half_t *)k; p.v = (const half_t *)v;
     p.dO = (const half_t *)dO;
+    p.o = (const half_t *)o;
     p.dq = (half_t *)dq; p.dk = (half_t *)dk; p.dv = (half_t *)dv;
     p.acc_dq = dq_acc; p.acc_dk = dk_acc; p.acc_dv = dv_acc;
     p.m = (float *)const_cast<void *>(stats);

@@ -469,12 +469,13 @@ struct AttentionBwdSpec : ThunkSpec {
     float alpha;
     AttentionBwdSpec(int64_t h, float a) : H(h), alpha(a) {}
     const char *name() const override { return "attention_bwd"; }
-    int arity() const override { return 5; }                       // (q, k, v, dO, stats) -> dq, dk, dv
+    int arity() const override { return 6; }                       // (q, k, v, dO, stats, o) -> dq, dk, dv
     int nout() const override { return 3; }
     int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
     {
-        TY_REQUIRE(a[0] == a[1] && a[0] == a[2] && a[0] == a[3] && a[0].shape.size() == 2 && a[4].dtype == F32,
-                   "attention_bwd: (q, k, v, dO f16 [S,H*Dh], stats f32) expected");
+        TY_REQUIRE(a[0] == a[1] && a[0] == a[2] && a[0] == a[3] && a[0] == a[5] && a[0].shape.size() == 2 &&
+                       a[4].dtype == F32,
+                   "attention_bwd: (q, k, v, dO f16 [S,H*Dh], stats f32, o) expected");
         o = {a[0], a[0], a[0]};
         return 0;
     }
@@ -486,7 +487,7 @@ struct AttentionBwdSpec : ThunkSpec {
             void *const *o, uint32_t acc, void *ws, size_t wsb) const override
     {
         const auto &s = aty[0].shape;
-        return cacti_hip_attention_bwd(s[0], H, s[1] / H, alpha, a[0], a[1], a[2], a[3], s[1], a[4], o[0],
+        return cacti_hip_attention_bwd(s[0], H, s[1] / H, alpha, a[0], a[1], a[2], a[5], a[3], s[1], a[4], o[0],
                                        acc & 1, o[1], (acc >> 1) & 1, o[2], (acc >> 2) & 1, ws, wsb, S(c));
     }
 };
@@ -518,7 +519,7 @@ struct AttentionSpec : ThunkSpec {
         if (!dy[0]) return 0;
         return c.adj_add({e.args[0], e.args[1], e.args[2]},
                          std::unique_ptr<ThunkSpec>(new AttentionBwdSpec(H, alpha)),
-                         {e.args[0], e.args[1], e.args[2], dy[0], e.outs[1]});
+                         {e.args[0], e.args[1], e.args[2], dy[0], e.outs[1], e.outs[0]});
     }
 };
 

@@ -78,7 +78,7 @@ SIGNATURES = {
     "cacti_hip_attention_stats_bytes": (sz, [i64, i64]),
     "cacti_hip_attention_fwd": (ci, [i64, i64, i64, f32, vp, vp, vp, i64, vp, vp, vp]),
     "cacti_hip_attention_bwd_workspace": (sz, [i64, i64]),
-    "cacti_hip_attention_bwd": (ci, [i64, i64, i64, f32, vp, vp, vp, vp, i64, vp, vp, ci, vp, ci, vp, ci,
+    "cacti_hip_attention_bwd": (ci, [i64, i64, i64, f32, vp, vp, vp, vp, vp, i64, vp, vp, ci, vp, ci, vp, ci,
                                      vp, sz, vp]),
     "cacti_hip_softmax_ce_fwd": (ci, [i64, i64, vp, vp, vp, vp, vp, vp, vp]),
     "cacti_hip_softmax_ce_bwd": (ci, [i64, i64, vp, vp, vp, vp, ci, vp]),

@@ -102,16 +102,20 @@ def attention_fwd(q, k, v, alpha):
     return o, stats
 
 
-def attention_bwd(q, k, v, dO, stats, alpha, acc=None):
-    """Adjoint of attention_fwd: returns (dq, dk, dv); acc = (dq, dk, dv) to accumulate into."""
+def attention_bwd(q, k, v, dO, stats, alpha, acc=None, o=None):
+    """Adjoint of attention_fwd: returns (dq, dk, dv); acc = (dq, dk, dv) to accumulate into; o = the forward
+    output (lets blocks of queries with spread probabilities skip the pass that forms the row sums)."""
     _chk(q), _chk(k), _chk(v), _chk(dO)
+    if o is not None:
+        _chk(o)
     S, H, Dh = q.shape
     dq, dk, dv = acc if acc is not None else (torch.empty_like(q), torch.empty_like(q), torch.empty_like(q))
     a = int(acc is not None)
     nbytes = ffi.lib().cacti_hip_attention_bwd_workspace(S, H)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
     ffi.call("cacti_hip_attention_bwd", S, H, Dh, alpha, q.data_ptr(), k.data_ptr(), v.data_ptr(),
-             dO.data_ptr(), H * Dh, stats.data_ptr(), dq.data_ptr(), a, dk.data_ptr(), a, dv.data_ptr(), a,
+             0 if o is None else o.data_ptr(), dO.data_ptr(), H * Dh, stats.data_ptr(), dq.data_ptr(), a,
+             dk.data_ptr(), a, dv.data_ptr(), a,
              ws.data_ptr(), nbytes, _stream())
     return dq, dk, dv
 

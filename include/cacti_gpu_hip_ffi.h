@@ -256,6 +256,11 @@ int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const vo
  * adjoint; workspace: cacti_hip_attention_bwd_workspace(S, H) bytes, contents undefined on return.
  * *_acc: 0 first write, 1 the product is added to the tensor in fp32 before the one rounding (the
  * GEMMs' beta = 1).
+ * o (adjoint): the forward call's output, or NULL.  With it a block of 128 queries whose rows all have their
+ * probability spread (sum_j exp(S16_ij - m_i) >= 8, i.e. no probability above 1/8) takes its row sums
+ * sum_j T_ij as sum_d dO_id O_id and skips the pass over the keys that forms them from the rounded dP16; the
+ * two agree to 2^-11 |dP| sqrt(sum_j P_ij^2), below the rounding of dS16.  Blocks with a concentrated row
+ * (the first of a sequence always: row 0 sees one key), o = NULL and the exactly rounded forms keep the pass.
  * Arithmetic between the rounding points.  By default a probability is formed as
  * 2^(s log2 e - c) with one fp32 offset c = m log2 e + log2 l per row (row maximum m, row sum l): the
  * rounding of c is an error common to the row, at most half an ulp of c times ln 2 relative -- 3e-6 for
@@ -271,7 +276,7 @@ int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float alpha, const
                             const void *v, int64_t ld, void *o, void *stats, void *stream);
 size_t cacti_hip_attention_bwd_workspace(int64_t S, int64_t H);
 int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float alpha, const void *q, const void *k,
-                            const void *v, const void *dO, int64_t ld, const void *stats,
+                            const void *v, const void *o, const void *dO, int64_t ld, const void *stats,
                             void *dq, int dq_acc, void *dk, int dk_acc, void *dv, int dv_acc,
                             void *workspace, size_t workspace_bytes, void *stream);
 

@@ -85,6 +85,12 @@ def test_fused_attention_one_layer_full_shape(oracle, attention_case):
     for name, t in (("dv", dv), ("dq", dq), ("dk", dk)):
         e2, em = assert_parity(host(t), c[name], name)
         say("  %s rel_l2 %.2e max_rel %.2e" % (name, e2, em))
+    # as the step calls it: with the forward output, so that all blocks of queries but the first take their row
+    # sums from dO . O
+    dq, dk, dv = ops.attention_bwd(Q, K_, V_, DO, stats, c["alpha"], o=o)
+    for name, t in (("dv", dv), ("dq", dq), ("dk", dk)):
+        e2, em = assert_parity(host(t), c[name], name + " (row sums from dO . O)")
+        say("  %s with o: rel_l2 %.2e max_rel %.2e" % (name, e2, em))
 
 
 def test_lm_head_and_cross_entropy_full_shape(oracle):

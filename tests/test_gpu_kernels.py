@@ -525,6 +525,15 @@ def test_fused_attention(ops, oracle, S, H, Dh):
     dq, dk, dv = ops.attention_bwd(Q, K_, V_, DO, stats, alpha)
     for name, got, want in (("dv", dv, dv_), ("dq", dq, dq_), ("dk", dk, dk_)):
         assert_parity(host(got), want, name)
+    # with the forward output handed over, blocks of queries with spread probabilities take their row sums from
+    # dO . O instead of a pass over the keys: the same bar; dV does not depend on the row sums at all
+    dq_o, dk_o, dv_o = ops.attention_bwd(Q, K_, V_, DO, stats, alpha, o=o)
+    for name, got, want in (("dv", dv_o, dv_), ("dq", dq_o, dq_), ("dk", dk_o, dk_)):
+        e2, em = assert_parity(host(got), want, name + " (row sums from dO . O)")
+        say("  %s with o: rel_l2 %.2e max_rel %.2e" % (name, e2, em))
+    assert_bits(host(dv_o), host(dv), "dv with and without o")
+    if S <= 128:                                    # a single block of queries holds row 0: always the pass
+        assert_bits(host(dq_o), host(dq), "dq: the first block of queries keeps the pass over the keys")
     # accumulate mode: the product is added to what the tensors hold, one rounding
     base = [randn16(r, (S, H, Dh)) for _ in range(3)]
     acc = tuple(dev(b) for b in base)
@@ -572,7 +581,8 @@ def _large_scores_case(ops, oracle, gain):
     o, stats = ops.attention_fwd(Q, K_, V_, alpha)
     e2, em = assert_parity(host(o), wo, "o")
     say("  o  rel_l2 %.2e max_rel %.2e" % (e2, em))
-    dq, dk, dv = ops.attention_bwd(Q, K_, V_, DO, stats, alpha)
+    # the forward output is handed over: rows this concentrated must all fall back to the pass over the keys
+    dq, dk, dv = ops.attention_bwd(Q, K_, V_, DO, stats, alpha, o=o)
     for name, got, want in (("dv", dv, dv_), ("dq", dq, dq_), ("dk", dk, dk_)):
         e2, em = assert_parity(host(got), want, name)
         say("  %s rel_l2 %.2e max_rel %.2e" % (name, e2, em))

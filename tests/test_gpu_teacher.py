@@ -89,7 +89,7 @@ def _replay(ops, c):
             return None
         q, k, v = dev(i["q"]), dev(i["k"]), dev(i["v"])
         _, stats = ops.attention_fwd(q, k, v, i["alpha"])
-        dq, dk, dv = ops.attention_bwd(q, k, v, dev(i["dO"]), stats, i["alpha"])
+        dq, dk, dv = ops.attention_bwd(q, k, v, dev(i["dO"]), stats, i["alpha"], o=dev(i["o"]))
         return dict(dq=host(dq), dk=host(dk), dv=host(dv))
     raise AssertionError("no replay for " + c.kind)
 
