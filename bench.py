@@ -65,32 +65,22 @@ def synth_inputs(cfg, seed=1, grad_scale=1024.0):
     return tok, lm_tok, scale
 
 
-# L2-miss traffic per launch of the GEMM kernels at the step's shapes, rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE in KiB per dispatch (profiles/llama3b_step_gemm_hbm_traffic.txt gives the commands);
-# a streaming kernel of known size reads FETCH_SIZE = half its bytes and WRITE_SIZE = its
-# bytes, so bytes = (2.0 * FETCH_SIZE + 1.0 * WRITE_SIZE) * 1024
-GEMM_TRAFFIC_KIB = {
-    ("NT", 2048, 3200, 3200): (48063, 12800), ("NT", 2048, 3200, 8640): (129663, 12800),
-    ("NT", 2048, 8640, 3200): (76884 + 17648, 32768 + 1792),       # two launches: 8192 + 448 columns
-    ("NT", 2048, 32000, 3200): (382107, 128000),
-    ("NN", 2048, 3200, 3200): (48064, 12800), ("NN", 2048, 3200, 3200, "acc"): (54465, 12800),
-    ("NN", 2048, 3200, 8640): (129664, 12800), ("NN", 2048, 3200, 8640, "acc"): (136065, 12800),
-    ("NN", 2048, 8640, 3200): (76886 + 17650, 32768 + 1792),       # two launches
-    ("NN", 2048, 3200, 32000): (480064, 12800),
-    ("TN", 3200, 3200, 2048): (46154, 20000), ("TN", 8640, 3200, 2048): (109965, 54000),
-    ("TN", 3200, 8640, 2048): (95674, 54000), ("TN", 32000, 3200, 2048): (516334, 200000),
-}
+# L2-miss traffic per launch of the GEMM kernels at the step's shapes: measured, not assumed, and tied to
+# the kernels it was measured on.  cacti_amd/gemm_traffic.json is written by `python -m cacti_amd.gemm_traffic`
+# from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) over `bench.py --workload gemm-traffic` and
+# records the hash of csrc/gemm_mfma.hip it was taken on; with any other build of the kernels the roofline
+# line carries "traffic": null instead of figures that no longer describe what runs.
+def _traffic_table():
+    from cacti_amd import gemm_traffic
+    return gemm_traffic.load_current()
 
 
-def gemm_traffic_bytes(label):
-    m = GEMM_RE.match(label)
-    key = (m.group(2) + m.group(3), int(m.group(5)), int(m.group(6)), int(m.group(7)))
-    if m.group(8) and key + ("acc",) in GEMM_TRAFFIC_KIB:
-        key = key + ("acc",)
-    if key not in GEMM_TRAFFIC_KIB:
+def gemm_traffic_bytes(label, table):
+    """Bytes per launch leaving the L2s for the product of a timing label, or None if not measured."""
+    if not table:
         return None
-    f, w = GEMM_TRAFFIC_KIB[key]
-    return (2.0 * f + 1.0 * w) * 1024.0
+    ent = table.get(label)
+    return None if ent is None else float(ent["bytes"])
 
 
 GEMM_RE = re.compile(r"^(block_matmul|matmul)\[([NT])([NT]),(\d+)x(\d+)x(\d+)x(\d+)(,acc)?\]$")
@@ -350,14 +340,18 @@ def run_step(args):
     sec = sum(tot_ms for _, tot_ms in rep.values()) * 1e-3
     cnt = sum(c for c, _ in rep.values())
     achieved = fl / sec / 1e12
-    tr = [(gemm_traffic_bytes(label), c) for label, (c, _) in rep.items()]
+    table = _traffic_table()
+    tr = [(gemm_traffic_bytes(label, table), c) for label, (c, _) in rep.items()]
     traffic = None if any(t is None for t, _ in tr) else sum(t * c for t, c in tr) / cnt
     roofline = {"bound": "mfma", "kernel": sym, "timed_launches": cnt,
                 "avg_launch_us": sec / cnt * 1e6, "flops_per_launch": fl / cnt,
                 "achieved": achieved, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_MFMA_F16_TFLOPS, "traffic": traffic,
-                "traffic_note": "bytes per launch leaving the L2s (MALL or HBM), mean over the timed "
-                                "launches; per-shape counter readings measured offline"}
+                "traffic_note": ("bytes per launch leaving the L2s (MALL or HBM), mean over the timed launches; "
+                                 "per-shape FETCH_SIZE / WRITE_SIZE readings of cacti_amd/gemm_traffic.json, "
+                                 "taken on this build of the kernels") if traffic is not None else
+                                "no counter readings for this build of the GEMM kernels (cacti_amd/gemm_traffic.json "
+                                "was taken on another)"}
     out = {
         "metric": "fwd+bwd tokens/sec, 3B-shaped fp16 step, 1 GPU", "value": tokens_s,
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -514,6 +508,29 @@ def run_adjoints(args):
             "roofline": {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["achieved_GBs"],
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": dom["frac_of_8TBs"], "traffic": None},
             "cpu_baseline": cpu, "kernels": res}
+
+
+def run_gemm_traffic(args):
+    """The dense products of the step, each launched gemm_traffic.LAUNCHES times in the order of
+    gemm_traffic.STEP_PRODUCTS and nothing else: the dispatch sequence `python -m cacti_amd.gemm_traffic`
+    expects in the counter files of a rocprofv3 --pmc run over this workload."""
+    import torch
+    from cacti_amd import gemm_traffic, ops
+    g = torch.Generator(device="cuda").manual_seed(0)
+    rn = lambda *s: (torch.randn(*s, device="cuda", generator=g) * 0.05).half()
+    n = 0
+    for label in gemm_traffic.STEP_PRODUCTS:
+        ta, tb, _, M, N, K = gemm_dims(label)
+        a = rn(K, M) if ta else rn(M, K)
+        b = rn(N, K) if tb else rn(K, N)
+        out = rn(M, N)
+        beta = 1.0 if label.endswith(",acc]") else 0.0
+        for _ in range(gemm_traffic.LAUNCHES):
+            ops.gemm(a, b, ta, tb, 1.0, beta, out)
+            n += 1
+        torch.cuda.synchronize()
+    return {"metric": "launches for the traffic counters", "value": n, "unit": "launches", "n_gpus": 1,
+            "config": {"workload": "every dense product of the step x %d" % gemm_traffic.LAUNCHES}}
 
 
 def run_gemm(args):
@@ -1034,7 +1051,8 @@ def main():
     ap.add_argument("--sustain", type=float, default=0.0, help="gemm workload: loop the largest product for this many seconds")
     ap.add_argument("--ckpt-format", choices=["safetensors", "pickle"], default="safetensors",
                     help="file format of the ingest workload's checkpoint")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "attention", "digests", "adamw", "ingest", "decode", "cycle"], default="step")
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "gemm-traffic", "attention", "digests", "adamw", "ingest",
+                                           "decode", "cycle"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path runs on ONE GPU (the reference is single-device and the step "
@@ -1058,6 +1076,8 @@ def main():
         out = run_cycle(args)
     elif args.workload == "attention":
         out = run_attention(args)
+    elif args.workload == "gemm-traffic":
+        out = run_gemm_traffic(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)
