@@ -1142,6 +1142,43 @@ int Ctx::compile()
                 for (CellPtr &a : log_[j].args)
                     if (a == x) a = y;
     }
+    // The mirror case: y := copy(x) where x is written again later (the gradient of the residual stream,
+    // which the next junction accumulates into) but every read of y comes before that write and nothing
+    // else writes y: the readers read x, which holds the same bytes until then, and the copy is dropped
+    // altogether (y never gets storage).
+    for (size_t i = 0; i < log_.size() && !no_forward; i++) {
+        const Entry &e = log_[i];
+        if (!(e.kind == E_APPLY && thunks_[e.thunk]->is_copy() && e.acc_mask == 0)) continue;
+        const CellPtr x = e.args[0], y = e.outs[0];
+        if (x == y || cells_[x].stable || cells_[y].stable || cells_[x].ty.bytes() != cells_[y].ty.bytes() ||
+            std::find(kept_.begin(), kept_.end(), y) != kept_.end())
+            continue;
+        size_t last_read_y = i, first_write_x = log_.size();
+        bool ok = true, x_read_later = false;
+        for (size_t j = i + 1; j < log_.size() && ok; j++) {
+            const Entry &f = log_[j];
+            if (f.kind == E_APPLY) {
+                if (std::find(f.outs.begin(), f.outs.end(), y) != f.outs.end()) ok = false;
+                if (std::find(f.args.begin(), f.args.end(), y) != f.args.end()) last_read_y = j;
+                if (std::find(f.args.begin(), f.args.end(), x) != f.args.end()) x_read_later = true;
+                if (first_write_x == log_.size() && std::find(f.outs.begin(), f.outs.end(), x) != f.outs.end())
+                    first_write_x = j;
+            } else if (f.kind == E_YIELD_SET) {
+                if (f.cell == y) ok = false;
+                if (f.cell == x && first_write_x == log_.size()) first_write_x = j;
+            }
+        }
+        // only where x lives on anyway (it is written or read again): otherwise the storage move below
+        // already makes the copy free
+        if (!ok || last_read_y == i || last_read_y >= first_write_x || !(x_read_later || first_write_x < log_.size()))
+            continue;
+        for (size_t j = i + 1; j <= last_read_y; j++)
+            if (log_[j].kind == E_APPLY)
+                for (CellPtr &a : log_[j].args)
+                    if (a == y) a = x;
+        log_.erase(log_.begin() + (std::ptrdiff_t)i);
+        i--;
+    }
     std::unordered_map<CellPtr, size_t> last;
     for (size_t i = 0; i < log_.size(); i++) {
         const Entry &e = log_[i];
