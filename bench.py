@@ -510,6 +510,44 @@ def run_adjoints(args):
             "cpu_baseline": cpu, "kernels": res}
 
 
+def run_mfma_power(args):
+    """The rate of MFMAs the device sustains over seconds (it is limited by power there, not by cycles): zero
+    against random operands, the 32 x 32 x 16 against the 16 x 16 x 32 product, with and without the fragment
+    reads of a 128 x 64 wave patch.  value = the sustained rate of the variant the large products of the step
+    are built on (16 x 16 x 32, 6 fragment reads per k step, random operands)."""
+    import torch
+    from cacti_amd import ffi
+    blocks, iters = 256, 100000
+    out = torch.empty(blocks * 512, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    per_launch = 262144.0 * iters * 8 * blocks
+    variants = [("32x32x16, zero operands, no LDS reads", 0, 0, 0), ("32x32x16, random operands, no LDS reads", 0, 0, 1),
+                ("32x32x16, random, 4 fragment reads per k step", 0, 4, 1), ("32x32x16, random, 6 fragment reads per k step", 0, 6, 1),
+                ("16x16x32, zero operands, no LDS reads", 1, 0, 0), ("16x16x32, random operands, no LDS reads", 1, 0, 1),
+                ("16x16x32, random, 4 fragment reads per k step", 1, 4, 1), ("16x16x32, random, 6 fragment reads per k step", 1, 6, 1),
+                ("32x32x16, random, 6 fragment reads per k step (again)", 0, 6, 1)]
+    res = []
+    for name, shape, reads, rnd in variants:
+        ffi.call("cacti_hip_mfma_probe", shape, reads, rnd, blocks, 2000, 1, out.data_ptr(), st)
+        torch.cuda.synchronize()
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < args.sustain_probe:
+            for _ in range(4):
+                ffi.call("cacti_hip_mfma_probe", shape, reads, rnd, blocks, iters, 12345 + n, out.data_ptr(), st)
+            torch.cuda.synchronize()
+            n += 4
+        dt = time.perf_counter() - t0
+        res.append({"variant": name, "tflops": per_launch * n / dt / 1e12, "seconds": dt})
+        log("%-56s %7.1f TFLOP/s sustained over %.1f s" % (name, res[-1]["tflops"], dt))
+    key = res[7]["tflops"]
+    return {"metric": "sustained MFMA rate, 16x16x32 f16 with fragment reads, random operands", "value": key,
+            "unit": "TFLOP/s", "n_gpus": 1, "higher_is_better": True, "dtype": "f16",
+            "config": {"workload": "MFMA-only probe, 256 workgroups of 8 waves, %.1f s per variant" % args.sustain_probe},
+            "roofline": {"bound": "mfma", "achieved": key, "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": key / PEAK_MFMA_F16_TFLOPS, "traffic": None},
+            "cpu_baseline": None, "variants": res}
+
+
 def run_gemm_traffic(args):
     """The dense products of the step, each launched gemm_traffic.LAUNCHES times in the order of
     gemm_traffic.STEP_PRODUCTS and nothing else: the dispatch sequence `python -m cacti_amd.gemm_traffic`
@@ -541,6 +579,8 @@ def run_gemm(args):
     g = torch.Generator(device="cuda").manual_seed(0)
 
     def rn(*shape, std=1.0):
+        if args.operands == "zeros":                # no toggling in the matrix pipes: the device keeps its full clock
+            return torch.zeros(*shape, device="cuda", dtype=torch.float16)
         return (torch.randn(*shape, device="cuda", generator=g) * std).half()
 
     res = []
@@ -1048,10 +1088,13 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-capped", action="store_true", help="skip the second run on a pool capped at 16 GiB")
     ap.add_argument("--yardstick", action="store_true", help="gemm workload: also time the vendor library on each shape")
+    ap.add_argument("--operands", choices=["randn", "zeros"], default="randn",
+                    help="gemm workload: operand values (zeros: the rate without the power limit that real operands meet)")
+    ap.add_argument("--sustain-probe", type=float, default=1.5, help="mfma-power workload: seconds per variant")
     ap.add_argument("--sustain", type=float, default=0.0, help="gemm workload: loop the largest product for this many seconds")
     ap.add_argument("--ckpt-format", choices=["safetensors", "pickle"], default="safetensors",
                     help="file format of the ingest workload's checkpoint")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "gemm-traffic", "attention", "digests", "adamw", "ingest",
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "gemm-traffic", "mfma-power", "attention", "digests", "adamw", "ingest",
                                            "decode", "cycle"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -1078,6 +1121,8 @@ def main():
         out = run_attention(args)
     elif args.workload == "gemm-traffic":
         out = run_gemm_traffic(args)
+    elif args.workload == "mfma-power":
+        out = run_mfma_power(args)
     else:
         out = run_gemm(args)
     print(json.dumps(out), flush=True)

@@ -74,6 +74,7 @@ SIGNATURES = {
     "cacti_hip_silu_gate_bwd": (ci, [i64, vp, vp, vp, vp, ci, vp, ci, vp]),
     "cacti_hip_causal_softmax_fwd": (ci, [i64, i64, vp, vp, vp]),
     "cacti_hip_causal_softmax_bwd": (ci, [i64, i64, vp, vp, vp, vp]),
+    "cacti_hip_mfma_probe": (ci, [ci, ci, ci, ci, i64, C.c_uint, vp, vp]),
     "cacti_hip_attention_set_exact": (ci, [ci]),
     "cacti_hip_attention_stats_bytes": (sz, [i64, i64]),
     "cacti_hip_attention_fwd": (ci, [i64, i64, i64, f32, vp, vp, vp, i64, vp, vp, vp]),

@@ -117,6 +117,15 @@ int cacti_hip_gemm_f16_strided_batched(int ta, int tb, int64_t nblk, int64_t M, 
                                        int64_t stride_b, float beta, void *C, int64_t ldc,
                                        int64_t stride_c, void *stream);
 
+/* Measurement aid with no counterpart in the reference (bench.py --workload mfma-power): one launch of
+ * `blocks` workgroups of 8 waves that do nothing but MFMAs on register fragments, `iters` (even) iterations
+ * of 262144 flops per wave.  shape 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_f32_16x16x32_f16; lds_reads: 0, 4
+ * or 6 fragments (16 bytes per lane each) refreshed from LDS per iteration; random_operands 0: all operands
+ * zero.  out: blocks * 512 floats of device memory.  Run for a second or more it shows the rate the device
+ * sustains under its power limit, which depends on all three. */
+int cacti_hip_mfma_probe(int shape, int lds_reads, int random_operands, int blocks, int64_t iters,
+                         unsigned seed, void *out, void *stream);
+
 /* Pointer-array batch, the shape of cublasGemmBatchedEx (cacti_gpu_cu_ffi/src/lib.rs:793-885):
  * nblk products of one shape, block z on A[z], B[z], C[z] (host arrays of device pointers, read
  * before the call returns).  With every operand 16-byte aligned up to four products share a launch,
