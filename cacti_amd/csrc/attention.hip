@@ -37,10 +37,17 @@
 // zero-padded); 16-byte chunk c of row r sits at chunk c ^ g(r), g(r) = 2 (r & 3) | ((r >> 2) & 1) |
 // 8 ((r >> 3) & 1): the 16-byte operand reads of 16 consecutive rows then cover all 16 bank groups,
 // and the 4 consecutive rows of a transposing read fall on 4 different pairs of them.
+//
+// How a K / V (Q / dO) tile gets there: straight from memory by global_load_lds_dwordx4 where the tensors
+// allow it (16-byte aligned, see DmaTileMap: every head addressed from the 16-byte boundary at or below
+// its start), else through registers (FastTileLoader, TileLoader8).  Measured at 32 heads x 2048 x 100:
+// forward 108.7 -> 92.9 us, adjoint 235.5 -> 209.8 us, 48 vector registers fewer per kernel.
 #include "common.h"
 #include "softmax_math.h"
 
+#include <algorithm>
 #include <atomic>
+#include <initializer_list>
 #include <type_traits>
 
 using namespace cacti;
@@ -102,10 +109,8 @@ __device__ __forceinline__ half8_t as_h8(uint2 lo, uint2 hi)
     return f;
 }
 
-// The K / V (Q / dO) tiles go from device memory through registers into LDS.  (Loading straight into LDS
-// with global_load_lds_dword -- dword granularity because the heads of a [S, H, 100] tensor start on
-// 8-byte, not 16-byte, boundaries -- was measured slower: 2.5 times the memory instructions, forward
-// 126 -> 153 us.)
+// The K / V (Q / dO) tiles through registers into LDS: the path for tensors whose tiles cannot be loaded
+// straight into LDS (DmaTileMap further down).
 
 // 16 bytes from device memory at an address that is only 8-byte aligned (the heads of a [S, H, 100]
 // tensor start every 200 bytes): one global_load_dwordx4, which needs dword alignment only
@@ -131,7 +136,7 @@ struct FastTileMap {
     int r0, gcol;
     int64_t ld;
     bool colok, tail, narrow;                            // narrow: a head of 4 columns, one 8-byte piece per row
-    __device__ __forceinline__ FastTileMap(int64_t ld_, int Dh)
+    __device__ __forceinline__ FastTileMap(int64_t ld_, int Dh, int)
     {
         const int t = threadIdx.x & (kNT - 1), pc = t & 15;
         r0 = t >> 4;
@@ -162,7 +167,7 @@ struct FastTileLoader {
     uint4 v[NP];
     int rows;                                            // rows of the tile inside the tensor (uniform)
     // src = &X[row0][head column 0]; rows_left = S - row0 >= 1
-    __device__ __forceinline__ void load(const FastTileMap &m, gptr_t src, int rows_left)
+    __device__ __forceinline__ void load(const FastTileMap &m, gptr_t src, int rows_left, unsigned char *)
     {
         rows = __builtin_amdgcn_readfirstlane(min(rows_left, kTileRows));
         if (m.narrow) {
@@ -220,7 +225,7 @@ struct TileMap8 {
     int r0, gcol;
     int64_t ld;
     bool colok;
-    __device__ __forceinline__ TileMap8(int64_t ld_, int Dh)
+    __device__ __forceinline__ TileMap8(int64_t ld_, int Dh, int)
     {
         const int t = threadIdx.x & (kNT - 1), pc = t & 31;
         r0 = t >> 5;
@@ -236,7 +241,7 @@ struct TileLoader8 {
     static constexpr int NP = kTileRows * 32 / kNT;      // 8-byte pieces per lane
     uint2 v[NP];
     int rows;
-    __device__ __forceinline__ void load(const TileMap8 &m, gptr_t src, int rows_left)
+    __device__ __forceinline__ void load(const TileMap8 &m, gptr_t src, int rows_left, unsigned char *)
     {
         rows = __builtin_amdgcn_readfirstlane(min(rows_left, kTileRows));
         if (rows == kTileRows) {
@@ -265,18 +270,89 @@ struct TileLoader8 {
     }
 };
 
+// Tiles straight into LDS (global_load_lds_dwordx4: the 16 bytes of lane l land at LDS address M0 + 16 l; no
+// staging registers, no LDS store instructions, no selects).  The load wants 16-byte aligned addresses and the
+// heads of a [S, H, Dh] tensor with Dh % 8 = 4 start on 8-byte boundaries every other head, so a head is
+// addressed from the 16-byte boundary at or below its start: a *window* of ceil((Dh + shift) / 8) chunks that
+// begins shift = (h Dh) % 8 elements (0 or 4) before the head.  Everything a kernel holds per head -- LDS tiles,
+// the fragments of the fixed operand, accumulator columns -- is in window positions, column d of the head at
+// position d + shift; the positions outside the head hold the neighbouring heads' elements in the tiles and
+// zeros in the fixed operand's fragments, so they add nothing to a product over the head dimension, and output
+// columns there are not stored.  (What that costs: a non-finite value in the 4 elements next to a head makes
+// that head's result non-finite too, where the reference keeps it to the neighbour until the output projection
+// mixes the heads.)  One instruction of a wave fills 4 tile rows; the chunk swizzle g(r) is applied on the
+// global side (the lane at chunk position p of row r fetches window chunk p ^ g(r)), lanes whose chunk lies
+// beyond the window stay out of the instruction, and those positions keep the zeros the kernel wrote at its
+// start.  The compiler neither counts these loads nor knows that they write LDS: the kernels wait for them
+// (vmcnt) before the barrier that publishes a tile.
+struct DmaTileMap {
+    uint32_t voff, slot;
+    int r0;
+    int64_t ld;
+    bool act;
+    __device__ __forceinline__ DmaTileMap(int64_t ld_, int Dh, int shift)
+    {
+        const int t = threadIdx.x & (kNT - 1), pc = t & 15;
+        r0 = t >> 4;
+        ld = ld_;
+        const int c = pc ^ gsw(r0);                      // g(r0 + 16 it) = g(r0)
+        act = c * 8 < Dh + shift;
+        voff = (uint32_t)((r0 * ld_ + c * 8) * 2);
+        slot = (uint32_t)(r0 * kRowB + pc * 16);
+    }
+};
+__device__ __forceinline__ void dma16(uint32_t lds, uint32_t voff, gptr_t base)
+{
+    const uint32_t m0 = __builtin_amdgcn_readfirstlane(lds);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(m0), "v"(voff), "s"(base) : "memory");
+}
+struct DmaTileLoader {
+    // src = the window's first element in the tile's first row; rows beyond the tensor are zeroed by the lanes
+    // that would have fetched them
+    __device__ __forceinline__ void load(const DmaTileMap &m, gptr_t src, int rows_left, unsigned char *tile) const
+    {
+        const int rows = __builtin_amdgcn_readfirstlane(min(rows_left, kTileRows));
+        const uint32_t wave = (uint32_t)(uintptr_t)tile + ((threadIdx.x & (kNT - 1)) >> 6) * 4 * kRowB;
+        if (rows == kTileRows) {
+            if (m.act) {
+#pragma unroll
+                for (int it = 0; it < 4; it++) dma16(wave + it * 16 * kRowB, m.voff, src + (int64_t)(16 * it) * m.ld);
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                if (m.r0 + 16 * it < rows) {
+                    if (m.act) dma16(wave + it * 16 * kRowB, m.voff, src + (int64_t)(16 * it) * m.ld);
+                } else {
+                    *reinterpret_cast<uint4 *>(tile + m.slot + it * 16 * kRowB) = make_uint4(0, 0, 0, 0);
+                }
+            }
+        }
+    }
+    __device__ __forceinline__ void store(const DmaTileMap &, unsigned char *) const {}
+};
+
+// the barrier that publishes the tiles just loaded (and retires the ones just read)
+template <bool DMA>
+__device__ __forceinline__ void tile_sync()
+{
+    if (DMA) __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));          // vmcnt(0) alone
+    __syncthreads();
+}
+
 // The fixed operand of a lane: row `row` of a [S, H, Dh] tensor as KS fragments (k step ks: the 8
-// halves at d = 16 ks + 8 lh ..), zero beyond Dh and for rows beyond S
+// halves at positions 16 ks + 8 lh .., position = column + shift), zero outside the head and for rows beyond S
 template <int KS>
-__device__ __forceinline__ void load_frags(half8_t (&f)[KS], gptr_t X, int64_t ld, int row, int S, int Dh, int lh)
+__device__ __forceinline__ void load_frags(half8_t (&f)[KS], gptr_t X, int64_t ld, int row, int S, int Dh, int lh,
+                                           int shift = 0)
 {
     const bool rok = row < S;
     gptr_t xr = X + (int64_t)min(row, S - 1) * ld;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-        const int d0 = 16 * ks + 8 * lh;
-        const bool ok0 = rok && d0 < Dh, ok1 = rok && d0 + 4 < Dh;
-        const uint2 a = gload8(xr + min(d0, Dh - 4));
+        const int d0 = 16 * ks + 8 * lh - shift;          // the head's column at the fragment's first position
+        const bool ok0 = rok && d0 >= 0 && d0 < Dh, ok1 = rok && d0 + 4 < Dh;
+        const uint2 a = gload8(xr + max(min(d0, Dh - 4), 0));
         const uint2 b = gload8(xr + min(d0 + 4, Dh - 4));
         f[ks] = as_h8(make_uint2(ok0 ? a.x : 0u, ok0 ? a.y : 0u), make_uint2(ok1 ? b.x : 0u, ok1 ? b.y : 0u));
     }
@@ -460,7 +536,7 @@ __device__ __forceinline__ void merge_partials(float16_t (&acc)[DT], unsigned ch
 // ---------------------------------------------------------------------------------------------
 // Workgroups take the tiles in descending order of their key count; a CU holds one workgroup at a
 // time (LDS), so the dispatcher hands the next tile to whichever CU is done first.
-template <int KS, int DT, bool FAST>
+template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
@@ -475,29 +551,32 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
     const int64_t ld = p.ld;
     const int nqt = (S + kBM - 1) / kBM;
     const int h = blockIdx.x % p.H, qt = nqt - 1 - blockIdx.x / p.H;
-    gptr_t Q = gp(p.q) + (int64_t)h * Dh, K = gp(p.k) + (int64_t)h * Dh, V = gp(p.v) + (int64_t)h * Dh;
+    const int shift = DMA ? (int)(((int64_t)h * Dh) & 7) : 0;          // the head's first column in its window
+    gptr_t Q = gp(p.q) + (int64_t)h * Dh, K = gp(p.k) + (int64_t)h * Dh - shift, V = gp(p.v) + (int64_t)h * Dh - shift;
     {
         const int i0 = qt * kBM, r0 = i0 + wid * 32, myrow = r0 + l32;
 
         half8_t qf[KS];
-        load_frags<KS>(qf, Q, ld, myrow, S, Dh, lh);
+        load_frags<KS>(qf, Q, ld, myrow, S, Dh, lh, shift);
 
         const int kend = min(i0 + kBM, S);                 // keys [0, kend) are visible to the tile
         const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
-        const FastTileMap tm(ld, Dh);
-        FastTileLoader tk, tv;
+        typedef typename std::conditional<DMA, DmaTileMap, FastTileMap>::type Map;
+        typedef typename std::conditional<DMA, DmaTileLoader, FastTileLoader>::type Loader;
+        const Map tm(ld, Dh, shift);
+        Loader tk, tv;
 
         // ---- pass 1: row maximum and sum; each lane over its half of the keys of its group's tiles
         float m_run = -INFINITY, l_run = 0.f;
         if (g < njt) {
-            tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+            tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
             tk.store(tm, Ks);
         }
-        __syncthreads();
+        tile_sync<DMA>();
         for (int it = 0; it < niter; it++) {
             const int jt = 2 * it + g, cur = it & 1;
             const bool nxt = jt + 2 < njt;
-            if (nxt) tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
+            if (nxt) tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Ks + (cur ^ 1) * kTileB);
             if (jt < njt) {
 #pragma unroll
                 for (int kt = 0; kt < 2; kt++) {
@@ -557,7 +636,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                 }
             }
             if (nxt) tk.store(tm, Ks + (cur ^ 1) * kTileB);
-            __syncthreads();
+            tile_sync<DMA>();
         }
         float m, l;
         {
@@ -593,18 +672,18 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
         if (g < njt) {
-            tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows);
-            tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+            tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
+            tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
             tk.store(tm, Ks);
             tv.store(tm, Vs);
         }
-        __syncthreads();
+        tile_sync<DMA>();
         for (int it = 0; it < niter; it++) {
             const int jt = 2 * it + g, cur = it & 1;
             const bool nxt = jt + 2 < njt;
             if (nxt) {
-                tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
-                tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
+                tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Ks + (cur ^ 1) * kTileB);
+                tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Vs + (cur ^ 1) * kTileB);
             }
             if (jt < njt) {
 #pragma unroll
@@ -643,7 +722,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                 tk.store(tm, Ks + (cur ^ 1) * kTileB);
                 tv.store(tm, Vs + (cur ^ 1) * kTileB);
             }
-            __syncthreads();
+            tile_sync<DMA>();
         }
         merge_partials<DT>(oacc, smem + kGroupLds, g, tig);
         if (g == 0 && myrow < S) {
@@ -652,8 +731,8 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const int d0 = 32 * dt + 8 * q + 4 * lh;
-                    if (d0 < Dh)
+                    const int d0 = 32 * dt + 8 * q + 4 * lh - shift;
+                    if (d0 >= 0 && d0 < Dh)
                         store_row4(orow + d0, oacc[dt][4 * q], oacc[dt][4 * q + 1], oacc[dt][4 * q + 2],
                                    oacc[dt][4 * q + 3], 1.0f, 0);
                 }
@@ -665,7 +744,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 // dQ: queries fixed, loop over the key tiles at or before them, work split as in the forward kernel.
 // Pass 0 forms sigma = sum_j P' f32(dP16); pass 1 dS16 and dQ.  Leaves y = 1 / l and sigma per row for
 // the dK / dV kernel.
-template <int KS, int DT, bool FAST>
+template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
@@ -680,13 +759,14 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
     const int nqt = (S + kBM - 1) / kBM;
     const int h = blockIdx.x % p.H, qt = nqt - 1 - blockIdx.x / p.H;
     const int64_t hoff = (int64_t)h * Dh;
-    gptr_t K = gp(p.k) + hoff, V = gp(p.v) + hoff;
+    const int shift = DMA ? (int)(hoff & 7) : 0;                        // the head's first column in its window
+    gptr_t K = gp(p.k) + hoff - shift, V = gp(p.v) + hoff - shift;
     {
         const int i0 = qt * kBM, r0 = i0 + wid * 32, myrow = r0 + l32;
 
         half8_t qf[KS], gf[KS];
-        load_frags<KS>(qf, gp(p.q) + hoff, ld, myrow, S, Dh, lh);
-        load_frags<KS>(gf, gp(p.dO) + hoff, ld, myrow, S, Dh, lh);
+        load_frags<KS>(qf, gp(p.q) + hoff, ld, myrow, S, Dh, lh, shift);
+        load_frags<KS>(gf, gp(p.dO) + hoff, ld, myrow, S, Dh, lh, shift);
         float m = ((gfptr_t)p.m)[(int64_t)h * S + min(myrow, S - 1)];
         float l = ((gfptr_t)p.l)[(int64_t)h * S + min(myrow, S - 1)];
         float sig = 0.f;
@@ -699,25 +779,27 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 
         const int kend = min(i0 + kBM, S);
         const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
-        const TileMap8 tm(ld, Dh);
-        TileLoader8 tk, tv;
+        typedef typename std::conditional<DMA, DmaTileMap, TileMap8>::type Map;
+        typedef typename std::conditional<DMA, DmaTileLoader, TileLoader8>::type Loader;
+        const Map tm(ld, Dh, shift);
+        Loader tk, tv;
         float16_t dacc[DT];
         auto run_pass = [&](auto pass_c) __attribute__((always_inline)) {
             constexpr int PASS = decltype(pass_c)::value;
             float part = 0.f;
             if (g < njt) {
-                tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows);
-                tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows);
+                tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
+                tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
                 tk.store(tm, Ks);
                 tv.store(tm, Vs);
             }
-            __syncthreads();
+            tile_sync<DMA>();
             for (int it = 0; it < niter; it++) {
                 const int jt = 2 * it + g, cur = it & 1;
                 const bool nxt = jt + 2 < njt;
                 if (nxt) {
-                    tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
-                    tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows);
+                    tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Ks + (cur ^ 1) * kTileB);
+                    tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Vs + (cur ^ 1) * kTileB);
                 }
                 if (jt < njt) {
 #pragma unroll
@@ -775,7 +857,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
                     tk.store(tm, Ks + (cur ^ 1) * kTileB);
                     tv.store(tm, Vs + (cur ^ 1) * kTileB);
                 }
-                __syncthreads();
+                tile_sync<DMA>();
             }
             return part;
         };
@@ -793,7 +875,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
         }
         if (short_sigma) {
             half8_t of[KS];
-            load_frags<KS>(of, gp(p.o) + hoff, ld, myrow, S, Dh, lh);
+            load_frags<KS>(of, gp(p.o) + hoff, ld, myrow, S, Dh, lh, shift);
             float part = 0.f;
 #pragma unroll
             for (int ks = 0; ks < KS; ks++)
@@ -823,8 +905,8 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const int d0 = 32 * dt + 8 * q + 4 * lh;
-                    if (d0 < Dh)
+                    const int d0 = 32 * dt + 8 * q + 4 * lh - shift;
+                    if (d0 >= 0 && d0 < Dh)
                         store_row4(drow + d0, dacc[dt][4 * q], dacc[dt][4 * q + 1], dacc[dt][4 * q + 2],
                                    dacc[dt][4 * q + 3], p.alpha, p.acc_dq);
                 }
@@ -835,7 +917,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 // ---------------------------------------------------------------------------------------------
 // dK, dV: keys fixed (128 per workgroup of 4 waves, a lane owns one), loop over the query tiles at or
 // after them; the key tiles with the most queries first.
-template <int KS, int DT, bool FAST>
+template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
@@ -849,7 +931,8 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
     const int64_t ld = p.ld;
     const int h = blockIdx.x % p.H, pr = blockIdx.x / p.H;
     const int64_t hoff = (int64_t)h * Dh;
-    gptr_t Q = gp(p.q) + hoff, G = gp(p.dO) + hoff;
+    const int shift = DMA ? (int)(hoff & 7) : 0;                        // the head's first column in its window
+    gptr_t Q = gp(p.q) + hoff - shift, G = gp(p.dO) + hoff - shift;
     // the four per-row statistics of a 64-query tile: lane t of wave w fetches array w, row t
     gfptr_t stat_src = (gfptr_t)(wid == 0 ? p.m : wid == 1 ? p.l : wid == 2 ? p.y : p.sig) + (int64_t)h * S;
     const float stat_pad = (wid == 1 || wid == 2) ? 1.f : 0.f;
@@ -859,8 +942,8 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
         const int c00 = kt_ * kBM, c0 = c00 + wid * 32, mykey = c0 + l32;
 
         half8_t kf[KS], vf[KS];
-        load_frags<KS>(kf, gp(p.k) + hoff, ld, mykey, S, Dh, lh);
-        load_frags<KS>(vf, gp(p.v) + hoff, ld, mykey, S, Dh, lh);
+        load_frags<KS>(kf, gp(p.k) + hoff, ld, mykey, S, Dh, lh, shift);
+        load_frags<KS>(vf, gp(p.v) + hoff, ld, mykey, S, Dh, lh, shift);
 
         float16_t kacc[DT], vacc[DT];
 #pragma unroll
@@ -871,26 +954,28 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 vacc[dt][r] = 0.f;
             }
         const int iq0 = c00 / kTileRows, niq = (S + kTileRows - 1) / kTileRows;
-        const FastTileMap tm(ld, Dh);
-        FastTileLoader tq, tg;
+        typedef typename std::conditional<DMA, DmaTileMap, FastTileMap>::type Map;
+        typedef typename std::conditional<DMA, DmaTileLoader, FastTileLoader>::type Loader;
+        const Map tm(ld, Dh, shift);
+        Loader tq, tg;
         float st;
         auto load_stat = [&](int iq) __attribute__((always_inline)) {
             const int row = iq * kTileRows + lane;
             const float t = stat_src[row < S ? row : S - 1];
             st = row < S ? t : stat_pad;          // rows beyond S are masked; the pad only has to be finite
         };
-        tq.load(tm, Q + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows);
-        tg.load(tm, G + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows);
+        tq.load(tm, Q + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows, Qs);
+        tg.load(tm, G + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows, Gs);
         load_stat(iq0);
         tq.store(tm, Qs);
         tg.store(tm, Gs);
         St[wid * 64 + lane] = st;
-        __syncthreads();
+        tile_sync<DMA>();
         for (int iq = iq0; iq < niq; iq++) {
             const int cur = (iq - iq0) & 1;
             if (iq + 1 < niq) {
-                tq.load(tm, Q + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows);
-                tg.load(tm, G + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows);
+                tq.load(tm, Q + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows, Qs + (cur ^ 1) * kTileB);
+                tg.load(tm, G + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows, Gs + (cur ^ 1) * kTileB);
                 load_stat(iq + 1);
             }
             const float *stc = St + cur * 256;
@@ -944,7 +1029,7 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 tg.store(tm, Gs + (cur ^ 1) * kTileB);
                 St[(cur ^ 1) * 256 + wid * 64 + lane] = st;
             }
-            __syncthreads();
+            tile_sync<DMA>();
         }
         if (mykey < S) {
             half_t *krow = p.dk + (int64_t)mykey * ld + hoff, *vrow = p.dv + (int64_t)mykey * ld + hoff;
@@ -952,8 +1037,8 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const int d0 = 32 * dt + 8 * q + 4 * lh;
-                    if (d0 < Dh) {
+                    const int d0 = 32 * dt + 8 * q + 4 * lh - shift;
+                    if (d0 >= 0 && d0 < Dh) {
                         store_row4(vrow + d0, vacc[dt][4 * q], vacc[dt][4 * q + 1], vacc[dt][4 * q + 2],
                                    vacc[dt][4 * q + 3], 1.0f, p.acc_dv);
                         store_row4(krow + d0, kacc[dt][4 * q], kacc[dt][4 * q + 1], kacc[dt][4 * q + 2],
@@ -973,44 +1058,78 @@ int set_smem(K kern, size_t bytes)
     return 0;
 }
 
-// Which arithmetic the kernels are built with (AttnMath).  Measured at 32 heads x 2048 x 100 on MI355X, in a
-// hot loop: forward 93 us / adjoint 232 us with the fast form, 123 / 305 us with the exact one; the two
+// Which arithmetic the kernels are launched with (AttnMath).  Measured at 32 heads x 2048 x 100 on MI355X, in a
+// hot loop with the register loaders: forward 93 us / adjoint 232 us with the fast form, 123 / 305 us with the exact one; the two
 // differ by 3e-5 .. 4e-5 relative L2 in O, dQ, dK, dV, and O, dQ, dK, dV of the fast form agree with
 // the CPU restatement of the reference to 4.9e-5 .. 7.1e-5.
-constexpr bool kFastMath = true;
 std::atomic<int> g_exact{0};             // cacti_hip_attention_set_exact: launch the exactly rounded forms
 
-template <int KS, int DT, bool FAST = kFastMath>
+template <int KS, int DT, bool FAST, bool DMA>
 int launch_fwd(const AttnArgs &p, hipStream_t st)
 {
     static DeviceOnce ready;
     if (!ready.fresh()) {
-        int rc = set_smem(attn_fwd_kernel<KS, DT, FAST>, kQmSmem);
+        int rc = set_smem(attn_fwd_kernel<KS, DT, FAST, DMA>, kQmSmem);
         if (rc) return rc;
         ready.mark();
     }
     const int nqt = (p.S + kBM - 1) / kBM;
-    hipLaunchKernelGGL((attn_fwd_kernel<KS, DT, FAST>), dim3((unsigned)(nqt * p.H)), dim3(kNT2), kQmSmem, st, p);
+    hipLaunchKernelGGL((attn_fwd_kernel<KS, DT, FAST, DMA>), dim3((unsigned)(nqt * p.H)), dim3(kNT2), kQmSmem, st, p);
     return launch_status("attention_fwd");
 }
 
-template <int KS, int DT, bool FAST = kFastMath>
+template <int KS, int DT, bool FAST, bool DMA>
 int launch_bwd(const AttnArgs &p, hipStream_t st)
 {
     static DeviceOnce ready;
     if (!ready.fresh()) {
-        int rc = set_smem(attn_bwd_dq_kernel<KS, DT, FAST>, kQmSmem);
+        int rc = set_smem(attn_bwd_dq_kernel<KS, DT, FAST, DMA>, kQmSmem);
         if (rc) return rc;
-        if ((rc = set_smem(attn_bwd_dkv_kernel<KS, DT, FAST>, kDkvSmem))) return rc;
+        if ((rc = set_smem(attn_bwd_dkv_kernel<KS, DT, FAST, DMA>, kDkvSmem))) return rc;
         ready.mark();
     }
     const int nqt = (p.S + kBM - 1) / kBM;
-    hipLaunchKernelGGL((attn_bwd_dq_kernel<KS, DT, FAST>), dim3((unsigned)(nqt * p.H)), dim3(kNT2), kQmSmem, st, p);
+    hipLaunchKernelGGL((attn_bwd_dq_kernel<KS, DT, FAST, DMA>), dim3((unsigned)(nqt * p.H)), dim3(kNT2), kQmSmem, st, p);
     int rc = launch_status("attention_bwd_dq");
     if (rc) return rc;
-    hipLaunchKernelGGL((attn_bwd_dkv_kernel<KS, DT, FAST>), dim3((unsigned)(nqt * p.H)), dim3(kNT), kDkvSmem, st, p);
+    hipLaunchKernelGGL((attn_bwd_dkv_kernel<KS, DT, FAST, DMA>), dim3((unsigned)(nqt * p.H)), dim3(kNT), kDkvSmem, st, p);
     return launch_status("attention_bwd_dkv");
 }
+
+// Whether the tiles of these tensors can be loaded straight into LDS: 16-byte aligned tensors and rows, and
+// every head's window (from the 16-byte boundary at or below its start, whole 16-byte chunks) inside its row.
+// *span = the window positions a head can occupy (Dh + the largest shift).
+bool direct_tiles(int64_t H, int64_t Dh, int64_t ld, std::initializer_list<const void *> tensors, int64_t *span)
+{
+    *span = Dh;
+    if (ld % 8 != 0) return false;
+    for (const void *t : tensors)
+        if (!aligned(t, 16)) return false;
+    int64_t most = 0;
+    for (int64_t h = 0; h < H; h++) {
+        const int64_t shift = (h * Dh) & 7, start = h * Dh - shift, chunks = (Dh + shift + 7) / 8;
+        if (start + 8 * chunks > ld || 8 * chunks > kDP) return false;
+        most = std::max(most, Dh + shift);
+    }
+    *span = most;
+    return true;
+}
+
+// the instantiation by the window span (16 KS and 32 DT positions must cover it), the arithmetic and the loader
+template <template <int, int, bool, bool> class L>
+int dispatch(int64_t span, bool exact, bool dma, const AttnArgs &p, hipStream_t st)
+{
+    auto by_size = [&](auto fast_c, auto dma_c) {
+        constexpr bool F = decltype(fast_c)::value, D = decltype(dma_c)::value;
+        if (span <= 64) return L<4, 2, F, D>::run(p, st);
+        if (span <= 112) return L<7, 4, F, D>::run(p, st);
+        return L<8, 4, F, D>::run(p, st);
+    };
+    if (exact) return dma ? by_size(std::false_type{}, std::true_type{}) : by_size(std::false_type{}, std::false_type{});
+    return dma ? by_size(std::true_type{}, std::true_type{}) : by_size(std::true_type{}, std::false_type{});
+}
+template <int KS, int DT, bool F, bool D> struct Fwd { static int run(const AttnArgs &p, hipStream_t st) { return launch_fwd<KS, DT, F, D>(p, st); } };
+template <int KS, int DT, bool F, bool D> struct Bwd { static int run(const AttnArgs &p, hipStream_t st) { return launch_bwd<KS, DT, F, D>(p, st); } };
 
 int check_shape(const char *who, int64_t S, int64_t H, int64_t Dh, int64_t ld)
 {
@@ -1060,14 +1179,9 @@ CACTI_API int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float al
     p.m = (float *)stats;
     p.l = p.m + S * H;
     hipStream_t st = (hipStream_t)stream;
-    if (g_exact.load(std::memory_order_relaxed)) {
-        if (Dh <= 64) return launch_fwd<4, 2, false>(p, st);
-        if (Dh <= 112) return launch_fwd<7, 4, false>(p, st);
-        return launch_fwd<8, 4, false>(p, st);
-    }
-    if (Dh <= 64) return launch_fwd<4, 2>(p, st);
-    if (Dh <= 112) return launch_fwd<7, 4>(p, st);
-    return launch_fwd<8, 4>(p, st);
+    int64_t span;
+    const bool dma = direct_tiles(H, Dh, ld, {k, v}, &span);
+    return dispatch<Fwd>(span, g_exact.load(std::memory_order_relaxed) != 0, dma, p, st);
 }
 
 CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float alpha, const void *q, const void *k,
@@ -1097,12 +1211,7 @@ CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float al
     p.y = (float *)workspace;
     p.sig = p.y + S * H;
     hipStream_t st = (hipStream_t)stream;
-    if (g_exact.load(std::memory_order_relaxed)) {
-        if (Dh <= 64) return launch_bwd<4, 2, false>(p, st);
-        if (Dh <= 112) return launch_bwd<7, 4, false>(p, st);
-        return launch_bwd<8, 4, false>(p, st);
-    }
-    if (Dh <= 64) return launch_bwd<4, 2>(p, st);
-    if (Dh <= 112) return launch_bwd<7, 4>(p, st);
-    return launch_bwd<8, 4>(p, st);
+    int64_t span;
+    const bool dma = direct_tiles(H, Dh, ld, {q, k, v, dO}, &span);
+    return dispatch<Bwd>(span, g_exact.load(std::memory_order_relaxed) != 0, dma, p, st);
 }
