@@ -386,6 +386,48 @@ __device__ __forceinline__ float16_t prod_direct(const unsigned char *tile, int 
     return acc;
 }
 
+// The same product with independent vector arithmetic issued between its MFMAs (the softmax arithmetic of the
+// score tile before this one): a chain of dependent MFMAs leaves the wave nothing to issue for 32 cycles per
+// link, and the two waves of a SIMD do not fill each other's gaps reliably.  `work(integral_constant<i>)` is
+// piece i of NP pieces of that arithmetic: piece 0 covers the latency of the fragment reads, the others follow
+// the MFMAs in equal shares; scheduling barriers keep the order as written.
+template <int KS, int NP, class F>
+__device__ __forceinline__ float16_t prod_direct_with(const unsigned char *tile, int row_base, const half8_t (&yf)[KS],
+                                                      int l32, int lh, F &&work)
+{
+    float16_t acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    const int row = row_base + l32;
+    const unsigned char *rp = tile + row * kRowB;
+    const int g = gsw(row);
+    half8_t x[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) x[ks] = *reinterpret_cast<const half8_t *>(rp + (((2 * ks + lh) ^ g) << 4));
+    __builtin_amdgcn_sched_barrier(0);
+    work(std::integral_constant<int, 0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    auto link = [&](auto ks_c) __attribute__((always_inline)) {
+        constexpr int ks = decltype(ks_c)::value;
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[ks], yf[ks], acc, 0, 0, 0);
+        constexpr int p0 = 1 + ks * (NP - 1) / KS, p1 = 1 + (ks + 1) * (NP - 1) / KS;
+        if constexpr (p0 < p1) work(std::integral_constant<int, p0>{});
+        if constexpr (p0 + 1 < p1) work(std::integral_constant<int, p0 + 1>{});
+        static_assert(p1 - p0 <= 2, "at most two pieces per MFMA");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    link(std::integral_constant<int, 0>{});
+    link(std::integral_constant<int, 1>{});
+    link(std::integral_constant<int, 2>{});
+    link(std::integral_constant<int, 3>{});
+    if constexpr (KS > 4) link(std::integral_constant<int, 4>{});
+    if constexpr (KS > 5) link(std::integral_constant<int, 5>{});
+    if constexpr (KS > 6) link(std::integral_constant<int, 6>{});
+    if constexpr (KS > 7) link(std::integral_constant<int, 7>{});
+    static_assert(KS >= 4 && KS <= 8, "4 to 8 k steps");
+    return acc;
+}
+
 // acc[dt] += sum over the 32 tile rows k_base .. k_base + 31 of X[row][32 dt + .] Y[.][row]: X by
 // transposing reads of the LDS tile, Y = the packed registers y0 (rows 0..15) and y1 (rows 16..31) in
 // the row permutation described at the top
@@ -481,6 +523,17 @@ __device__ __forceinline__ void round16(half_t (&h)[16], const float16_t &a)
         h[e + 1] = t[1];
     }
 }
+// two f32 -> packed f16 (round to nearest even) as one v_cvt_pk_f16_f32, said so: left to itself the compiler
+// may fold the multiplication in front into two v_fma_mixlo / mixhi_f16, which cost 4.4 ns each per SIMD where
+// a multiplication costs 2.1 and this instruction 2.8 for the pair
+__device__ __forceinline__ half2v_t cvt_pk(float a, float b)
+{
+    uint32_t u;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(u) : "v"(a), "v"(b));
+    half2v_t h;
+    __builtin_memcpy(&h, &u, 4);
+    return h;
+}
 // the exponent offset of a row's probabilities: m log2(e) + log2(l)
 __device__ __forceinline__ float prob_shift(float m, float l)
 {
@@ -573,7 +626,63 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             tk.store(tm, Ks);
         }
         tile_sync<DMA>();
-        for (int it = 0; it < niter; it++) {
+        int it0 = 0;
+        if constexpr (FAST) {
+            // The key tiles wholly below the diagonal for every wave (iterations 0 .. qt - 1 of both groups) as a
+            // pipeline: the products of a score tile run while the statistics of the tile before it are updated.
+            // The same operations on the same values in the same order as the general loop below.
+            // in 8 pieces: round the scores; their maximum; 4 x (4 exponentials and their sum); the running pair
+            half2v_t sp[8];
+            float m_new, cexp, sum;
+            auto stat_piece = [&](const float16_t &acc, auto i_c) __attribute__((always_inline)) {
+                constexpr int i = decltype(i_c)::value;
+                if constexpr (i == 0) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++)
+                        sp[e] = __builtin_convertvector(float2v_t{p.alpha * acc[2 * e], p.alpha * acc[2 * e + 1]}, half2v_t);
+                } else if constexpr (i == 1) {
+                    half2v_t mx = sp[0];
+#pragma unroll
+                    for (int e = 1; e < 8; e++) mx = __builtin_elementwise_max(mx, sp[e]);
+                    m_new = fmaxf(m_run, (float)__builtin_fmaxf16(mx[0], mx[1]));
+                    cexp = m_new * kLog2e;
+                    sum = 0.f;
+                } else if constexpr (i < 6) {
+#pragma unroll
+                    for (int e = 4 * (i - 2); e < 4 * (i - 1); e++) sum += exp2_mix(sp[e >> 1][e & 1], cexp);
+                } else if constexpr (i == 6) {
+                    l_run = ((m_run == -INFINITY) ? 0.f : l_run * M::ex(m_run, m_new)) + sum;
+                    m_run = m_new;
+                }
+            };
+            auto stat_full = [&](const float16_t &acc) __attribute__((always_inline)) {
+                stat_piece(acc, std::integral_constant<int, 0>{});
+                stat_piece(acc, std::integral_constant<int, 1>{});
+                stat_piece(acc, std::integral_constant<int, 2>{});
+                stat_piece(acc, std::integral_constant<int, 3>{});
+                stat_piece(acc, std::integral_constant<int, 4>{});
+                stat_piece(acc, std::integral_constant<int, 5>{});
+                stat_piece(acc, std::integral_constant<int, 6>{});
+            };
+            const int nfull = min(qt, niter);
+            if (nfull > 0) {
+                float16_t accp = prod_direct<KS>(Ks, 0, qf, l32, lh);
+                for (int it = 0; it < nfull; it++) {
+                    const int jt = 2 * it + g, cur = it & 1;
+                    const bool nxt = jt + 2 < njt;
+                    if (nxt) tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Ks + (cur ^ 1) * kTileB);
+                    accp = prod_direct_with<KS, 7>(Ks + cur * kTileB, 32, qf, l32, lh, [&](auto i_c) { stat_piece(accp, i_c); });
+                    if (nxt) tk.store(tm, Ks + (cur ^ 1) * kTileB);
+                    tile_sync<DMA>();
+                    if (it + 1 < nfull)
+                        accp = prod_direct_with<KS, 7>(Ks + (cur ^ 1) * kTileB, 0, qf, l32, lh, [&](auto i_c) { stat_piece(accp, i_c); });
+                    else
+                        stat_full(accp);
+                }
+                it0 = nfull;
+            }
+        }
+        for (int it = it0; it < niter; it++) {
             const int jt = 2 * it + g, cur = it & 1;
             const bool nxt = jt + 2 < njt;
             if (nxt) tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Ks + (cur ^ 1) * kTileB);
@@ -917,14 +1026,25 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 // ---------------------------------------------------------------------------------------------
 // dK, dV: keys fixed (128 per workgroup of 4 waves, a lane owns one), loop over the query tiles at or
 // after them; the key tiles with the most queries first.
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+constexpr int kDkvBufs = 3;                      // tile buffers per tensor (Q, dO) and sets of row statistics
+
 template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    zero_lds(smem, 4 * kTileB);                    // the pad columns of the tile buffers: zero from here on
-    unsigned char *Qs = smem, *Gs = smem + 2 * kTileB;
-    float *St = reinterpret_cast<float *>(smem + 4 * kTileB);          // [2][4][64]: m, l, y, sigma of the tile's rows
+    zero_lds(smem, 2 * kDkvBufs * kTileB);         // the pad columns of the tile buffers: zero from here on
+    unsigned char *Qs = smem, *Gs = smem + kDkvBufs * kTileB;
+    float *St = reinterpret_cast<float *>(smem + 2 * kDkvBufs * kTileB);   // [3][4][64]: m, l, y, sigma of a tile's rows
     const int lane = threadIdx.x & 63, wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l32 = lane & 31,
               lh = lane >> 5;
     const int S = p.S, Dh = p.Dh;
@@ -964,72 +1084,250 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
             const float t = stat_src[row < S ? row : S - 1];
             st = row < S ? t : stat_pad;          // rows beyond S are masked; the pad only has to be finite
         };
-        tq.load(tm, Q + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows, Qs);
-        tg.load(tm, G + (int64_t)iq0 * kTileRows * ld, S - iq0 * kTileRows, Gs);
-        load_stat(iq0);
-        tq.store(tm, Qs);
-        tg.store(tm, Gs);
-        St[wid * 64 + lane] = st;
-        tile_sync<DMA>();
-        for (int iq = iq0; iq < niq; iq++) {
-            const int cur = (iq - iq0) & 1;
-            if (iq + 1 < niq) {
-                tq.load(tm, Q + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows, Qs + (cur ^ 1) * kTileB);
-                tg.load(tm, G + (int64_t)(iq + 1) * kTileRows * ld, S - (iq + 1) * kTileRows, Gs + (cur ^ 1) * kTileB);
-                load_stat(iq + 1);
+        auto buf_of = [&](int iq) __attribute__((always_inline)) { return (iq - iq0) % kDkvBufs; };
+        auto fetch = [&](int iq) __attribute__((always_inline)) {        // tile iq on its way (registers or LDS)
+            const int bf = buf_of(iq);
+            tq.load(tm, Q + (int64_t)iq * kTileRows * ld, S - iq * kTileRows, Qs + bf * kTileB);
+            tg.load(tm, G + (int64_t)iq * kTileRows * ld, S - iq * kTileRows, Gs + bf * kTileB);
+            if constexpr (DMA) {
+                // the statistics the same way (rows beyond S: the last row's, finite like the pad), so that no
+                // register load stands between these loads and the point where the kernel waits for them
+                const int row = min(iq * kTileRows + lane, S - 1);
+                const uint32_t m0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(St + bf * 256 + wid * 64));
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                             :
+                             : "s"(m0), "v"((uint32_t)row * 4u), "s"(stat_src)
+                             : "memory");
+            } else {
+                load_stat(iq);
             }
-            const float *stc = St + cur * 256;
+        };
+        auto land = [&](int iq) __attribute__((always_inline)) {         // ... into LDS, with its statistics
+            const int bf = buf_of(iq);
+            tq.store(tm, Qs + bf * kTileB);
+            tg.store(tm, Gs + bf * kTileB);
+            if constexpr (!DMA) St[bf * 256 + wid * 64 + lane] = st;
+        };
+        // one 32-query block of a tile, its three stages one after the other
+        auto block = [&](int iq, int qb) __attribute__((always_inline)) {
+            const int bf = buf_of(iq);
+            const float *stc = St + bf * 256;
+            const int qb0 = iq * kTileRows + 32 * qb;
+            if (qb0 + 31 < c0 || qb0 >= S) return;        // every query of the block is before every key of the wave
+            const float16_t sacc = prod_direct<KS, false>(Qs + bf * kTileB, 32 * qb, kf, l32, lh);
+            const float16_t pacc = prod_direct<KS, false>(Gs + bf * kTileB, 32 * qb, vf, l32, lh);
+            const bool full = qb0 >= c0 + 31 && qb0 + 32 <= S;
+            float pe[16], de[16];
+            half_t dph[16];
+            if constexpr (FAST) round16(dph, pacc);
+            auto elems = [&](auto full_c) __attribute__((always_inline)) {
+                constexpr bool FULL = decltype(full_c)::value;
 #pragma unroll
-            for (int qb = 0; qb < 2; qb++) {
-                const int qb0 = iq * kTileRows + 32 * qb;
-                if (qb0 + 31 < c0 || qb0 >= S) continue;     // every query of the block is before every key of the wave
-                const float16_t sacc = prod_direct<KS, false>(Qs + cur * kTileB, 32 * qb, kf, l32, lh);
-                const float16_t pacc = prod_direct<KS, false>(Gs + cur * kTileB, 32 * qb, vf, l32, lh);
-                const bool full = qb0 >= c0 + 31 && qb0 + 32 <= S;
-                float pe[16], de[16];
-                half_t dph[16];
-                if constexpr (FAST) round16(dph, pacc);
-                auto elems = [&](auto full_c) __attribute__((always_inline)) {
-                    constexpr bool FULL = decltype(full_c)::value;
+                for (int q = 0; q < 4; q++) {
+                    const int qi = 32 * qb + 8 * q + 4 * lh;
+                    float4_t mm, ll;
+                    if constexpr (!FAST) {
+                        mm = *reinterpret_cast<const float4_t *>(stc + 0 * 64 + qi);
+                        ll = *reinterpret_cast<const float4_t *>(stc + 1 * 64 + qi);
+                    }
+                    const float4_t yy = *reinterpret_cast<const float4_t *>(stc + 2 * 64 + qi);
+                    const float4_t sg = *reinterpret_cast<const float4_t *>(stc + 3 * 64 + qi);
 #pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        const int qi = 32 * qb + 8 * q + 4 * lh;
-                        float4_t mm, ll;
-                        if constexpr (!FAST) {
-                            mm = *reinterpret_cast<const float4_t *>(stc + 0 * 64 + qi);
-                            ll = *reinterpret_cast<const float4_t *>(stc + 1 * 64 + qi);
+                    for (int r = 0; r < 4; r++) {
+                        const int e = 4 * q + r, query = iq * kTileRows + qi + r;
+                        float pr_, ds;
+                        if constexpr (FAST) {                 // yy holds the exponent offset of the row
+                            pr_ = exp2_mix(f2h(p.alpha * sacc[e]), yy[r]);
+                            ds = __builtin_fmaf((float)dph[e], pr_, -(sg[r] * pr_));
+                        } else {
+                            pr_ = M::prob(rnd16(p.alpha * sacc[e]), mm[r], ll[r], yy[r]);
+                            const float tt = pr_ * rnd16(pacc[e]);
+                            ds = tt - sg[r] * pr_;
                         }
-                        const float4_t yy = *reinterpret_cast<const float4_t *>(stc + 2 * 64 + qi);
-                        const float4_t sg = *reinterpret_cast<const float4_t *>(stc + 3 * 64 + qi);
+                        const bool live = FULL || (query >= mykey && query < S);
+                        pe[e] = live ? pr_ : 0.f;
+                        de[e] = live ? ds : 0.f;
+                    }
+                }
+            };
+            if (full) elems(std::true_type{});           // no masks on blocks wholly past the diagonal
+            else elems(std::false_type{});
+            prod_tr<DT>(vacc, Gs + bf * kTileB, 32 * qb, pack8(pe), pack8(pe + 8), lane);
+            prod_tr<DT>(kacc, Qs + bf * kTileB, 32 * qb, pack8(de), pack8(de + 8), lane);
+        };
+        // tiles [a, b), tile a in LDS and published
+        auto run_tiles = [&](int a, int b) __attribute__((always_inline)) {
+            for (int iq = a; iq < b; iq++) {
+                if (iq + 1 < niq) fetch(iq + 1);
+                block(iq, 0);
+                block(iq, 1);
+                if (iq + 1 < niq) land(iq + 1);
+                tile_sync<DMA>();
+            }
+        };
+
+        fetch(iq0);
+        land(iq0);
+        tile_sync<DMA>();
+        // The tiles that hold the diagonal (two: 128 keys) and a ragged last tile run block by block.  The tiles
+        // between them, whose 32-query blocks are whole and past the diagonal for every wave, run as a pipeline
+        // (fast arithmetic, tiles loaded straight into LDS): while the vector unit forms P and dS of block b, the
+        // matrix unit forms S and dP of block b + 1 and adds block b - 1 to dV and dK.  A wave has its SIMD to
+        // itself here, so nothing else would fill the one unit while the other works.
+        const int iqB = iq0 + 2, iqE = S / kTileRows;
+        if (FAST && DMA && iqE > iqB) {
+            run_tiles(iq0, iqB);
+            if constexpr (FAST && DMA) {
+                const int a4 = (lane >> 2) & 3, b4 = lane & 3, n16 = (lane >> 4) & 1;
+                const int colb = 16 * n16 + 4 * b4;
+                // blocks alternate between two register sets: SP = the S and dP accumulators (formed in one
+                // step, consumed in the next), PD = the packed P and dS of a block (likewise)
+                float16_t SPs[2], SPp[2];
+                half8_t PD[2][4];                               // P rows 0..15, P rows 16..31, dS likewise
+                half8_t xs[KS], xp[KS], xt[2][DT];
+                float4_t yy, sg;
+                // S1: the fragment reads of k step t of block (tile q1 / g1, qb1)
+                auto x_read = [&](auto t_c, const unsigned char *q1, const unsigned char *g1, int qb1) __attribute__((always_inline)) {
+                    constexpr int t = decltype(t_c)::value;
+                    const int row = 32 * qb1 + l32, o = row * kRowB + (((2 * t + lh) ^ gsw(row)) << 4);
+                    xs[t] = *reinterpret_cast<const half8_t *>(q1 + o);
+                    xp[t] = *reinterpret_cast<const half8_t *>(g1 + o);
+                };
+                // S3: the 2 DT transposing reads of group g = 2 which + kk (which: 0 dV from the dO tile, 1 dK from
+                // the Q tile; kk: rows 0..15 or 16..31 of the block), and MFMA j = g DT + dt
+                auto t_read = [&](auto g_c, const unsigned char *q3, const unsigned char *g3, int qb3) __attribute__((always_inline)) {
+                    constexpr int g = decltype(g_c)::value, which = g >> 1, kk = g & 1;
+                    const unsigned char *tile = which ? q3 : g3;
+                    const int r1 = 32 * qb3 + 16 * kk + 4 * lh + a4, r2 = r1 + 8;
+                    const unsigned char *p1 = tile + r1 * kRowB + ((colb & 4) << 1);
+                    const unsigned char *p2 = tile + r2 * kRowB + ((colb & 4) << 1);
+                    const int g1_ = gsw(r1), g2_ = gsw(r2);
 #pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            const int e = 4 * q + r, query = iq * kTileRows + qi + r;
-                            float pr_, ds;
-                            if constexpr (FAST) {                 // yy holds the exponent offset of the row
-                                pr_ = exp2_mix(f2h(p.alpha * sacc[e]), yy[r]);
-                                ds = __builtin_fmaf((float)dph[e], pr_, -(sg[r] * pr_));
-                            } else {
-                                pr_ = M::prob(rnd16(p.alpha * sacc[e]), mm[r], ll[r], yy[r]);
-                                const float tt = pr_ * rnd16(pacc[e]);
-                                ds = tt - sg[r] * pr_;
-                            }
-                            const bool live = FULL || (query >= mykey && query < S);
-                            pe[e] = live ? pr_ : 0.f;
-                            de[e] = live ? ds : 0.f;
-                        }
+                    for (int dt = 0; dt < DT; dt++) {
+                        const int c = (32 * dt + colb) >> 3;
+                        xt[g & 1][dt] = as_h8(lds_read_tr(p1 + ((c ^ g1_) << 4)), lds_read_tr(p2 + ((c ^ g2_) << 4)));
                     }
                 };
-                if (full) elems(std::true_type{});           // no masks on blocks wholly past the diagonal
-                else elems(std::false_type{});
-                prod_tr<DT>(vacc, Gs + cur * kTileB, 32 * qb, pack8(pe), pack8(pe + 8), lane);
-                prod_tr<DT>(kacc, Qs + cur * kTileB, 32 * qb, pack8(de), pack8(de + 8), lane);
+                constexpr int NQ = 32, NM = 2 * KS + 4 * DT;     // quarter pieces of S2 and MFMAs of a step
+                // One step.  PAR: parity of the block in S2 (its qb).  S1 forms block (tile1, qb = PAR ^ 1) into
+                // set PAR ^ 1, S2 turns set PAR into PD[PAR], S3 adds PD[PAR ^ 1] (block tile3, qb = PAR ^ 1).
+                auto step = [&](auto par_c, auto has1_c, auto has3_c, int buf1, int buf2, int buf3) __attribute__((always_inline)) {
+                    constexpr int PAR = decltype(par_c)::value, OTH = PAR ^ 1;
+                    constexpr bool HAS1 = decltype(has1_c)::value, HAS3 = decltype(has3_c)::value;
+                    const unsigned char *q1 = Qs + buf1 * kTileB, *g1 = Gs + buf1 * kTileB;
+                    const unsigned char *q3 = Qs + buf3 * kTileB, *g3 = Gs + buf3 * kTileB;
+                    const float *stc = St + buf2 * 256;
+                    const float16_t &sC = SPs[PAR], &pC = SPp[PAR];
+                    // S2 in 32 quarter pieces (8 pairs of elements x 4): the roundings S16 and dP16; the exponentials;
+                    // dS; the packed results.  The same operations on the same values as the block-by-block form.
+                    half2v_t s2, d2;
+                    float pr2[2], ds2[2];
+                    auto valu = [&](auto j_c) __attribute__((always_inline)) {
+                        constexpr int j = decltype(j_c)::value, pc = j >> 2, qr = j & 3, q = pc >> 1, hf = pc & 1, e0 = 4 * q + 2 * hf;
+                        if constexpr (qr == 0) {
+                            if constexpr (hf == 0) {
+                                const int qi = 32 * PAR + 8 * q + 4 * lh;
+                                yy = *reinterpret_cast<const float4_t *>(stc + 2 * 64 + qi);
+                                sg = *reinterpret_cast<const float4_t *>(stc + 3 * 64 + qi);
+                            }
+                            s2 = cvt_pk(p.alpha * sC[e0], p.alpha * sC[e0 + 1]);
+                            d2 = cvt_pk(pC[e0], pC[e0 + 1]);
+                        } else if constexpr (qr == 1) {
+                            pr2[0] = exp2_mix(s2[0], yy[2 * hf]);
+                            pr2[1] = exp2_mix(s2[1], yy[2 * hf + 1]);
+                        } else if constexpr (qr == 2) {
+                            ds2[0] = __builtin_fmaf((float)d2[0], pr2[0], -(sg[2 * hf] * pr2[0]));
+                            ds2[1] = __builtin_fmaf((float)d2[1], pr2[1], -(sg[2 * hf + 1] * pr2[1]));
+                        } else {
+                            half2v_t pn = cvt_pk(pr2[0], pr2[1]), dn = cvt_pk(ds2[0], ds2[1]);
+                            // the values are used a step later; without a use here the compiler moves the whole piece there
+                            asm volatile("" : "+v"(pn), "+v"(dn));
+                            PD[PAR][e0 >> 3][e0 & 7] = pn[0];
+                            PD[PAR][e0 >> 3][(e0 & 7) + 1] = pn[1];
+                            PD[PAR][2 + (e0 >> 3)][e0 & 7] = dn[0];
+                            PD[PAR][2 + (e0 >> 3)][(e0 & 7) + 1] = dn[1];
+                        }
+                    };
+                    if constexpr (HAS1) {
+                        x_read(std::integral_constant<int, 0>{}, q1, g1, OTH);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            SPs[OTH][r] = 0.f;
+                            SPp[OTH][r] = 0.f;
+                        }
+                    }
+                    if constexpr (HAS3) {
+                        t_read(std::integral_constant<int, 0>{}, q3, g3, OTH);
+                        t_read(std::integral_constant<int, 1>{}, q3, g3, OTH);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    // One MFMA, its share of the 32 quarter pieces, a scheduling barrier: the matrix unit takes 32
+                    // cycles per MFMA and a second one issued behind it stalls the wave -- and with it the vector
+                    // instructions behind that -- until the first is through.
+                    auto slot_end = [&](auto m_c) __attribute__((always_inline)) {
+                        constexpr int m = decltype(m_c)::value;
+                        __builtin_amdgcn_sched_barrier(0);
+                        static_for<m * NQ / NM, (m + 1) * NQ / NM>([&](auto j_c) __attribute__((always_inline)) { valu(j_c); });
+                        __builtin_amdgcn_sched_barrier(0);
+                    };
+                    static_for<0, KS>([&](auto t_c) __attribute__((always_inline)) {
+                        constexpr int t = decltype(t_c)::value;
+                        constexpr int j0 = t * 4 * DT / KS, j1 = (t + 1) * 4 * DT / KS, m0 = 2 * t + j0;
+                        if constexpr (HAS1) SPs[OTH] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xs[t], kf[t], SPs[OTH], 0, 0, 0);
+                        slot_end(std::integral_constant<int, m0>{});
+                        if constexpr (HAS1) {
+                            SPp[OTH] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xp[t], vf[t], SPp[OTH], 0, 0, 0);
+                            if constexpr (t + 1 < KS) x_read(std::integral_constant<int, t + 1>{}, q1, g1, OTH);
+                        }
+                        slot_end(std::integral_constant<int, m0 + 1>{});
+                        static_for<j0, j1>([&](auto j_c) __attribute__((always_inline)) {
+                            constexpr int j = decltype(j_c)::value, g = j / DT, dt = j % DT, which = g >> 1, kk = g & 1;
+                            if constexpr (HAS3) {
+                                const half8_t y = PD[OTH][2 * which + kk];
+                                if constexpr (which)
+                                    kacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xt[g & 1][dt], y, kacc[dt], 0, 0, 0);
+                                else
+                                    vacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xt[g & 1][dt], y, vacc[dt], 0, 0, 0);
+                                // the reads of group g + 2 (two register sets, g & 1) once the last MFMA of group g is out
+                                if constexpr (dt == DT - 1 && g + 2 < 4) t_read(std::integral_constant<int, g + 2>{}, q3, g3, OTH);
+                            }
+                            slot_end(std::integral_constant<int, 2 * t + 2 + j>{});
+                        });
+                    });
+                };
+                const std::integral_constant<int, 0> par0;
+                const std::integral_constant<int, 1> par1;
+                // the first and the last step stand outside the loop, so that the loop holds one form of each step
+                // A tile is fetched two steps before its first use and waited for one step before it (the barrier
+                // after every second step), so the latency of the loads has a whole step to pass.
+                if (iqB + 1 < niq) fetch(iqB + 1);
+                SPs[0] = prod_direct<KS, false>(Qs + buf_of(iqB) * kTileB, 0, kf, l32, lh);
+                SPp[0] = prod_direct<KS, false>(Gs + buf_of(iqB) * kTileB, 0, vf, l32, lh);
+                {
+                    const int bc = buf_of(iqB);
+                    step(par0, std::true_type{}, std::false_type{}, bc, bc, bc);       // S1 (iqB, 1), S2 (iqB, 0)
+                    tile_sync<DMA>();
+                }
+                for (int iq = iqB; iq + 1 < iqE; iq++) {
+                    const int bc = buf_of(iq), bn = buf_of(iq + 1);
+                    // step (iq, 1): S1 (iq + 1, 0), S2 (iq, 1), S3 (iq, 0); tile iq + 2 takes the buffer of tile
+                    // iq - 1, which the step before was the last to read
+                    if (iq + 2 < niq) fetch(iq + 2);
+                    step(par1, std::true_type{}, std::true_type{}, bn, bc, bc);
+                    // step (iq + 1, 0): S1 (iq + 1, 1), S2 (iq + 1, 0), S3 (iq, 1)
+                    step(par0, std::true_type{}, std::true_type{}, bn, bn, bc);
+                    tile_sync<DMA>();
+                }
+                {
+                    const int bc = buf_of(iqE - 1);
+                    step(par1, std::false_type{}, std::true_type{}, bc, bc, bc);       // S2 (iqE - 1, 1), S3 (iqE - 1, 0)
+                }
+                prod_tr<DT>(vacc, Gs + buf_of(iqE - 1) * kTileB, 32, PD[1][0], PD[1][1], lane);
+                prod_tr<DT>(kacc, Qs + buf_of(iqE - 1) * kTileB, 32, PD[1][2], PD[1][3], lane);
             }
-            if (iq + 1 < niq) {
-                tq.store(tm, Qs + (cur ^ 1) * kTileB);
-                tg.store(tm, Gs + (cur ^ 1) * kTileB);
-                St[(cur ^ 1) * 256 + wid * 64 + lane] = st;
-            }
-            tile_sync<DMA>();
+            run_tiles(iqE, niq);
+        } else {
+            run_tiles(iq0, niq);
         }
         if (mykey < S) {
             half_t *krow = p.dk + (int64_t)mykey * ld + hoff, *vrow = p.dv + (int64_t)mykey * ld + hoff;
@@ -1049,7 +1347,7 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
     }
 }
 
-constexpr size_t kDkvSmem = 4 * kTileB + 2 * 4 * 64 * sizeof(float);
+constexpr size_t kDkvSmem = 2 * kDkvBufs * kTileB + kDkvBufs * 4 * 64 * sizeof(float);
 
 template <class K>
 int set_smem(K kern, size_t bytes)

@@ -23,31 +23,41 @@ that may be widened at will is no bar.  Three more conditions keep it honest:
 """
 import itertools
 
+import numpy as np
+
 from tests.util import max_rel, rel_l2
 
 ABS_CAP = 2e-3
 OUTLIER_SLACK = 1.02
+LOSS_ABS_CAP = 2e-4
 
 
 class Envelope(dict):
-    """{tensor: (rel_l2, max_rel)} plus the runs it was measured from (restatement -> {tensor: grad})."""
+    """{tensor: (rel_l2, max_rel)} plus the runs it was measured from (restatement -> {tensor: grad}) and the
+    same pair of figures for the per-position loss."""
     runs = None
+    loss = None
+    loss_to_default = None
 
 
 def order_envelope(oracle, cfg, flat, tok, lm_tok, scale, grad_cached=None, count=None):
     """Returns (runs: restatement -> {tensor: grad}, env: Envelope); count: only the first `count`
     restatements (large shapes)."""
-    runs = {}
+    runs, losses = {}, {}
     try:
         for name in list(oracle.RESTATEMENTS)[:count]:
             oracle.set_restatement(name)
             out = oracle.llama_step(cfg, flat, tok, lm_tok, scale, grad_cached=grad_cached)
             runs[name] = oracle.split_params(cfg, out["grad"])
+            losses[name] = np.asarray(out["loss"], np.float64)
     finally:
         oracle.set_restatement("ascending")
     env = Envelope()
     env.runs = runs
     pairs = list(itertools.combinations(runs, 2))
+    env.loss = (max(rel_l2(losses[a], losses[b]) for a, b in pairs),
+                max(max_rel(losses[a], losses[b]) for a, b in pairs))
+    env.loss_to_default = {n: rel_l2(losses[n], losses["ascending"]) for n in losses if n != "ascending"}
     for t in runs["ascending"]:
         env[t] = (max(rel_l2(runs[a][t], runs[b][t]) for a, b in pairs),
                   max(max_rel(runs[a][t], runs[b][t]) for a, b in pairs))
@@ -104,3 +114,20 @@ def assert_inside_envelope(got, want, env, tag, verbose=True, abs_cap=ABS_CAP):
             "%s:%s the device is an outlier: mean distance %.3e to the restatements, theirs at most %.3e" % (
                 tag, t, dm, max(mean.values()))
     return worst
+
+
+def assert_loss_inside_envelope(loss, want, env, tag):
+    """The per-position loss of a composed run is the end of the same chain of f16-rounded products as the
+    gradients: at the 3B shapes the restatements' own losses are 0.9e-4 .. 1.4e-4 relative L2 from the default
+    one after a single layer.  So it is held to the largest distance between two restatements, and to the
+    absolute cap LOSS_ABS_CAP beside it; the loss thunk by itself is held to 1e-5 on the oracle's logits
+    (tests/test_gpu_full_shapes.py::test_lm_head_and_cross_entropy_full_shape, tests/test_gpu_teacher.py)."""
+    e2, em = rel_l2(loss, want), max_rel(loss, want)
+    f2, fm = env.loss
+    print("%s: loss rel_l2 %.3e  envelope %.3e  ratio %.2f   max_rel %.3e  envelope %.3e; restatements to the "
+          "default one: %s" % (tag, e2, f2, e2 / f2, em, fm,
+                               " ".join("%.2e" % v for v in env.loss_to_default.values())), flush=True)
+    assert e2 <= f2, "%s: loss rel_l2 %.3e outside the envelope %.3e" % (tag, e2, f2)
+    assert e2 <= LOSS_ABS_CAP, "%s: loss rel_l2 %.3e above the absolute cap %.1e" % (tag, e2, LOSS_ABS_CAP)
+    assert em <= max(fm, 1e-3), "%s: loss max_rel %.3e outside the envelope %.3e" % (tag, em, fm)
+    return e2
