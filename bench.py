@@ -571,6 +571,76 @@ def run_gemm_traffic(args):
             "config": {"workload": "every dense product of the step x %d" % gemm_traffic.LAUNCHES}}
 
 
+def run_gemm_step(args):
+    """The dense products of one 26-layer step in the step's order, back to back and nothing else, so that
+    the device sits in the thermal and power state of the step: time per pass and sustained TFLOP/s; with
+    --yardstick the same sequence through the vendor library (torch.matmul / addmm -> hipBLASLt) beside it,
+    a yardstick for what the device sustains on these shapes, no part of the product path."""
+    import torch
+    from cacti_amd import ops
+    S, D, F, V, L = 2048, 3200, 8640, 32000, 26
+    g = torch.Generator(device="cuda").manual_seed(0)
+    rn = lambda *s, std=1.0: (torch.randn(*s, device="cuda", generator=g) * std).half()
+    R = 3                                                   # operand sets in rotation
+    x_d, x_f = [rn(S, D) for _ in range(R)], [rn(S, F) for _ in range(R)]
+    w_dd, w_fd, w_df = [rn(D, D, std=0.02) for _ in range(R)], [rn(F, D, std=0.02) for _ in range(R)], \
+        [rn(D, F, std=0.02) for _ in range(R)]
+    o_d, o_f = torch.empty(S, D, device="cuda", dtype=torch.float16), torch.empty(S, F, device="cuda", dtype=torch.float16)
+    g_dd, g_fd, g_df = (torch.empty(*s, device="cuda", dtype=torch.float16) for s in ((D, D), (F, D), (D, F)))
+    x_v, w_vd, o_v, g_vd = rn(S, V, std=0.01), rn(V, D, std=0.02), torch.empty(S, V, device="cuda", dtype=torch.float16), \
+        torch.empty(V, D, device="cuda", dtype=torch.float16)
+    # (A, B, ta, tb, beta, out): the 21 products of a layer, then the 3 of the head
+    def layer(i):
+        a, f, wdd, wfd, wdf = x_d[i % R], x_f[i % R], w_dd[i % R], w_fd[i % R], w_df[i % R]
+        fwd = [(a, wdd, 0, 1, 0.0, o_d)] * 4 + [(a, wfd, 0, 1, 0.0, o_f)] * 2 + [(f, wdf, 0, 1, 0.0, o_d)]
+        bwd = [(a, wdf, 0, 0, 0.0, o_f), (a, f, 1, 0, 0.0, g_df),                        # down: dgrad, wgrad
+               (f, wfd, 0, 0, 0.0, o_d), (f, a, 1, 0, 0.0, g_fd), (f, wfd, 0, 0, 1.0, o_d), (f, a, 1, 0, 0.0, g_fd),
+               (a, wdd, 0, 0, 0.0, o_d), (a, a, 1, 0, 0.0, g_dd),                        # o
+               (a, wdd, 0, 0, 0.0, o_d), (a, a, 1, 0, 0.0, g_dd), (a, wdd, 0, 0, 1.0, o_d), (a, a, 1, 0, 0.0, g_dd),
+               (a, wdd, 0, 0, 1.0, o_d), (a, a, 1, 0, 0.0, g_dd)]
+        return fwd, bwd
+    head = [(x_d[0], w_vd, 0, 1, 0.0, o_v), (x_v, w_vd, 0, 0, 0.0, o_d), (x_v, x_d[0], 1, 0, 0.0, g_vd)]
+    seq = [c for i in range(L) for c in layer(i)[0]] + head[:1] + head[1:] + [c for i in range(L) for c in layer(i)[1]]
+    flops = 0.0
+    for a, b, ta, tb, beta, out in seq:
+        flops += 2.0 * out.shape[0] * out.shape[1] * (a.shape[0] if ta else a.shape[1])
+
+    def ours():
+        for a, b, ta, tb, beta, out in seq:
+            ops.gemm(a, b, bool(ta), bool(tb), 1.0, beta, out)
+
+    def library():
+        for a, b, ta, tb, beta, out in seq:
+            A_, B_ = (a.t() if ta else a), (b.t() if tb else b)
+            if beta:
+                torch.addmm(out, A_, B_, out=out)
+            else:
+                torch.matmul(A_, B_, out=out)
+
+    def timed(fn, passes):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(passes):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / passes
+
+    passes = max(args.steps, 3)
+    ms = timed(ours, passes)
+    log("%d dense products of a step back to back: %.2f ms per pass, %.0f TFLOP/s sustained" % (len(seq), ms, flops / ms / 1e9))
+    out = {"metric": "dense products of one step, back to back", "value": ms, "unit": "ms", "n_gpus": 1,
+           "higher_is_better": False, "dtype": "f16", "tflops": flops / ms / 1e9, "products": len(seq), "passes": passes,
+           "config": {"workload": "the %d dense products of the 26-layer 3B step in its order" % len(seq)}}
+    if args.yardstick:
+        yms = timed(library, passes)
+        log("the same through the vendor library:            %.2f ms per pass, %.0f TFLOP/s sustained" % (yms, flops / yms / 1e9))
+        out.update(library_ms=yms, library_tflops=flops / yms / 1e9)
+    return out
+
+
 def run_gemm(args):
     """Every GEMM shape of the step, standalone: TFLOP/s per shape."""
     import torch
@@ -1094,7 +1164,7 @@ def main():
     ap.add_argument("--sustain", type=float, default=0.0, help="gemm workload: loop the largest product for this many seconds")
     ap.add_argument("--ckpt-format", choices=["safetensors", "pickle"], default="safetensors",
                     help="file format of the ingest workload's checkpoint")
-    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "gemm-traffic", "mfma-power", "attention", "digests", "adamw", "ingest",
+    ap.add_argument("--workload", choices=["step", "adjoints", "gemm", "gemm-traffic", "gemm-step", "mfma-power", "attention", "digests", "adamw", "ingest",
                                            "decode", "cycle"], default="step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -1119,6 +1189,8 @@ def main():
         out = run_cycle(args)
     elif args.workload == "attention":
         out = run_attention(args)
+    elif args.workload == "gemm-step":
+        out = run_gemm_step(args)
     elif args.workload == "gemm-traffic":
         out = run_gemm_traffic(args)
     elif args.workload == "mfma-power":
