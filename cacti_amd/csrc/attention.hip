@@ -155,6 +155,17 @@ __device__ __forceinline__ void zero_lds(unsigned char *smem, int bytes)
     for (int o = threadIdx.x * 16; o < bytes; o += blockDim.x * 16) *reinterpret_cast<uint4 *>(smem + o) = make_uint4(0, 0, 0, 0);
     __syncthreads();
 }
+// The same for tiles that are loaded straight into LDS: only the chunks no load writes (window chunks nch .. 15 of
+// every row), without a barrier of its own -- the loads of the first tiles are already in flight when this runs
+// and touch none of these chunks; the barrier that publishes those tiles publishes the zeros.
+__device__ __forceinline__ void zero_pads(unsigned char *smem, int rows, int nch)
+{
+    const int npad = 16 - nch;
+    for (int i = threadIdx.x; i < rows * npad; i += blockDim.x) {
+        const int r = i / npad, c = nch + i % npad;
+        *reinterpret_cast<uint4 *>(smem + toff(r, c)) = make_uint4(0, 0, 0, 0);
+    }
+}
 
 // 64 rows x Dh of a [S, H, Dh] tensor -> registers -> LDS tile, by the 256 lanes of one wave group, with
 // the constants above (the forward and the dK / dV kernel; the dQ kernel has no registers to spare for
@@ -594,7 +605,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    zero_lds(smem, 2 * kGroupLds);                 // the pad columns of the tile buffers: zero from here on
+    if constexpr (!DMA) zero_lds(smem, 2 * kGroupLds);   // the pad columns of the tile buffers: zero from here on
     // wave-uniform values kept in scalar registers, so that the branches on them are scalar branches
     const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8), tig = threadIdx.x & (kNT - 1);
     unsigned char *Ks = smem + g * kGroupLds, *Vs = Ks + 2 * kTileB;
@@ -624,7 +635,10 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
         if (g < njt) {
             tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
             tk.store(tm, Ks);
+            // the V buffers idle through pass 1: the first V tile of pass 2 comes in now
+            if constexpr (DMA) tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
         }
+        if constexpr (DMA) zero_pads(smem, 2 * kGroupLds / kRowB, (Dh + shift + 7) >> 3);
         tile_sync<DMA>();
         int it0 = 0;
         if constexpr (FAST) {
@@ -747,6 +761,10 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             if (nxt) tk.store(tm, Ks + (cur ^ 1) * kTileB);
             tile_sync<DMA>();
         }
+        // pass 2 starts from the group's first K tile again: on its way while the statistics are merged
+        if constexpr (DMA) {
+            if (g < njt) tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
+        }
         float m, l;
         {
             // the four partial (maximum, sum) pairs of a row -- two lanes in each of two groups -- merged
@@ -780,7 +798,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
         for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
-        if (g < njt) {
+        if (!DMA && g < njt) {
             tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
             tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
             tk.store(tm, Ks);
@@ -858,7 +876,6 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    zero_lds(smem, 2 * kGroupLds);                 // the pad columns of the tile buffers: zero from here on
     const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8), tig = threadIdx.x & (kNT - 1);
     unsigned char *Ks = smem + g * kGroupLds, *Vs = Ks + 2 * kTileB;
     float *xs = reinterpret_cast<float *>(smem + kXsOff);
@@ -869,6 +886,9 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
     const int h = blockIdx.x % p.H, qt = nqt - 1 - blockIdx.x / p.H;
     const int64_t hoff = (int64_t)h * Dh;
     const int shift = DMA ? (int)(hoff & 7) : 0;                        // the head's first column in its window
+    // the pad columns of the tile buffers: zero from here on (published by the first pass's first barrier)
+    if constexpr (DMA) zero_pads(smem, 2 * kGroupLds / kRowB, (Dh + shift + 7) >> 3);
+    else zero_lds(smem, 2 * kGroupLds);
     gptr_t K = gp(p.k) + hoff - shift, V = gp(p.v) + hoff - shift;
     {
         const int i0 = qt * kBM, r0 = i0 + wid * 32, myrow = r0 + l32;
@@ -1042,7 +1062,6 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
 {
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    zero_lds(smem, 2 * kDkvBufs * kTileB);         // the pad columns of the tile buffers: zero from here on
     unsigned char *Qs = smem, *Gs = smem + kDkvBufs * kTileB;
     float *St = reinterpret_cast<float *>(smem + 2 * kDkvBufs * kTileB);   // [3][4][64]: m, l, y, sigma of a tile's rows
     const int lane = threadIdx.x & 63, wid = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), l32 = lane & 31,
@@ -1053,6 +1072,9 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
     const int64_t hoff = (int64_t)h * Dh;
     const int shift = DMA ? (int)(hoff & 7) : 0;                        // the head's first column in its window
     gptr_t Q = gp(p.q) + hoff - shift, G = gp(p.dO) + hoff - shift;
+    // the pad columns of the tile buffers: zero from here on (published by the first tile's barrier)
+    if constexpr (DMA) zero_pads(smem, 2 * kDkvBufs * kTileB / kRowB, (Dh + shift + 7) >> 3);
+    else zero_lds(smem, 2 * kDkvBufs * kTileB);
     // the four per-row statistics of a 64-query tile: lane t of wave w fetches array w, row t
     gfptr_t stat_src = (gfptr_t)(wid == 0 ? p.m : wid == 1 ? p.l : wid == 2 ? p.y : p.sig) + (int64_t)h * S;
     const float stat_pad = (wid == 1 || wid == 2) ? 1.f : 0.f;
