@@ -83,7 +83,13 @@ def gemm_traffic_bytes(label, table):
     return None if ent is None else float(ent["bytes"])
 
 
-GEMM_RE = re.compile(r"^(block_matmul|matmul)\[([NT])([NT]),(\d+)x(\d+)x(\d+)x(\d+)(,acc)?\]$")
+# "...]x3": three products of that shape staged as one thunk and launched together
+GEMM_RE = re.compile(r"^(block_matmul|matmul)\[([NT])([NT]),(\d+)x(\d+)x(\d+)x(\d+)(,acc)?\](?:x(\d+))?$")
+
+
+def gemm_group(label):
+    m = GEMM_RE.match(label)
+    return int(m.group(9) or 1) if m else 1
 
 
 def gemm_flops(label):
@@ -91,7 +97,7 @@ def gemm_flops(label):
     if not m:
         return None
     H, M, N, K = (int(m.group(i)) for i in (4, 5, 6, 7))
-    return 2.0 * H * M * N * K
+    return 2.0 * H * M * N * K * gemm_group(label)
 
 
 N_CUS = 256
@@ -158,6 +164,8 @@ def is_split(label):
     a second launch of 64 x 64 tiles): its event pair then brackets both, so it is left out of a
     single kernel's roofline sample."""
     ta, tb, H, M, N, K = gemm_dims(label)
+    if gemm_group(label) > 1:                              # a grouped thunk: never one launch of one product
+        return True
     if ta or H != 1 or M < 1024 or N < 1024 or K % 64:
         return False
     return plan_tokens_product(M, N)[1] < N

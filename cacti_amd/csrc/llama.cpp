@@ -26,6 +26,7 @@ struct cacti_llama {
     std::vector<CellPtr> params, grads;
     bool grads_written = false;                                 // a gradient cycle has been staged
     int attention_mode = 0;                                     // 0 fused thunk, 1 the chain of separate thunks
+    int group_products = 1;                                     // 0 none, 1 up + gate forward, 2 also q, k, v and the weight gradients
     std::vector<CellPtr> master, grad_avg, grad2_avg;           // f32 optimiser state (adamw_init)
     std::vector<std::string> names;
     CellPtr embed, head_norm, lm_head;
@@ -438,6 +439,13 @@ CACTI_API int cacti_llama_set_attention(cacti_llama *m, int mode)
     return 0;
 }
 
+CACTI_API int cacti_llama_set_product_groups(cacti_llama *m, int on)
+{
+    CACTI_REQUIRE(m && on >= 0 && on <= 2, CACTI_E_INVALID, "llama_set_product_groups: 0, 1 or 2");
+    m->group_products = on;
+    return 0;
+}
+
 CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
 {
     Ctx &c = m->ctx->c;
@@ -467,8 +475,18 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
         const LayerCells &w = m->layers[l];
         CellPtr pre, q, k, v, qr, kr, s16, p16, attn, o, post, up, gate, h, down;
         TRY(norm_of_stream(w.pre_norm, &pre));
-        TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.q}, &q));
-        TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
+        if (m->group_products >= 2) {
+            // the three projections of the normed input (llama.rs:478-497) as one thunk and one launch;
+            // values, and the order of the adjoint's accumulations, as with three matmul thunks
+            std::vector<CellPtr> po;
+            TRY(c.stage_apply(c.add_thunk(make_projections(3, true)), {pre, w.q, w.k, w.v}, &po));
+            q = po[0];
+            k = po[1];
+            v = po[2];
+        } else {
+            TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.q}, &q));
+            TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.k}, &k));
+        }
         {
             // symplectic_embed on the query and on the key (llama.rs:483, 490) as one two-output thunk:
             // one launch, the values and the order of the adjoint's accumulations as with two thunks
@@ -477,7 +495,7 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
             qr = ro[0];
             kr = ro[1];
         }
-        TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.v}, &v));
+        if (m->group_products < 2) TRY(ap(c, make_matmul(false, true, 1.f), {pre, w.v}, &v));
         if (m->attention_mode == 0) {
             // scores, mask, softmax and the product with v as one thunk: the [S, H, S] cells of
             // llama.rs:501-505 exist only tile by tile in registers
@@ -493,8 +511,15 @@ CACTI_API int cacti_llama_stage(cacti_llama *m, int want_prob, int want_grad)
         add_a = stream;                                       // x1 = stream + o
         add_b = o;
         TRY(norm_of_stream(w.post_norm, &post));
-        TRY(ap(c, make_matmul(false, true, 1.f), {post, w.up}, &up));
-        TRY(ap(c, make_matmul(false, true, 1.f), {post, w.gate}, &gate));
+        if (m->group_products >= 1) {
+            std::vector<CellPtr> po;
+            TRY(c.stage_apply(c.add_thunk(make_projections(2, m->group_products >= 2)), {post, w.up, w.gate}, &po));
+            up = po[0];
+            gate = po[1];
+        } else {
+            TRY(ap(c, make_matmul(false, true, 1.f), {post, w.up}, &up));
+            TRY(ap(c, make_matmul(false, true, 1.f), {post, w.gate}, &gate));
+        }
         TRY(ap(c, make_silu_gate(), {gate, up}, &h));
         TRY(ap(c, make_matmul(false, true, 1.f), {h, w.down}, &down));
         add_a = stream;                                       // x2 = x1 + down

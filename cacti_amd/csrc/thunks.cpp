@@ -309,6 +309,127 @@ struct MatMulSpec : ThunkSpec {
 };
 
 // ---------------------------------------------------------------------------
+// Several products of one shape that share an operand, as one thunk and one launch (a pointer-array batch,
+// cacti_hip_gemm_f16_batched: the shape of the reference's cublasGemmBatchedEx call,
+// cacti_gpu_cu_ffi/src/lib.rs:793-885).  The reference stages the query, key and value projections of a layer
+// (and the gate and up projections) as separate matmul thunks on the same input (src/librarium/llama.rs:
+// 478-497); each product here is computed by the same tiles in the same order as its own launch would, so the
+// results are those of the separate thunks bit for bit, and the adjoint stages what their adjoints would have
+// staged, in their order: the weight gradients (one grouped thunk), then the input gradients one after the other
+// (they accumulate into one cell: last product first, as the reverse sweep over separate thunks meets them).
+constexpr int kMaxGroup = 4;
+
+// dW_i = dy_i^T x: (dy_1 .. dy_n, x) -> (dW_1 .. dW_n)
+struct WgradNSpec : ThunkSpec {
+    int n;
+    explicit WgradNSpec(int n_) : n(n_) {}
+    const char *name() const override { return "matmul"; }
+    int arity() const override { return n + 1; }
+    int nout() const override { return n; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(n >= 2 && n <= kMaxGroup, "grouped weight gradients: 2 .. %d products", kMaxGroup);
+        for (int i = 0; i <= n; i++)
+            TY_REQUIRE(a[i].dtype == F16 && a[i].shape.size() == 2 && a[i].shape[0] == a[n].shape[0] &&
+                           (i == n || a[i] == a[0]),
+                       "grouped weight gradients: (dy f16 [S,N] x n, x f16 [S,K]) expected");
+        o.assign(n, CellType({a[0].shape[1], a[n].shape[1]}, F16));
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        const int64_t Sq = aty[0].shape[0], N = aty[0].shape[1], K = aty[n].shape[1];
+        const uint32_t all = (1u << n) - 1;
+        if ((acc & all) != 0 && (acc & all) != all) {          // mixed modes: one after the other
+            for (int i = 0; i < n; i++) {
+                const int rc = cacti_hip_gemm_f16(1, 0, N, K, Sq, 1.f, a[i], N, a[n], K, ((acc >> i) & 1) ? 1.f : 0.f,
+                                                  o[i], K, S(c));
+                if (rc) return rc;
+            }
+            return 0;
+        }
+        const void *A[kMaxGroup], *B[kMaxGroup];
+        void *C[kMaxGroup];
+        for (int i = 0; i < n; i++) {
+            A[i] = a[i];
+            B[i] = a[n];
+            C[i] = o[i];
+        }
+        return cacti_hip_gemm_f16_batched(1, 0, n, N, K, Sq, 1.f, A, N, B, K, (acc & 1) ? 1.f : 0.f, C, K, S(c));
+    }
+    std::string key(const std::vector<CellType> &aty, uint32_t acc) const override
+    {
+        char buf[128];
+        snprintf(buf, sizeof(buf), "matmul[TN,1x%lldx%lldx%lld%s]x%d", (long long)aty[0].shape[1],
+                 (long long)aty[n].shape[1], (long long)aty[0].shape[0], (acc & 1) ? ",acc" : "", n);
+        return buf;
+    }
+};
+
+// y_i = x W_i^T: (x, W_1 .. W_n) -> (y_1 .. y_n)
+struct ProjNSpec : ThunkSpec {
+    int n;
+    bool group_adj;                  // the weight gradients as one grouped thunk as well
+    explicit ProjNSpec(int n_, bool ga = true) : n(n_), group_adj(ga) {}
+    const char *name() const override { return "matmul"; }
+    int arity() const override { return n + 1; }
+    int nout() const override { return n; }
+    int out_ty(const std::vector<CellType> &a, std::vector<CellType> &o) const override
+    {
+        TY_REQUIRE(n >= 2 && n <= kMaxGroup, "grouped projections: 2 .. %d products", kMaxGroup);
+        for (int i = 0; i <= n; i++)
+            TY_REQUIRE(a[i].dtype == F16 && a[i].shape.size() == 2 && a[i].shape[1] == a[0].shape[1] &&
+                           (i == 0 || a[i] == a[1]),
+                       "grouped projections: (x f16 [S,K], W f16 [N,K] x n) expected");
+        o.assign(n, CellType({a[0].shape[0], a[1].shape[0]}, F16));
+        return 0;
+    }
+    int run(Ctx &c, const std::vector<CellType> &aty, void *const *a, const std::vector<CellType> &,
+            void *const *o, uint32_t acc, void *, size_t) const override
+    {
+        TY_REQUIRE(acc == 0, "grouped projections: accumulate mode not staged on this path");
+        const int64_t Sq = aty[0].shape[0], K = aty[0].shape[1], N = aty[1].shape[0];
+        const void *A[kMaxGroup], *B[kMaxGroup];
+        void *C[kMaxGroup];
+        for (int i = 0; i < n; i++) {
+            A[i] = a[0];
+            B[i] = a[1 + i];
+            C[i] = o[i];
+        }
+        return cacti_hip_gemm_f16_batched(0, 1, n, Sq, N, K, 1.f, A, K, B, K, 0.f, C, N, S(c));
+    }
+    std::string key(const std::vector<CellType> &aty, uint32_t) const override
+    {
+        char buf[128];
+        snprintf(buf, sizeof(buf), "matmul[NT,1x%lldx%lldx%lld]x%d", (long long)aty[0].shape[0],
+                 (long long)aty[1].shape[0], (long long)aty[0].shape[1], n);
+        return buf;
+    }
+    int pop_adj(Ctx &c, const Entry &e, const std::vector<CellPtr> &dy) const override
+    {
+        const CellPtr x = e.args[0];
+        bool all = group_adj;
+        for (int i = 0; i < n; i++) all = all && dy[i];
+        int rc;
+        if (all) {
+            std::vector<CellPtr> ws(e.args.begin() + 1, e.args.end()), in(dy.begin(), dy.begin() + n);
+            in.push_back(x);
+            if ((rc = c.adj_add(ws, std::unique_ptr<ThunkSpec>(new WgradNSpec(n)), in))) return rc;
+        }
+        for (int i = n - 1; i >= 0; i--) {
+            if (!dy[i]) continue;
+            const CellPtr W = e.args[1 + i];
+            if (!all && (rc = c.adj_add({W}, std::unique_ptr<ThunkSpec>(new MatMulSpec(true, false, 1.f, 0)), {dy[i], x})))
+                return rc;                                                     // G^T A
+            if ((rc = c.adj_add({x}, std::unique_ptr<ThunkSpec>(new MatMulSpec(false, false, 1.f, 0)), {dy[i], W})))
+                return rc;                                                     // G B
+        }
+        return 0;
+    }
+};
+
+// ---------------------------------------------------------------------------
 // RoPE (symplectic_embed src/librarium/llama.rs:463-465); cos/sin are const_ cells
 // x is [S, H*Dh] (the reference's [1,S,H,Dh] flattened); the head count rides in the spec.
 struct RopeBwdSpec : ThunkSpec {
@@ -623,6 +744,10 @@ std::unique_ptr<ThunkSpec> make_rms_norm(float eps)
 std::unique_ptr<ThunkSpec> make_matmul(bool ta, bool tb, float alpha)
 {
     return std::unique_ptr<ThunkSpec>(new MatMulSpec(ta, tb, alpha, 0));
+}
+std::unique_ptr<ThunkSpec> make_projections(int n, bool group_adjoints)
+{
+    return std::unique_ptr<ThunkSpec>(new ProjNSpec(n, group_adjoints));
 }
 std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int64_t H)
 {

@@ -11,6 +11,9 @@ std::unique_ptr<ThunkSpec> make_embed();                              // (W, tok
 std::unique_ptr<ThunkSpec> make_rms_norm(float eps);                  // (x, w) -> y
 std::unique_ptr<ThunkSpec> make_matmul(bool ta, bool tb, float alpha);   // (a, b) -> c, 2-d
 std::unique_ptr<ThunkSpec> make_block_matmul(bool ta, bool tb, float alpha, int64_t H);   // [R,H*C]
+// n products x W_i^T of one shape in one launch: (x, W_1 .. W_n) -> (y_1 .. y_n), 2 <= n <= 4; group_adjoints:
+// their weight gradients as one grouped thunk too (else the adjoint thunks of n separate matmul thunks)
+std::unique_ptr<ThunkSpec> make_projections(int n, bool group_adjoints);
 // the two block products of causal attention, computed on the lower triangle only
 std::unique_ptr<ThunkSpec> make_causal_scores(float alpha, int64_t H);   // (q, k) -> a q k^T
 std::unique_ptr<ThunkSpec> make_causal_pv(int64_t H);                    // (p16, v) -> p16 v

@@ -161,6 +161,7 @@ SIGNATURES = {
     "cacti_llama_adamw_state_get": (ci, [vp, ci, ci, vp, sz]),
     "cacti_llama_io_cells": (ci, [vp] + [C.POINTER(ci)] * 7),
     "cacti_llama_set_attention": (ci, [vp, ci]),
+    "cacti_llama_set_product_groups": (ci, [vp, ci]),
     "cacti_llama_stage": (ci, [vp, ci, ci]),
     "cacti_llama_step": (ci, [vp, vp, vp, vp, ci, ci, vp]),
 }

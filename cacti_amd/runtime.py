@@ -146,6 +146,11 @@ class Llama:
         chain of separate thunks."""
         ffi.call("cacti_llama_set_attention", self._m, {"fused": 0, "thunks": 1}[mode])
 
+    def set_product_groups(self, on):
+        """0: one matmul thunk per product; 1 (default): the up and gate projections of a layer as one thunk and
+        launch; 2: also q, k, v, and the weight gradients of both groups.  Bit-identical results."""
+        ffi.call("cacti_llama_set_product_groups", self._m, int(on))
+
     def put_param(self, i, arr):
         arr = np.ascontiguousarray(arr, dtype=np.float16)
         assert arr.shape == self.params[i][1], (arr.shape, self.params[i])

@@ -174,6 +174,38 @@ def test_one_layer_cycle_full_shape(oracle, one_layer_case, attention):
     assert_inside_envelope(grads, want, k["env"], "one layer, full shape, " + attention)
 
 
+def test_grouped_products_are_the_separate_thunks_bit_for_bit_full_shape(one_layer_case):
+    """The projections that share an input staged as one thunk and one launch (mode 1, the default: up and
+    gate; mode 2: also q, k, v, and the weight gradients of both groups) against one matmul thunk per product
+    (mode 0), at the 3B shapes, where the N = 8640 products run as a main launch plus a launch of small tiles:
+    loss and all 12 gradient tensors identical bit for bit, also when the cycle accumulates into held
+    gradients."""
+    from cacti_amd.runtime import Ctx, Llama
+    k = one_layer_case
+    got = {}
+    for groups in (0, 1, 2):
+        ctx = Ctx(0, 8 << 30, True)
+        m = Llama(ctx, **k["cfgd"])
+        m.set_product_groups(groups)
+        m.put_params_flat(k["flat"])
+        loss = m.step(k["tok"], k["lm_tok"], k["scale"])
+        g1 = m.grads()
+        loss2 = m.step(k["tok"], k["lm_tok"], k["scale"], accumulate=True)
+        got[groups] = (loss, g1, loss2, m.grads(), ctx.log_names().count("matmul"))
+        m.close(); ctx.close()
+    b = got[0]
+    for groups in (1, 2):
+        a = got[groups]
+        assert a[4] < b[4]                                          # fewer thunks in the log
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[2], b[2])
+        for which in (1, 3):
+            assert len(a[which]) == 12
+            for n in a[which]:
+                assert np.array_equal(a[which][n].view(np.uint16), b[which][n].view(np.uint16)), (groups, n, which)
+    say("  matmul thunks per cycle: %d separate, %d with up + gate grouped, %d with everything grouped"
+        % (got[0][4], got[1][4], got[2][4]))
+
+
 def test_every_thunk_of_one_layer_full_shape(oracle):
     """Teacher-forced at the 3B shapes: the oracle's cycle of one decoder layer + head is traced thunk by
     thunk (tests/teacher.py) and every recorded call is replayed on the device with the ORACLE's inputs and

@@ -64,6 +64,24 @@ def test_tiny_llama_step_all_gradients(oracle, attention):
     m.close(); ctx.close()
 
 
+def test_grouped_products_are_the_separate_thunks_bit_for_bit():
+    """Small shapes (every product through the register path): the grouped stagings of the projections and
+    of their weight gradients (modes 1 and 2) give the loss and all gradients of the separate matmul thunks
+    (mode 0), bit for bit."""
+    cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=3, norm_mean=1.0, grad_scale=1024.0)
+    got = {}
+    for groups in (0, 1, 2):
+        ctx, m = _model(cfg)
+        m.set_product_groups(groups)
+        m.put_params_flat(flat)
+        got[groups] = (m.step(tok, lm_tok, scale), m.grads())
+        m.close(); ctx.close()
+    for groups in (1, 2):
+        assert np.array_equal(got[groups][0], got[0][0])
+        for n, g in got[groups][1].items():
+            assert np.array_equal(g.view(np.uint16), got[0][1][n].view(np.uint16)), (groups, n)
+
+
 def test_tiny_llama_literal_config(oracle):
     """BASELINE config 1 as written: every weight ~N(0, 0.02), loss scale 1/(S-1).
     The q/k/gate/up/down gradients (1e-8 .. 1e-11) underflow f16 in the reference's own
