@@ -579,8 +579,18 @@ gemm_mfma_kernel(GemmArgs p)
     // tiles_m - 1 - r, whose k ranges add up to the same length for every r
     const int rows_m = p.pair ? p.tiles_m / 2 : p.tiles_m;
     const int tiles = rows_m * p.tiles_n;
-    const int64_t bz = bid / tiles;
-    bid -= (int)bz * tiles;
+    int64_t bz;
+    if (p.ztab) {
+        // a pointer-table batch is a handful of whole products that share an operand (the projections of one
+        // input, the weight gradients against one input): product fastest, so that the workgroups resident
+        // together on an XCD work on the same tile of every product and fetch the shared panel once
+        const int nz = nb / tiles;
+        bz = bid % nz;
+        bid /= nz;
+    } else {
+        bz = bid / tiles;
+        bid -= (int)bz * tiles;
+    }
     // within a block of the batch, tiles are walked in groups of 8 tile rows x all tile
     // columns, row fastest: the ~64 blocks resident on an XCD then form an 8 x 8 patch of C
     // and each operand panel fetched into its L2 is shared by 8 blocks
