@@ -147,6 +147,10 @@ CACTI_API int cacti_env_host_pagelocked(void)
     return e && strcmp(e, "pagelocked") == 0;
 }
 
+// The primary-context calls below are the ones the reference's CudaPrimaryCtx binds (cacti_gpu_cu_ffi/src/lib.rs:
+// 158-199); HIP marks them deprecated and keeps them working, and they are wanted here under exactly these names.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wdeprecated-declarations"
 CACTI_API int cacti_hip_primary_ctx_retain(int dev, void **pctx)
 {
     CACTI_REQUIRE(pctx, CACTI_E_INVALID, "primary_ctx_retain: null out pointer");
@@ -177,4 +181,6 @@ CACTI_API int cacti_hip_primary_ctx_reset(int dev)
 }
 
 // The null stream: the handle every entry point accepts for "the device's default stream".
+#pragma clang diagnostic pop
+
 CACTI_API void *cacti_hip_stream_null(void) { return nullptr; }
