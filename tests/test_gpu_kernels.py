@@ -499,11 +499,15 @@ def test_attention_block_via_thunks(ops, oracle, S, H, Dh, tri):
 
 
 @pytest.mark.parametrize("S,H,Dh", [(128, 4, 64), (256, 3, 100), (200, 2, 100), (72, 2, 128), (1024, 2, 100),
-                                    (384, 6, 100), (8, 1, 4)])
+                                    (384, 6, 100), (8, 1, 4), (192, 4, 60), (130, 2, 124), (448, 2, 100)])
 def test_fused_attention(ops, oracle, S, H, Dh):
     """The fused forward and adjoint kernels against the oracle's chain of separate thunks: O, the row
     statistics they keep (maximum and sum of exp of the f16 scores), dQ, dK, dV; ragged sequence lengths
-    (rows and keys beyond S are masked) and head dims 4 .. 128; accumulation into existing gradients."""
+    (rows and keys beyond S are masked) and head dims 4 .. 128; accumulation into existing gradients.
+    Both ways of loading tiles are covered: straight into LDS (even head counts with Dh % 8 = 4: every other
+    head addressed 4 elements before its start, windows of 8, 13 and 16 chunks; Dh % 8 = 0) and through
+    registers (3 heads of 100, 1 head of 4); 448 rows give the dK, dV kernel whole tiles past the diagonal,
+    which run as its in-wave pipeline, and a last tile."""
     say("fused attention", S, H, Dh)
     r = rng(1200 + S + Dh)
     alpha = float(np.float32(1.0) / np.sqrt(np.float32(Dh)))
