@@ -444,7 +444,7 @@ def cpu_baseline_adjoints(N, D, H, Dh, F, V):
 
 
 def run_adjoints(args):
-    """BASELINE config 2-4 kernels at 3B shapes; buffers rotate over > 256 MB so every launch
+    """The memory-bound adjoint kernels at 3B shapes; buffers rotate over > 256 MB so every launch
     reads HBM, not the Infinity Cache."""
     import torch
     from cacti_amd import ops

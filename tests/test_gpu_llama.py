@@ -83,7 +83,7 @@ def test_grouped_products_are_the_separate_thunks_bit_for_bit():
 
 
 def test_tiny_llama_literal_config(oracle):
-    """BASELINE config 1 as written: every weight ~N(0, 0.02), loss scale 1/(S-1).
+    """The reference's small training configuration as written: every weight ~N(0, 0.02), loss scale 1/(S-1).
     The q/k/gate/up/down gradients (1e-8 .. 1e-11) underflow f16 in the reference's own
     arithmetic, so those tensors are compared in absolute terms (f16 subnormal quanta)."""
     cfg, flat, tok, lm_tok, scale = make_inputs(TINY, seed=0)
@@ -292,7 +292,7 @@ def test_pool_too_small_is_a_clean_error(oracle):
 
 
 def test_full_size_step_properties():
-    """BASELINE's configuration at full shapes (S=2048, D=3200, H=32 x 100, F=8640, V=32000) with
+    """The reference's 3B configuration at full shapes (S=2048, D=3200, H=32 x 100, F=8640, V=32000) with
     4 of the 26 layers (the oracle would need a minute per layer): properties that hold at any
     size.  (a) the loss is -log softmax(logit)[target] of the logits the step returns, recomputed
     in fp64; (b) a second cycle is bit-identical; (c) doubling the loss scale (a power of two)
