@@ -369,6 +369,24 @@ __device__ __forceinline__ void load_frags(half8_t (&f)[KS], gptr_t X, int64_t l
     }
 }
 
+// The same fragments out of an LDS tile that holds the operand's rows in window positions (a tile loaded
+// straight into LDS; row = the lane's row inside the tile): what lies outside the head there is the
+// neighbouring heads' data, cleared here.  Rows beyond S are zero in such a tile already.
+template <int KS>
+__device__ __forceinline__ void frags_from_tile(half8_t (&f)[KS], const unsigned char *tile, int row, int Dh, int lh,
+                                                int shift)
+{
+    const unsigned char *rp = tile + row * kRowB;
+    const int g = gsw(row);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(rp + (((2 * ks + lh) ^ g) << 4));
+        const int d0 = 16 * ks + 8 * lh - shift;
+        const bool ok0 = d0 >= 0 && d0 < Dh, ok1 = d0 + 4 < Dh;
+        f[ks] = as_h8(make_uint2(ok0 ? v.x : 0u, ok0 ? v.y : 0u), make_uint2(ok1 ? v.z : 0u, ok1 ? v.w : 0u));
+    }
+}
+
 // acc = sum over d of X[row_base + .][d] Y[.][d]: X from the LDS tile (16-byte reads), Y = fixed fragments.
 // PRIO: the wave runs its chain of dependent MFMAs at raised priority, so that the other wave of the SIMD
 // fills the gaps of the chain with its arithmetic instead of delaying it (forward and dQ kernel -2 %; the
@@ -568,6 +586,42 @@ __device__ __forceinline__ void store_row4(half_t *dst, float a0, float a1, floa
     *reinterpret_cast<half4_t *>(dst) = o;
 }
 
+// An output tile of 128 rows leaves through LDS when the tiles are direct (16-byte aligned rows): stores in which
+// every lane addresses its own row are served at about one lane per clock and CU like such loads (16 of them per
+// lane and output: 4 k cycles per workgroup), whole row segments of 16 bytes per lane are not.  stage_rows: a
+// wave's 32 rows as f16(scale acc), in window positions, in the layout of an operand tile; write_rows: the
+// staged rows [0, rows) to memory by all threads, the head's columns only (dst = the window's first element in
+// row 0).  The same values as store_row4 writes.
+template <int DT>
+__device__ __forceinline__ void stage_rows(unsigned char *stage, const float16_t (&acc)[DT], int row, int lh, float scale)
+{
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            half4_t o;
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[r] = f2h(scale * acc[dt][4 * q + r]);
+            *reinterpret_cast<half4_t *>(stage + toff(row, 4 * dt + q) + 8 * lh) = o;
+        }
+}
+__device__ __forceinline__ void write_rows(const unsigned char *stage, half_t *dst, int64_t ld, int rows, int Dh,
+                                           int shift, int tid, int nthr)
+{
+    const int nch = (Dh + shift + 7) >> 3;
+    for (int i = tid; i < kBM * 16; i += nthr) {
+        const int row = i >> 4, c = i & 15;
+        if (row >= rows || c >= nch) continue;
+        const uint4 v = *reinterpret_cast<const uint4 *>(stage + toff(row, c));
+        const int d0 = 8 * c - shift;                    // the head's column at the chunk's first position
+        const bool lo = d0 >= 0 && d0 < Dh, hi = d0 + 4 < Dh;
+        half_t *q = dst + (int64_t)row * ld + 8 * c;
+        if (lo && hi) *reinterpret_cast<uint4 *>(q) = v;
+        else if (lo) *reinterpret_cast<uint2 *>(q) = make_uint2(v.x, v.y);
+        else if (hi) *reinterpret_cast<uint2 *>(q + 4) = make_uint2(v.z, v.w);
+    }
+}
+
 // Work split of the query-major kernels (forward, dQ).  A workgroup is two wave groups of 4 waves on
 // the same 128 query rows; group g takes the key tiles g, g + 2, ... with its own LDS buffers, and the
 // two partial results (row statistics, output tile) meet in LDS at the end: the 2 waves a SIMD holds
@@ -620,8 +674,10 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
     {
         const int i0 = qt * kBM, r0 = i0 + wid * 32, myrow = r0 + l32;
 
+        // the queries: with direct tiles they come as two tiles straight into LDS below, beside the first key
+        // and value tiles (a load in which every lane addresses its own row is served at one lane per clock)
         half8_t qf[KS];
-        load_frags<KS>(qf, Q, ld, myrow, S, Dh, lh, shift);
+        if constexpr (!DMA) load_frags<KS>(qf, Q, ld, myrow, S, Dh, lh, shift);
 
         const int kend = min(i0 + kBM, S);                 // keys [0, kend) are visible to the tile
         const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
@@ -638,8 +694,15 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             // the V buffers idle through pass 1: the first V tile of pass 2 comes in now
             if constexpr (DMA) tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
         }
-        if constexpr (DMA) zero_pads(smem, 2 * kGroupLds / kRowB, (Dh + shift + 7) >> 3);
+        if constexpr (DMA) {
+            // rows 64 g .. 64 g + 63 of the workgroup's queries into this group's second V buffer, which idles
+            // until the second pass; every wave then takes its fragments from the tile that holds its rows
+            tv.load(tm, Q - shift + (int64_t)(i0 + g * kTileRows) * ld, S - (i0 + g * kTileRows), Vs + kTileB);
+            zero_pads(smem, 2 * kGroupLds / kRowB, (Dh + shift + 7) >> 3);
+        }
         tile_sync<DMA>();
+        if constexpr (DMA)
+            frags_from_tile<KS>(qf, smem + (wid >> 1) * kGroupLds + 3 * kTileB, (wid & 1) * 32 + l32, Dh, lh, shift);
         int it0 = 0;
         if constexpr (FAST) {
             // The key tiles wholly below the diagonal for every wave (iterations 0 .. qt - 1 of both groups) as a
@@ -852,7 +915,12 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             tile_sync<DMA>();
         }
         merge_partials<DT>(oacc, smem + kGroupLds, g, tig);
-        if (g == 0 && myrow < S) {
+        if constexpr (DMA) {
+            if (g == 0) stage_rows<DT>(smem, oacc, wid * 32 + l32, lh, 1.0f);
+            __syncthreads();
+            write_rows(smem, p.out + (int64_t)i0 * ld + (int64_t)h * Dh - shift, ld, min(kBM, S - i0), Dh, shift,
+                       threadIdx.x, kNT2);
+        } else if (g == 0 && myrow < S) {
             half_t *orow = p.out + (int64_t)myrow * ld + (int64_t)h * Dh;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
@@ -892,12 +960,56 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
     gptr_t K = gp(p.k) + hoff - shift, V = gp(p.v) + hoff - shift;
     {
         const int i0 = qt * kBM, r0 = i0 + wid * 32, myrow = r0 + l32;
-
-        half8_t qf[KS], gf[KS];
-        load_frags<KS>(qf, gp(p.q) + hoff, ld, myrow, S, Dh, lh, shift);
-        load_frags<KS>(gf, gp(p.dO) + hoff, ld, myrow, S, Dh, lh, shift);
+        const int kend = min(i0 + kBM, S);
+        const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
+        typedef typename std::conditional<DMA, DmaTileMap, TileMap8>::type Map;
+        typedef typename std::conditional<DMA, DmaTileLoader, TileLoader8>::type Loader;
+        const Map tm(ld, Dh, shift);
+        Loader tk, tv;
+        auto first_tiles = [&]() __attribute__((always_inline)) {
+            if (g < njt) {
+                tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
+                tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
+                tk.store(tm, Ks);
+                tv.store(tm, Vs);
+            }
+        };
+        // The fixed operands.  A load in which every lane addresses its own row is served at about one lane
+        // per clock and CU (42 such instructions in each of 8 waves: 21 k of the 29 k cycles this kernel used
+        // to spend before its first product), so with direct tiles the workgroup's 128 rows of q, dO and the
+        // forward output (used by the short form of sigma, decided below from the statistics) come as six
+        // tiles straight into LDS, whole row segments per instruction, and each wave picks its fragments out
+        // of them; both wave groups hold the same rows and share the tiles.  Then the first key and value
+        // tiles go out, into the same buffers, before anything else is computed.
+        bool tiles_on_the_way = false;
         float m = ((gfptr_t)p.m)[(int64_t)h * S + min(myrow, S - 1)];
         float l = ((gfptr_t)p.l)[(int64_t)h * S + min(myrow, S - 1)];
+        half8_t qf[KS], gf[KS], of[FAST ? KS : 1];
+        if constexpr (DMA) {
+            const int64_t off = hoff - shift + (int64_t)(i0 + g * kTileRows) * ld;
+            const int left = S - (i0 + g * kTileRows);
+            const bool want_o = FAST && p.o;
+            tk.load(tm, gp(p.q) + off, left, smem + g * kTileB);
+            tk.load(tm, gp(p.dO) + off, left, smem + (2 + g) * kTileB);
+            if (want_o) tk.load(tm, gp(p.o) + off, left, smem + (4 + g) * kTileB);
+            tile_sync<DMA>();
+            const unsigned char *mine = smem + (wid >> 1) * kTileB;
+            const int trow = (wid & 1) * 32 + l32;
+            frags_from_tile<KS>(qf, mine, trow, Dh, lh, shift);
+            frags_from_tile<KS>(gf, mine + 2 * kTileB, trow, Dh, lh, shift);
+            if constexpr (FAST) {
+                if (want_o) frags_from_tile<KS>(of, mine + 4 * kTileB, trow, Dh, lh, shift);
+            }
+            __syncthreads();                      // every wave holds its fragments: the buffers are free again
+            first_tiles();
+            tiles_on_the_way = true;
+        } else {
+            load_frags<KS>(qf, gp(p.q) + hoff, ld, myrow, S, Dh, lh, shift);
+            load_frags<KS>(gf, gp(p.dO) + hoff, ld, myrow, S, Dh, lh, shift);
+            if constexpr (FAST) {
+                if (p.o) load_frags<KS>(of, gp(p.o) + hoff, ld, myrow, S, Dh, lh, shift);
+            }
+        }
         float sig = 0.f;
         if (myrow >= S) {
             m = 0.f;
@@ -906,22 +1018,12 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
         const float y = recip_refined(l);
         const float cs = prob_shift(m, l);
 
-        const int kend = min(i0 + kBM, S);
-        const int njt = (kend + kTileRows - 1) / kTileRows, niter = (njt + 1) / 2;
-        typedef typename std::conditional<DMA, DmaTileMap, TileMap8>::type Map;
-        typedef typename std::conditional<DMA, DmaTileLoader, TileLoader8>::type Loader;
-        const Map tm(ld, Dh, shift);
-        Loader tk, tv;
         float16_t dacc[DT];
         auto run_pass = [&](auto pass_c) __attribute__((always_inline)) {
             constexpr int PASS = decltype(pass_c)::value;
             float part = 0.f;
-            if (g < njt) {
-                tk.load(tm, K + (int64_t)g * kTileRows * ld, S - g * kTileRows, Ks);
-                tv.load(tm, V + (int64_t)g * kTileRows * ld, S - g * kTileRows, Vs);
-                tk.store(tm, Ks);
-                tv.store(tm, Vs);
-            }
+            if (!tiles_on_the_way) first_tiles();
+            tiles_on_the_way = false;
             tile_sync<DMA>();
             for (int it = 0; it < niter; it++) {
                 const int jt = 2 * it + g, cur = it & 1;
@@ -1003,11 +1105,9 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             if (p.o) short_sigma = __syncthreads_and(myrow >= S || l >= kSpread) != 0;
         }
         if (short_sigma) {
-            half8_t of[KS];
-            load_frags<KS>(of, gp(p.o) + hoff, ld, myrow, S, Dh, lh, shift);
             float part = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++)
+            for (int ks = 0; ks < (FAST ? KS : 1); ks++)
 #pragma unroll
                 for (int e = 0; e < 8; e++) part = __builtin_fmaf((float)gf[ks][e], (float)of[ks][e], part);
             sig = part + __shfl_xor(part, 32, 64);                     // the two lanes of a row
@@ -1028,7 +1128,11 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             for (int r = 0; r < 16; r++) dacc[dt][r] = 0.f;
         run_pass(std::integral_constant<int, 1>{});
         merge_partials<DT>(dacc, smem + kGroupLds, g, tig);
-        if (g == 0 && myrow < S) {
+        if (DMA && !p.acc_dq) {
+            if (g == 0) stage_rows<DT>(smem, dacc, wid * 32 + l32, lh, p.alpha);
+            __syncthreads();
+            write_rows(smem, p.dq + (int64_t)i0 * ld + hoff - shift, ld, min(kBM, S - i0), Dh, shift, threadIdx.x, kNT2);
+        } else if (g == 0 && myrow < S) {
             half_t *drow = p.dq + (int64_t)myrow * ld + hoff;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
@@ -1083,9 +1187,13 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
         const int kt_ = pr;                                             // low key tiles see the most queries
         const int c00 = kt_ * kBM, c0 = c00 + wid * 32, mykey = c0 + l32;
 
+        // the keys and values of the workgroup: with direct tiles they come as tiles straight into LDS, beside the
+        // first query tile (below)
         half8_t kf[KS], vf[KS];
-        load_frags<KS>(kf, gp(p.k) + hoff, ld, mykey, S, Dh, lh, shift);
-        load_frags<KS>(vf, gp(p.v) + hoff, ld, mykey, S, Dh, lh, shift);
+        if constexpr (!DMA) {
+            load_frags<KS>(kf, gp(p.k) + hoff, ld, mykey, S, Dh, lh, shift);
+            load_frags<KS>(vf, gp(p.v) + hoff, ld, mykey, S, Dh, lh, shift);
+        }
 
         float16_t kacc[DT], vacc[DT];
 #pragma unroll
@@ -1190,7 +1298,21 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
 
         fetch(iq0);
         land(iq0);
+        if constexpr (DMA) {
+            // the 128 key and value rows into the second and third buffers, idle until the first tile is worked on
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const int64_t off = hoff - shift + (int64_t)(c00 + t * kTileRows) * ld;
+                tq.load(tm, gp(p.k) + off, S - (c00 + t * kTileRows), Qs + (1 + t) * kTileB);
+                tg.load(tm, gp(p.v) + off, S - (c00 + t * kTileRows), Gs + (1 + t) * kTileB);
+            }
+        }
         tile_sync<DMA>();
+        if constexpr (DMA) {
+            frags_from_tile<KS>(kf, Qs + (1 + (wid >> 1)) * kTileB, (wid & 1) * 32 + l32, Dh, lh, shift);
+            frags_from_tile<KS>(vf, Gs + (1 + (wid >> 1)) * kTileB, (wid & 1) * 32 + l32, Dh, lh, shift);
+            __syncthreads();                      // every wave holds its fragments: the buffers take query tiles now
+        }
         // The tiles that hold the diagonal (two: 128 keys) and a ragged last tile run block by block.  The tiles
         // between them, whose 32-query blocks are whole and past the diagonal for every wave, run as a pipeline
         // (fast arithmetic, tiles loaded straight into LDS): while the vector unit forms P and dS of block b, the
@@ -1351,7 +1473,17 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
         } else {
             run_tiles(iq0, niq);
         }
-        if (mykey < S) {
+        const bool staged_v = DMA && !p.acc_dv, staged_k = DMA && !p.acc_dk;
+        if (staged_v || staged_k) {
+            __syncthreads();                              // the last products have read their tiles
+            if (staged_k) stage_rows<DT>(Qs, kacc, wid * 32 + l32, lh, p.alpha);
+            if (staged_v) stage_rows<DT>(Gs, vacc, wid * 32 + l32, lh, 1.0f);
+            __syncthreads();
+            const int64_t off = (int64_t)c00 * ld + hoff - shift;
+            if (staged_k) write_rows(Qs, p.dk + off, ld, min(kBM, S - c00), Dh, shift, threadIdx.x, kNT);
+            if (staged_v) write_rows(Gs, p.dv + off, ld, min(kBM, S - c00), Dh, shift, threadIdx.x, kNT);
+        }
+        if (mykey < S && !(staged_v && staged_k)) {
             half_t *krow = p.dk + (int64_t)mykey * ld + hoff, *vrow = p.dv + (int64_t)mykey * ld + hoff;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
@@ -1359,10 +1491,12 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 for (int q = 0; q < 4; q++) {
                     const int d0 = 32 * dt + 8 * q + 4 * lh - shift;
                     if (d0 >= 0 && d0 < Dh) {
-                        store_row4(vrow + d0, vacc[dt][4 * q], vacc[dt][4 * q + 1], vacc[dt][4 * q + 2],
-                                   vacc[dt][4 * q + 3], 1.0f, p.acc_dv);
-                        store_row4(krow + d0, kacc[dt][4 * q], kacc[dt][4 * q + 1], kacc[dt][4 * q + 2],
-                                   kacc[dt][4 * q + 3], p.alpha, p.acc_dk);
+                        if (!staged_v)
+                            store_row4(vrow + d0, vacc[dt][4 * q], vacc[dt][4 * q + 1], vacc[dt][4 * q + 2],
+                                       vacc[dt][4 * q + 3], 1.0f, p.acc_dv);
+                        if (!staged_k)
+                            store_row4(krow + d0, kacc[dt][4 * q], kacc[dt][4 * q + 1], kacc[dt][4 * q + 2],
+                                       kacc[dt][4 * q + 3], p.alpha, p.acc_dk);
                     }
                 }
         }
@@ -1500,7 +1634,7 @@ CACTI_API int cacti_hip_attention_fwd(int64_t S, int64_t H, int64_t Dh, float al
     p.l = p.m + S * H;
     hipStream_t st = (hipStream_t)stream;
     int64_t span;
-    const bool dma = direct_tiles(H, Dh, ld, {k, v}, &span);
+    const bool dma = direct_tiles(H, Dh, ld, {q, k, v, o}, &span);
     return dispatch<Fwd>(span, g_exact.load(std::memory_order_relaxed) != 0, dma, p, st);
 }
 
@@ -1532,6 +1666,6 @@ CACTI_API int cacti_hip_attention_bwd(int64_t S, int64_t H, int64_t Dh, float al
     p.sig = p.y + S * H;
     hipStream_t st = (hipStream_t)stream;
     int64_t span;
-    const bool dma = direct_tiles(H, Dh, ld, {q, k, v, dO}, &span);
+    const bool dma = direct_tiles(H, Dh, ld, {q, k, v, dO, o, dq, dk, dv}, &span);     // o may be null: passes
     return dispatch<Bwd>(span, g_exact.load(std::memory_order_relaxed) != 0, dma, p, st);
 }

@@ -894,9 +894,62 @@ gemm_mfma_kernel(GemmArgs p)
         if (kt0 + NBUF <= nk) wait_vmem<(NBUF - 1) * ND>();       // the first tile; the others stay in flight
         else wait_vmem<0>();
         __syncthreads();
+        int t = kt0, cb = 0;
+        if constexpr (TM * TN == 1) {
+        // One 32 x 32 block per wave: a half is two MFMAs (32 cycles), far less than an LDS read takes, so
+        // reads issued one half ahead leave the wave waiting in every half.  Here the fragments of a whole
+        // k tile (two register sets) are read while the eight MFMAs of the tile before run: behind the
+        // barrier of tile t (tile t + 1 has landed; every wave holds tile t in registers, the barrier's own
+        // wait for LDS sees to that) come the reads of tile t + 1, the loads of tile t + NBUF into the
+        // buffer of tile t, and then the MFMAs of tile t.
+        half8_t ga[2][2][NA], gb[2][2][NB];
+        auto read_tile = [&](auto set_c, int buf) __attribute__((always_inline)) {
+            constexpr int S = decltype(set_c)::value;
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+                for (int a = 0; a < NA; a++) ga[S][ks][a] = read_a(buf, ks, a);
+#pragma unroll
+                for (int b = 0; b < NB; b++) gb[S][ks][b] = read_b(buf, ks, b);
+            }
+        };
+        auto body = [&](auto set_c, auto main_c) __attribute__((always_inline)) {
+            constexpr int S = decltype(set_c)::value;
+            constexpr bool MAIN = decltype(main_c)::value;
+            const int nb = next_buf(cb);
+            if (MAIN || t + 1 < nk) {
+                if (MAIN) wait_vmem<(NBUF - 2) * ND>();
+                else wait_vmem<0>();
+                __syncthreads();
+                read_tile(std::integral_constant<int, S ^ 1>{}, nb);
+                __builtin_amdgcn_sched_barrier(0);
+                if (MAIN || t + NBUF < nk) issue_all(t + NBUF, cb);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+                for (int a = 0; a < NA; a++)
+#pragma unroll
+                    for (int b = 0; b < NB; b++)
+                        c16[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(gb[S][ks][b], ga[S][ks][a], c16[a][b], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            cb = nb;
+            t++;
+        };
+        read_tile(std::integral_constant<int, 0>{}, 0);
+        while (t + NBUF + 1 < nk) {                               // both steps load inside K
+            body(std::integral_constant<int, 0>{}, std::true_type{});
+            body(std::integral_constant<int, 1>{}, std::true_type{});
+        }
+        while (t < nk) {
+            body(std::integral_constant<int, 0>{}, std::false_type{});
+            if (t < nk) body(std::integral_constant<int, 1>{}, std::false_type{});
+        }
+        __syncthreads();
+        } else {
 #pragma unroll
         for (int u = 0; u < TM + NB; u++) next_read(u, 0, 0, 0);
-        int t = kt0, cb = 0;
         for (; t + NBUF < nk; t++) {                              // every load of the body lies inside K
             first_halves(cb);
             const int nb = next_buf(cb);
@@ -937,6 +990,7 @@ gemm_mfma_kernel(GemmArgs p)
             cb = nb;
         }
         __syncthreads();                                          // every wave is done with the operand buffers
+        }
     } else {
         la.load(ra[0], Ao, (int64_t)kt0 * BK);
         lb.load(rb[0], Bo, (int64_t)kt0 * BK);
