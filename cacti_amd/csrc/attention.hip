@@ -41,7 +41,11 @@
 // How a K / V (Q / dO) tile gets there: straight from memory by global_load_lds_dwordx4 where the tensors
 // allow it (16-byte aligned, see DmaTileMap: every head addressed from the 16-byte boundary at or below
 // its start), else through registers (FastTileLoader, TileLoader8).  Measured at 32 heads x 2048 x 100:
-// forward 108.7 -> 92.9 us, adjoint 235.5 -> 209.8 us, 48 vector registers fewer per kernel.
+// forward 108.7 -> 92.9 us, adjoint 235.5 -> 209.8 us, 48 vector registers fewer per kernel.  On that path the
+// fixed operand of a workgroup (its 128 rows) arrives as tiles in LDS as well and every wave picks its fragments
+// out of them (frags_from_tile), and the outputs leave through LDS as whole row segments (stage_rows,
+// write_rows): a load or store in which every lane addresses its own row costs about a clock per lane.
+// Forward 85.9 -> 79.0 us, dQ 95.8 -> 84.8, dK / dV 101.9 -> 97.0.
 #include "common.h"
 #include "softmax_math.h"
 

@@ -264,9 +264,10 @@ int cacti_hip_causal_softmax_bwd(int64_t S, int64_t H, const void *s16, const vo
  * Dh % 4 == 0, Dh <= 128, ld % 4 == 0.  stats: cacti_hip_attention_stats_bytes(S, H) bytes of device
  * memory, written by the forward call (row maximum and sum per head and row, f32) and read by the
  * adjoint; workspace: cacti_hip_attention_bwd_workspace(S, H) bytes, contents undefined on return.
- * Faster with 16-byte aligned q, k, v, dO, ld % 8 == 0 and, for Dh % 8 == 4, an even number of heads filling
- * the row (every head then lies inside whole 16-byte pieces of its row that start at or 8 bytes before it):
- * the kernels load their tiles straight into LDS, 12 % less time at 32 heads x 100.  In that form a head's
+ * Faster with every tensor of the call 16-byte aligned, ld % 8 == 0 and, for Dh % 8 == 4, an even number of
+ * heads filling the row (every head then lies inside whole 16-byte pieces of its row that start at or 8 bytes
+ * before it): the kernels move all their tiles, operands and results, as whole row segments between memory and
+ * LDS, 20 % less time at 32 heads x 100.  In that form a head's
  * products run over those whole pieces, the elements of the neighbouring head in them multiplied by zeros: for
  * finite inputs the same values; a non-finite element in the 4 columns next to a head makes that head's
  * result non-finite as well (the reference: the neighbour's only, until the output projection mixes them).
