@@ -661,6 +661,11 @@ __device__ __forceinline__ void merge_partials(float16_t (&acc)[DT], unsigned ch
 template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 {
+    // the whole argument block in scalar registers at once (read field by field where the control flow first
+    // wants it, it costs several dependent round trips to memory before the first tile is requested)
+    asm volatile("" ::"s"(p.S), "s"(p.H), "s"(p.Dh), "s"(p.ld), "s"(p.alpha), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.dO),
+                 "s"(p.o), "s"(p.out), "s"(p.dq), "s"(p.dk), "s"(p.dv), "s"(p.m), "s"(p.l), "s"(p.y), "s"(p.sig),
+                 "s"(p.acc_dq), "s"(p.acc_dk), "s"(p.acc_dv));
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     if constexpr (!DMA) zero_lds(smem, 2 * kGroupLds);   // the pad columns of the tile buffers: zero from here on
@@ -946,6 +951,11 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 {
+    // the whole argument block in scalar registers at once (read field by field where the control flow first
+    // wants it, it costs several dependent round trips to memory before the first tile is requested)
+    asm volatile("" ::"s"(p.S), "s"(p.H), "s"(p.Dh), "s"(p.ld), "s"(p.alpha), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.dO),
+                 "s"(p.o), "s"(p.out), "s"(p.dq), "s"(p.dk), "s"(p.dv), "s"(p.m), "s"(p.l), "s"(p.y), "s"(p.sig),
+                 "s"(p.acc_dq), "s"(p.acc_dk), "s"(p.acc_dv));
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int g = __builtin_amdgcn_readfirstlane(threadIdx.x >> 8), tig = threadIdx.x & (kNT - 1);
@@ -958,9 +968,9 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
     const int h = blockIdx.x % p.H, qt = nqt - 1 - blockIdx.x / p.H;
     const int64_t hoff = (int64_t)h * Dh;
     const int shift = DMA ? (int)(hoff & 7) : 0;                        // the head's first column in its window
-    // the pad columns of the tile buffers: zero from here on (published by the first pass's first barrier)
-    if constexpr (DMA) zero_pads(smem, 2 * kGroupLds / kRowB, (Dh + shift + 7) >> 3);
-    else zero_lds(smem, 2 * kGroupLds);
+    // the pad columns of the tile buffers: zero from the first barrier on (direct tiles: cleared below, behind
+    // the first loads)
+    if constexpr (!DMA) zero_lds(smem, 2 * kGroupLds);
     gptr_t K = gp(p.k) + hoff - shift, V = gp(p.v) + hoff - shift;
     {
         const int i0 = qt * kBM, r0 = i0 + wid * 32, myrow = r0 + l32;
@@ -996,6 +1006,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
             tk.load(tm, gp(p.q) + off, left, smem + g * kTileB);
             tk.load(tm, gp(p.dO) + off, left, smem + (2 + g) * kTileB);
             if (want_o) tk.load(tm, gp(p.o) + off, left, smem + (4 + g) * kTileB);
+            zero_pads(smem, 2 * kGroupLds / kRowB, (Dh + shift + 7) >> 3);
             tile_sync<DMA>();
             const unsigned char *mine = smem + (wid >> 1) * kTileB;
             const int trow = (wid & 1) * 32 + l32;
@@ -1168,6 +1179,11 @@ constexpr int kDkvBufs = 3;                      // tile buffers per tensor (Q, 
 template <int KS, int DT, bool FAST, bool DMA>
 __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
 {
+    // the whole argument block in scalar registers at once (read field by field where the control flow first
+    // wants it, it costs several dependent round trips to memory before the first tile is requested)
+    asm volatile("" ::"s"(p.S), "s"(p.H), "s"(p.Dh), "s"(p.ld), "s"(p.alpha), "s"(p.q), "s"(p.k), "s"(p.v), "s"(p.dO),
+                 "s"(p.o), "s"(p.out), "s"(p.dq), "s"(p.dk), "s"(p.dv), "s"(p.m), "s"(p.l), "s"(p.y), "s"(p.sig),
+                 "s"(p.acc_dq), "s"(p.acc_dk), "s"(p.acc_dv));
     typedef AttnMath<FAST> M;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     unsigned char *Qs = smem, *Gs = smem + kDkvBufs * kTileB;
@@ -1180,9 +1196,9 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
     const int64_t hoff = (int64_t)h * Dh;
     const int shift = DMA ? (int)(hoff & 7) : 0;                        // the head's first column in its window
     gptr_t Q = gp(p.q) + hoff - shift, G = gp(p.dO) + hoff - shift;
-    // the pad columns of the tile buffers: zero from here on (published by the first tile's barrier)
-    if constexpr (DMA) zero_pads(smem, 2 * kDkvBufs * kTileB / kRowB, (Dh + shift + 7) >> 3);
-    else zero_lds(smem, 2 * kDkvBufs * kTileB);
+    // the pad columns of the tile buffers: zero from the first tile's barrier on (direct tiles: cleared below,
+    // behind the first loads)
+    if constexpr (!DMA) zero_lds(smem, 2 * kDkvBufs * kTileB);
     // the four per-row statistics of a 64-query tile: lane t of wave w fetches array w, row t
     gfptr_t stat_src = (gfptr_t)(wid == 0 ? p.m : wid == 1 ? p.l : wid == 2 ? p.y : p.sig) + (int64_t)h * S;
     const float stat_pad = (wid == 1 || wid == 2) ? 1.f : 0.f;
@@ -1310,6 +1326,7 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                 tq.load(tm, gp(p.k) + off, S - (c00 + t * kTileRows), Qs + (1 + t) * kTileB);
                 tg.load(tm, gp(p.v) + off, S - (c00 + t * kTileRows), Gs + (1 + t) * kTileB);
             }
+            zero_pads(smem, 2 * kDkvBufs * kTileB / kRowB, (Dh + shift + 7) >> 3);
         }
         tile_sync<DMA>();
         if constexpr (DMA) {

@@ -553,6 +553,11 @@ template <bool TA, bool TB, int BM, int BN, int WM, int WN, int AL, bool KTAIL, 
 __global__ void __launch_bounds__(WM * WN * 64, min_waves(BM, BN, WM * WN, NBUF))
 gemm_mfma_kernel(GemmArgs p)
 {
+    // the whole argument block in scalar registers before anything else: read field by field where the control
+    // flow first wants it, it costs five dependent round trips to memory before the first operand load
+    asm volatile("" ::"s"(p.M), "s"(p.N), "s"(p.K), "s"(p.alpha), "s"(p.beta), "s"(p.A), "s"(p.lda), "s"(p.sa), "s"(p.B),
+                 "s"(p.ldb), "s"(p.sb), "s"(p.C), "s"(p.ldc), "s"(p.sc), "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.tri),
+                 "s"(p.gm), "s"(p.xcd), "s"(p.pair), "s"(p.win), "s"(p.ztab));
     static_assert(DMA ? (STAGES == 1 && AL == 8 && !KTAIL) : NBUF == 2,
                   "direct loads: 16-byte aligned operands, whole k tiles");
     constexpr bool TR_A = DMA && TA, TR_B = DMA && !TB;           // fragments by transposing reads
@@ -656,6 +661,17 @@ gemm_mfma_kernel(GemmArgs p)
         lb.init(p.ldb, (p.win ? (nw + 7) / 8 * 8 : nw) - n0, p.K);
     }
     uint4 ra[STAGES][LA::NREG], rb[STAGES][LB::NREG];
+    // direct loads: the first NBUF tiles are requested here, before the accumulators are cleared and the
+    // fragment addresses worked out (some thousand cycles of set-up that need not stand in front of them)
+    if constexpr (DMA) {
+#pragma unroll
+        for (int u = 0; u < NBUF; u++)
+            if (kt0 + u < nk) {
+                la.dma((uint32_t)(uintptr_t)(As + u * BM * BK), Ao, (int64_t)(kt0 + u) * BK);
+                lb.dma((uint32_t)(uintptr_t)(Bs + u * BN * BK), Bo, (int64_t)(kt0 + u) * BK);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+    }
 
     // direct path: 16 x 16 results of v_mfma_f32_16x16x32_f16, [A fragment][B fragment]; lane l holds row
     // l % 16 of the fragment pair's block and columns 4 (l / 16) .. + 3
@@ -888,9 +904,6 @@ gemm_mfma_kernel(GemmArgs p)
             SchedStep<NMH, RA, 0>::run();
             __builtin_amdgcn_sched_barrier(0);
         };
-#pragma unroll
-        for (int u = 0; u < NBUF; u++)
-            if (kt0 + u < nk) issue_all(kt0 + u, u);
         if (kt0 + NBUF <= nk) wait_vmem<(NBUF - 1) * ND>();       // the first tile; the others stay in flight
         else wait_vmem<0>();
         __syncthreads();
@@ -1036,7 +1049,30 @@ gemm_mfma_kernel(GemmArgs p)
     constexpr int CSW = (CPRC & (CPRC - 1)) == 0 ? CPRC - 1 : 7;  // chunk swizzle mask
     static_assert(CPRC % (CSW + 1) == 0, "the chunk swizzle must stay inside the row");
     const bool has_beta = p.beta != 0.f;
-    if (has_beta) {
+    // (the lane's index as a value the compiler cannot trace back: the addresses of the batched paths below are
+    // otherwise computed before the k loop, kept across it and spilled inside it)
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    // a tile wholly inside C, 16-byte aligned: all of a lane's pieces of the old tile requested before the first is
+    // stored (the general loop below waits for every piece in turn: 9,000 cycles more per workgroup measured)
+    // (tiles of up to 256 x 128: the larger ones have no registers for it and spill in their main loop with it)
+    constexpr bool C_BATCH = BM * BN <= 256 * 128 && BM * CPRC % NT == 0;
+    const bool c_inside = C_BATCH && AL == 8 && shift == 0 && m0 + BM <= p.M && n0 + BN <= nw;
+    if (has_beta && c_inside) {
+        constexpr int NC = C_BATCH ? BM * CPRC / NT : 1;
+        uint4 old[NC];
+#pragma unroll
+        for (int i = 0; i < NC; i++) {
+            const int c = tid + i * NT, row = c / CPRC, cc = c % CPRC;
+            old[i] = *reinterpret_cast<const uint4 *>(C + (m0 + row) * p.ldc + n0 + cc * 8);
+        }
+#pragma unroll
+        for (int i = 0; i < NC; i++) {
+            const int c = tid + i * NT, row = c / CPRC, cc = c % CPRC;
+            *reinterpret_cast<uint4 *>(Cs + row * BN + ((cc ^ (row & CSW)) << 3)) = old[i];
+        }
+        __syncthreads();
+    } else if (has_beta) {
         for (int c = threadIdx.x; c < BM * CPRC; c += NT) {
             const int row = c / CPRC, cc = c % CPRC;
             const int64_t m = m0 + row, n = n0 + cc * 8;
