@@ -26,7 +26,9 @@ sys.path.insert(0, ROOT)
 LLAMA_3B = dict(S=2048, D=3200, H=32, Dh=100, F=8640, V=32000, L=26, eps=1e-6)
 PEAK_MFMA_F16_TFLOPS = 2500.0      # MI355X dense fp16 MFMA
 PEAK_HBM_GBS = 8000.0              # MI355X HBM3E
-EVENT_STRIDE = 5                   # timed region: 1 in 5 launches of the dominant kernel carries events
+EVENT_STRIDE = 17                  # timed region: 1 in 17 launches of the dominant kernel carries events (a pair
+                                   # costs about 17 us of stream time, two gaps in the kernel trace; at 1 in 5 that
+                                   # was 0.55 ms of a 50 ms step)
 
 
 def log(*a):
@@ -318,7 +320,8 @@ def run_step(args):
     prefix = next(iter(prefixes))
 
     # timed region: exactly K steps, events around every EVENT_STRIDE-th launch of the dominant
-    # kernel (the stride is coprime to the 7 such launches per layer, so all shapes are sampled)
+    # kernel (the stride is coprime to the 6 such launches per layer and the 157 per step, so all
+    # shapes are sampled)
     ctx.set_timing(0)
     ctx.set_timing_filter(prefix, EVENT_STRIDE)
     ctx.set_timing(2)
