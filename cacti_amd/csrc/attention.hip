@@ -35,8 +35,11 @@
 //
 // LDS tiles are [rows][128 halves] (256 bytes per row = one pass over all 64 banks, head dim
 // zero-padded); 16-byte chunk c of row r sits at chunk c ^ g(r), g(r) = 2 (r & 3) | ((r >> 2) & 1) |
-// 8 ((r >> 3) & 1): the 16-byte operand reads of 16 consecutive rows then cover all 16 bank groups,
-// and the 4 consecutive rows of a transposing read fall on 4 different pairs of them.
+// 8 (((r >> 3) ^ r) & 1): a permutation of r mod 16, so the 16-byte operand reads of 16 consecutive rows
+// cover all 16 bank groups, and the 8 rows of a transposing read (64 bytes each out of one aligned
+// 64-byte quarter of the row) fall two to a quarter, which is all 64 banks twice -- the least 512 bytes
+// can take.  (With bit 3 of g taken from bit 3 of r alone those 8 rows shared two quarters: a quarter of
+// all LDS cycles were bank conflicts then, 4 % now.)
 //
 // How a K / V (Q / dO) tile gets there: straight from memory by global_load_lds_dwordx4 where the tensors
 // allow it (16-byte aligned, see DmaTileMap: every head addressed from the 16-byte boundary at or below
@@ -93,7 +96,7 @@ __device__ __forceinline__ uint2 gload8(gptr_t q)
     return make_uint2(t.x, t.y);
 }
 
-__device__ __forceinline__ int gsw(int r) { return ((r & 3) << 1) | ((r >> 2) & 1) | (r & 8); }
+__device__ __forceinline__ int gsw(int r) { return ((r & 3) << 1) | ((r >> 2) & 1) | ((r & 8) ^ ((r & 1) << 3)); }
 __device__ __forceinline__ int toff(int r, int c) { return r * kRowB + ((c ^ gsw(r)) << 4); }
 
 __device__ __forceinline__ uint2 lds_read_tr(const unsigned char *q)
