@@ -488,6 +488,48 @@ __device__ __forceinline__ void prod_tr(float16_t (&acc)[DT], const unsigned cha
     }
 }
 
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// The same with independent vector arithmetic between its 2 DT MFMAs (NP pieces, `work(integral_constant<i>)`):
+// every transposing read is issued first, scheduling barriers keep the order as written.
+template <int DT, int NP, class F>
+__device__ __forceinline__ void prod_tr_with(float16_t (&acc)[DT], const unsigned char *tile, int k_base, half8_t y0,
+                                             half8_t y1, int lane, F &&work)
+{
+    const int a4 = (lane >> 2) & 3, b4 = lane & 3, n16 = (lane >> 4) & 1, lh = lane >> 5;
+    const int colb = 16 * n16 + 4 * b4;
+    half8_t x[2][DT];
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+        const int r1 = k_base + 16 * kk + 4 * lh + a4, r2 = r1 + 8;
+        const unsigned char *p1 = tile + r1 * kRowB + ((colb & 4) << 1);
+        const unsigned char *p2 = tile + r2 * kRowB + ((colb & 4) << 1);
+        const int g1 = gsw(r1), g2 = gsw(r2);
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            const int c = (32 * dt + colb) >> 3;
+            x[kk][dt] = as_h8(lds_read_tr(p1 + ((c ^ g1) << 4)), lds_read_tr(p2 + ((c ^ g2) << 4)));
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    static_for<0, 2 * DT>([&](auto j_c) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_c)::value, kk = j / DT, dt = j % DT;
+        acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[kk][dt], kk ? y1 : y0, acc[dt], 0, 0, 0);
+        constexpr int p0 = j * NP / (2 * DT), p1 = (j + 1) * NP / (2 * DT);
+        if constexpr (p0 < p1) work(std::integral_constant<int, p0>{});
+        if constexpr (p0 + 1 < p1) work(std::integral_constant<int, p0 + 1>{});
+        static_assert(p1 - p0 <= 2, "at most two pieces per MFMA");
+        __builtin_amdgcn_sched_barrier(0);
+    });
+}
+
 __device__ __forceinline__ half8_t pack8(const float *p)
 {
     half8_t h;
@@ -576,6 +618,17 @@ __device__ __forceinline__ float prob_shift(float m, float l)
     return __builtin_fmaf(m, kLog2e, __builtin_amdgcn_logf(l));
 }
 
+// a x as an f32 value of its own: the reference scales a product in f32 and rounds the result to f16, two
+// roundings; written as f2h(a * x) the compiler is free to use one instruction that multiplies and rounds to f16
+// once (v_fma_mixlo_f16), which differs from that in one element of some 20,000 by an f16 ulp -- and costs
+// more than the multiplication and half a packed conversion
+__device__ __forceinline__ float scaled(float a, float x)
+{
+    float t = a * x;
+    asm volatile("" : "+v"(t));
+    return t;
+}
+
 // 4 consecutive d of one output row: f16(scale a[0..3] [+ old])
 __device__ __forceinline__ void store_row4(half_t *dst, float a0, float a1, float a2, float a3, float scale,
                                            int acc_old)
@@ -585,10 +638,10 @@ __device__ __forceinline__ void store_row4(half_t *dst, float a0, float a1, floa
     if (acc_old) {
         const half4_t old = *reinterpret_cast<const half4_t *>(dst);
 #pragma unroll
-        for (int r = 0; r < 4; r++) o[r] = f2h(scale * a[r] + h2f(old[r]));
+        for (int r = 0; r < 4; r++) o[r] = f2h(scaled(scale, a[r]) + h2f(old[r]));
     } else {
 #pragma unroll
-        for (int r = 0; r < 4; r++) o[r] = f2h(scale * a[r]);
+        for (int r = 0; r < 4; r++) o[r] = f2h(scaled(scale, a[r]));
     }
     *reinterpret_cast<half4_t *>(dst) = o;
 }
@@ -608,7 +661,7 @@ __device__ __forceinline__ void stage_rows(unsigned char *stage, const float16_t
         for (int q = 0; q < 4; q++) {
             half4_t o;
 #pragma unroll
-            for (int r = 0; r < 4; r++) o[r] = f2h(scale * acc[dt][4 * q + r]);
+            for (int r = 0; r < 4; r++) o[r] = f2h(scaled(scale, acc[dt][4 * q + r]));
             *reinterpret_cast<half4_t *>(stage + toff(row, 4 * dt + q) + 8 * lh) = o;
         }
 }
@@ -728,7 +781,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                 if constexpr (i == 0) {
 #pragma unroll
                     for (int e = 0; e < 8; e++)
-                        sp[e] = __builtin_convertvector(float2v_t{p.alpha * acc[2 * e], p.alpha * acc[2 * e + 1]}, half2v_t);
+                        sp[e] = __builtin_convertvector(float2v_t{scaled(p.alpha, acc[2 * e]), scaled(p.alpha, acc[2 * e + 1])}, half2v_t);
                 } else if constexpr (i == 1) {
                     half2v_t mx = sp[0];
 #pragma unroll
@@ -787,12 +840,12 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                         half_t sh[16];
                         if (full) {
 #pragma unroll
-                            for (int e = 0; e < 16; e++) sh[e] = f2h(p.alpha * acc[e]);
+                            for (int e = 0; e < 16; e++) sh[e] = f2h(scaled(p.alpha, acc[e]));
                         } else {
 #pragma unroll
                             for (int e = 0; e < 16; e++) {
                                 const int key = kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                                sh[e] = key <= myrow ? f2h(p.alpha * acc[e]) : (half_t)-INFINITY;
+                                sh[e] = key <= myrow ? f2h(scaled(p.alpha, acc[e])) : (half_t)-INFINITY;
                             }
                         }
                         const float m_new = fmaxf(m_run, max16(sh)), c = m_new * kLog2e;
@@ -809,7 +862,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                     } else if (full) {                   // no masks on tiles wholly below the diagonal
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
-                            sv[e] = rnd16(p.alpha * acc[e]);
+                            sv[e] = rnd16(scaled(p.alpha, acc[e]));
                             mt = fmaxf(mt, sv[e]);
                         }
                         const float m_new = fmaxf(m_run, mt);
@@ -821,7 +874,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             const int key = kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                            const float s = rnd16(p.alpha * acc[e]);
+                            const float s = rnd16(scaled(p.alpha, acc[e]));
                             sv[e] = key <= myrow ? s : -INFINITY;
                             mt = fmaxf(mt, sv[e]);
                         }
@@ -880,7 +933,56 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
             tv.store(tm, Vs);
         }
         tile_sync<DMA>();
-        for (int it = 0; it < niter; it++) {
+        int it2 = 0;
+        if constexpr (FAST && DMA) {
+            // The key tiles wholly below the diagonal for every wave, as in pass 1, with the vector arithmetic of a
+            // block between the MFMAs of its neighbours: per tile, the scores of its second block are formed while
+            // the probabilities of the first are, the first block's P V products run while the second's
+            // probabilities are formed, then the second's P V; the first scores of the next tile follow the barrier
+            // that publishes it (the P V products read the V tile, which the next iteration's loads overwrite, so
+            // they cannot move behind the barrier).  The same operations on the same values in the same order as the
+            // general loop below.
+            const int nfull = min(qt, niter);
+            if (nfull > 0) {
+                half2v_t sp[8];
+                float pe[16];
+                half8_t pk[2][2];                               // packed probabilities of the tile's two blocks
+                auto prob_piece = [&](const float16_t &acc, half8_t (&out)[2], auto i_c) __attribute__((always_inline)) {
+                    constexpr int i = decltype(i_c)::value;
+                    if constexpr (i == 0) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++)
+                            sp[e] = __builtin_convertvector(float2v_t{scaled(p.alpha, acc[2 * e]), scaled(p.alpha, acc[2 * e + 1])}, half2v_t);
+                    } else if constexpr (i < 5) {
+#pragma unroll
+                        for (int e = 4 * (i - 1); e < 4 * i; e++) pe[e] = exp2_mix(sp[e >> 1][e & 1], cs);
+                    } else {
+                        out[0] = pack8(pe);
+                        out[1] = pack8(pe + 8);
+                    }
+                };
+                float16_t accp = prod_direct<KS>(Ks, 0, qf, l32, lh);
+                for (int it = 0; it < nfull; it++) {
+                    const int jt = 2 * it + g, cur = it & 1;
+                    const bool nxt = jt + 2 < njt;
+                    if (nxt) {
+                        tk.load(tm, K + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Ks + (cur ^ 1) * kTileB);
+                        tv.load(tm, V + (int64_t)(jt + 2) * kTileRows * ld, S - (jt + 2) * kTileRows, Vs + (cur ^ 1) * kTileB);
+                    }
+                    const float16_t acc2 = prod_direct_with<KS, 6>(Ks + cur * kTileB, 32, qf, l32, lh,
+                                                                   [&](auto i_c) { prob_piece(accp, pk[0], i_c); });
+                    asm volatile("" : "+v"(pk[0][0]), "+v"(pk[0][1]));
+                    prod_tr_with<DT, 6>(oacc, Vs + cur * kTileB, 0, pk[0][0], pk[0][1], lane,
+                                        [&](auto i_c) { prob_piece(acc2, pk[1], i_c); });
+                    asm volatile("" : "+v"(pk[1][0]), "+v"(pk[1][1]));
+                    prod_tr<DT>(oacc, Vs + cur * kTileB, 32, pk[1][0], pk[1][1], lane);
+                    tile_sync<DMA>();
+                    if (it + 1 < nfull) accp = prod_direct<KS>(Ks + (cur ^ 1) * kTileB, 0, qf, l32, lh);
+                }
+                it2 = nfull;
+            }
+        }
+        for (int it = it2; it < niter; it++) {
             const int jt = 2 * it + g, cur = it & 1;
             const bool nxt = jt + 2 < njt;
             if (nxt) {
@@ -898,22 +1000,22 @@ __global__ void __launch_bounds__(kNT2, 2) attn_fwd_kernel(AttnArgs p)
                     if constexpr (FAST) {
                         if (full) {
 #pragma unroll
-                            for (int e = 0; e < 16; e++) pe[e] = exp2_mix(f2h(p.alpha * acc[e]), cs);
+                            for (int e = 0; e < 16; e++) pe[e] = exp2_mix(f2h(scaled(p.alpha, acc[e])), cs);
                         } else {
 #pragma unroll
                             for (int e = 0; e < 16; e++) {
                                 const int key = kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                                pe[e] = key <= myrow ? exp2_mix(f2h(p.alpha * acc[e]), cs) : 0.f;
+                                pe[e] = key <= myrow ? exp2_mix(f2h(scaled(p.alpha, acc[e])), cs) : 0.f;
                             }
                         }
                     } else if (full) {
 #pragma unroll
-                        for (int e = 0; e < 16; e++) pe[e] = M::prob(rnd16(p.alpha * acc[e]), m, l, y);
+                        for (int e = 0; e < 16; e++) pe[e] = M::prob(rnd16(scaled(p.alpha, acc[e])), m, l, y);
                     } else {
 #pragma unroll
                         for (int e = 0; e < 16; e++) {
                             const int key = kb + 8 * (e >> 2) + 4 * lh + (e & 3);
-                            const float pr_ = M::prob(rnd16(p.alpha * acc[e]), m, l, y);
+                            const float pr_ = M::prob(rnd16(scaled(p.alpha, acc[e])), m, l, y);
                             pe[e] = key <= myrow ? pr_ : 0.f;
                         }
                     }
@@ -1066,7 +1168,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
                             if (full) {
 #pragma unroll
                                 for (int e = 0; e < 16; e++) {
-                                    const float pr_ = exp2_mix(f2h(p.alpha * sacc[e]), cs);
+                                    const float pr_ = exp2_mix(f2h(scaled(p.alpha, sacc[e])), cs);
                                     const half_t dp = dph[e];
                                     if (PASS == 0) part = __builtin_fmaf((float)dp, pr_, part);
                                     else de[e] = __builtin_fmaf((float)dp, pr_, -(sig * pr_));
@@ -1075,7 +1177,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 #pragma unroll
                                 for (int e = 0; e < 16; e++) {
                                     const bool live = kb + 8 * (e >> 2) + 4 * lh + (e & 3) <= myrow;
-                                    const float pr_ = exp2_mix(f2h(p.alpha * sacc[e]), cs);
+                                    const float pr_ = exp2_mix(f2h(scaled(p.alpha, sacc[e])), cs);
                                     const half_t dp = dph[e];
                                     if (PASS == 0) part += live ? (float)dp * pr_ : 0.f;
                                     else de[e] = live ? __builtin_fmaf((float)dp, pr_, -(sig * pr_)) : 0.f;
@@ -1084,7 +1186,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
                         } else if (full) {
 #pragma unroll
                             for (int e = 0; e < 16; e++) {
-                                const float pr_ = M::prob(rnd16(p.alpha * sacc[e]), m, l, y);
+                                const float pr_ = M::prob(rnd16(scaled(p.alpha, sacc[e])), m, l, y);
                                 const float tt = pr_ * rnd16(pacc[e]);
                                 if (PASS == 0) part += tt;
                                 else de[e] = tt - sig * pr_;
@@ -1093,7 +1195,7 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 #pragma unroll
                             for (int e = 0; e < 16; e++) {
                                 const bool live = kb + 8 * (e >> 2) + 4 * lh + (e & 3) <= myrow;
-                                const float pr_ = M::prob(rnd16(p.alpha * sacc[e]), m, l, y);
+                                const float pr_ = M::prob(rnd16(scaled(p.alpha, sacc[e])), m, l, y);
                                 const float tt = pr_ * rnd16(pacc[e]);
                                 if (PASS == 0) part += live ? tt : 0.f;
                                 else de[e] = live ? tt - sig * pr_ : 0.f;
@@ -1168,14 +1270,6 @@ __global__ void __launch_bounds__(kNT2, 2) attn_bwd_dq_kernel(AttnArgs p)
 // ---------------------------------------------------------------------------------------------
 // dK, dV: keys fixed (128 per workgroup of 4 waves, a lane owns one), loop over the query tiles at or
 // after them; the key tiles with the most queries first.
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F &&f)
-{
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
 
 constexpr int kDkvBufs = 3;                      // tile buffers per tensor (Q, dO) and sets of row statistics
 
@@ -1290,10 +1384,10 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                         const int e = 4 * q + r, query = iq * kTileRows + qi + r;
                         float pr_, ds;
                         if constexpr (FAST) {                 // yy holds the exponent offset of the row
-                            pr_ = exp2_mix(f2h(p.alpha * sacc[e]), yy[r]);
+                            pr_ = exp2_mix(f2h(scaled(p.alpha, sacc[e])), yy[r]);
                             ds = __builtin_fmaf((float)dph[e], pr_, -(sg[r] * pr_));
                         } else {
-                            pr_ = M::prob(rnd16(p.alpha * sacc[e]), mm[r], ll[r], yy[r]);
+                            pr_ = M::prob(rnd16(scaled(p.alpha, sacc[e])), mm[r], ll[r], yy[r]);
                             const float tt = pr_ * rnd16(pacc[e]);
                             ds = tt - sg[r] * pr_;
                         }
@@ -1398,7 +1492,7 @@ __global__ void __launch_bounds__(kNT, 1) attn_bwd_dkv_kernel(AttnArgs p)
                                 yy = *reinterpret_cast<const float4_t *>(stc + 2 * 64 + qi);
                                 sg = *reinterpret_cast<const float4_t *>(stc + 3 * 64 + qi);
                             }
-                            s2 = cvt_pk(p.alpha * sC[e0], p.alpha * sC[e0 + 1]);
+                            s2 = cvt_pk(scaled(p.alpha, sC[e0]), scaled(p.alpha, sC[e0 + 1]));
                             d2 = cvt_pk(pC[e0], pC[e0 + 1]);
                         } else if constexpr (qr == 1) {
                             pr2[0] = exp2_mix(s2[0], yy[2 * hf]);
